@@ -1,0 +1,149 @@
+/*
+ * libsmlm_hip -- Segmented Multi-LoRA Multiplication for AMD gfx950 (MI355X).
+ *
+ * C ABI of the shared library built from loquetier_amd/csrc/.  Plain pointers
+ * and sizes only; every device pointer is an address in the memory of the GPU
+ * that is current when the call is made.  Every call is asynchronous and
+ * stream-ordered on `stream` (a hipStream_t passed as void*; NULL = the null
+ * stream); none synchronises the host, none allocates or frees memory, none
+ * keeps state between calls.  Return value: SMLM_OK or a negative SMLM_ERR_*.
+ *
+ * Maths (weights in the layout the reference passes, is_row_major = False):
+ *   A_i [r, h_in] row-major, B_i [h_out, r] row-major,
+ *   v = x A_i^T,  y = v B_i^T  for the rows of segment i,
+ * rows [seg_indptr[i], seg_indptr[i+1]) forming segment i of the flat batch.
+ *
+ * Contract shared by all entry points (the reference's CUTLASS kernels are
+ * instantiated with alignment 8, smlm_forward_cutlass.cuh:88-92,133-137):
+ * 16-bit element types only (fp16 / bf16); every matrix pointer 16-byte
+ * aligned; d_in, d_out, h_in, h_out, r multiples of 8; seg_indptr
+ * non-decreasing with seg_indptr[0] >= 0 and seg_indptr[S] <= T.
+ */
+#ifndef SMLM_H_
+#define SMLM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SMLM_ABI_VERSION 1
+
+#if defined(__GNUC__)
+#define SMLM_API __attribute__((visibility("default")))
+#else
+#define SMLM_API
+#endif
+
+/* element types (reference: DISPATCH_TORCH_DTYPE, loquetier_ops.cc:54-76) */
+#define SMLM_DTYPE_F16 0
+#define SMLM_DTYPE_BF16 1
+
+/* what a plan groups segments by */
+#define SMLM_KEY_NONE 0 /* every segment is its own group                    */
+#define SMLM_KEY_I32 1  /* int32 adapter id per segment                      */
+#define SMLM_KEY_PTR 2  /* 64-bit weight address per segment                 */
+
+#define SMLM_OK 0
+#define SMLM_ERR_ARG (-1)       /* null pointer, negative size, bad enum      */
+#define SMLM_ERR_DTYPE (-2)     /* "No suitable kernel." (loquetier_ops.cc:318) */
+#define SMLM_ERR_ALIGN (-3)     /* dimension not a multiple of 8 / pointer not 16-byte aligned */
+#define SMLM_ERR_WORKSPACE (-4) /* workspace or plan buffer too small         */
+#define SMLM_ERR_LAUNCH (-5)    /* the HIP runtime refused a kernel launch    */
+#define SMLM_ERR_LIMIT (-6)     /* size beyond what the kernels index         */
+
+SMLM_API int smlm_abi_version(void);
+SMLM_API const char* smlm_strerror(int code);
+
+/*
+ * Replaces smlm_forward_tmp_size (smlm_forward_cutlass.cuh:48-52), exported to
+ * Python as smlm_forward_cutlass_tmp_size (loquetier_ops.cc:372).  The
+ * reference carves seven per-problem arrays (60 bytes per problem) out of
+ * `tmp`; this library keeps its per-call tables in the workspace sized by
+ * smlm_gemm_workspace_size, so the value only has to be what the caller
+ * allocates and passes back: 64 bytes per problem.
+ */
+SMLM_API int smlm_tmp_size(int num_problems, size_t* bytes);
+
+/*
+ * Tile plan.  Replaces precompute_smlm_forward_args
+ * (smlm_forward_cutlass.cuh:31-46): the per-problem table the grouped GEMM
+ * walks.  Here the table lists 16-row tiles; rows of segments that share a key
+ * (adapter) are gathered into common tiles so each adapter's weights are read
+ * once per tile column instead of once per segment.  The plan depends only on
+ * (seg_indptr, keys): one plan serves every layer and projection of a batch.
+ *   seg_key: NULL for SMLM_KEY_NONE, const int32_t* [S] for SMLM_KEY_I32,
+ *            const void* const* [S] for SMLM_KEY_PTR (device memory).
+ */
+SMLM_API int smlm_plan_size(int T, int S, size_t* bytes);
+SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr,
+                    const void* seg_key, int key_kind, int T, int S, void* stream);
+
+/*
+ * Grouped GEMM  Y_i = beta*Y_i + scale_i * X_i W_i  over the segments.
+ * Replaces dispatch_smlm_forward_cutlass / smlm_forward<DType,Layout>
+ * (loquetier_ops.cc:277-319, smlm_forward_cutlass.cuh:61-175), which computes
+ * the beta = 0, scale = 1 case.  w_ptrs[i] (device array of S device
+ * addresses) is a d_in x d_out matrix: element (k, n) at w[k*w_ld + n] when
+ * w_row_major, else at w[n*w_ld + k].  seg_scale: NULL or float [S] (device).
+ * Builds its own plan (grouped by weight address) inside `workspace`.
+ * Rows outside every segment are not touched.
+ */
+SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes);
+SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const int32_t* seg_indptr,
+              void* workspace, size_t workspace_bytes, int T, int S, int d_in, int d_out,
+              int w_ld, int w_row_major, int dtype, float beta, const float* seg_scale,
+              void* stream);
+
+/*
+ * Fused LoRA forward  y = beta*y + scale_i * round16(x A^T) B^T.
+ * Replaces the two kernel calls of add_lora.forward
+ * (src/loquetier_src/kernel_utils.py:115-119) plus, with beta = 1 and
+ * seg_scale, the scale multiply and residual add of MixedLoraLinear.forward
+ * (src/loquetier_src/models/mixed_lora.py:214-217).
+ *   a_ptrs / b_ptrs: device arrays of device addresses.  With seg_adapter
+ *     (int32 [S], device) they are per-adapter tables indexed by
+ *     seg_adapter[i] -- the gather wa_ptrs[lora_ids] of mixed_lora.py:182
+ *     done inside the kernel; with seg_adapter = NULL they are per-segment.
+ *   plan: built by smlm_plan_build for the same (seg_indptr, T, S).
+ *   v_out: NULL, or [T, r] receiving the rounded intermediate for backward.
+ */
+SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes);
+SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* const* a_ptrs,
+                  const void* const* b_ptrs, const int32_t* seg_adapter,
+                  const int32_t* seg_indptr, const void* plan, void* workspace,
+                  size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
+                  float beta, const float* seg_scale, void* stream);
+
+/*
+ * LoRA backward for fine-tuning rows.  Replaces add_lora.backward
+ * (src/loquetier_src/kernel_utils.py:128-147; the C++ side of the reference
+ * has only "// smlm backward // TODO", loquetier_ops.cc:321-322), with the
+ * products written for the weight layout the forward uses:
+ *   dV = s (dY B)   dX = dV A   dA_a = sum dV^T x   dB_a = sum dY^T (s v)
+ * Rows [part_indptr[p], part_indptr[p+1]) of dy / x / v / dx form train
+ * partition p, trained by adapter part_adapter[p] in [0, NA).  da_ptrs[a]
+ * ([r, h_in]) and db_ptrs[a] ([h_out, r]) are overwritten for every a with the
+ * sum over that adapter's partitions (zeros when it has none); summation order
+ * is fixed, no atomics.  dx rows [0, n_rows) covered by a partition are
+ * overwritten, others untouched.
+ *   plan: built by smlm_plan_build(part_indptr, part_adapter, SMLM_KEY_I32,
+ *         n_rows, P).   v: NULL (recomputed from x and A) or [n_rows, r].
+ *   part_scale: NULL or float [P] (device), the forward's seg_scale.
+ * Needs n_rows >= 1, P >= 1, NA >= 1 and r <= 64.
+ */
+SMLM_API int smlm_lora_bwd_workspace_size(int n_rows, int P, int NA, int h_in, int h_out, int r,
+                                 size_t* bytes);
+SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs, const void* dy,
+                  const void* x, const void* v, const void* const* a_ptrs,
+                  const void* const* b_ptrs, const int32_t* part_adapter,
+                  const int32_t* part_indptr, const void* plan, void* workspace,
+                  size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out, int r,
+                  int dtype, const float* part_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMLM_H_ */

@@ -1,0 +1,70 @@
+"""ctypes binding of libsmlm_hip.so (the C ABI declared in include/smlm.h).
+
+There is no CPU fallback: if the library is missing or fails to load, every
+operator raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "lib", "libsmlm_hip.so")
+
+SMLM_DTYPE_F16, SMLM_DTYPE_BF16 = 0, 1
+SMLM_KEY_NONE, SMLM_KEY_I32, SMLM_KEY_PTR = 0, 1, 2
+SMLM_ERR_DTYPE = -2
+
+_vp, _i, _sz, _f = C.c_void_p, C.c_int, C.c_size_t, C.c_float
+_psz = C.POINTER(C.c_size_t)
+
+# name -> (restype, argtypes); must list every symbol include/smlm.h declares
+SIGNATURES = {
+    "smlm_abi_version": (_i, []),
+    "smlm_strerror": (C.c_char_p, [_i]),
+    "smlm_tmp_size": (_i, [_i, _psz]),
+    "smlm_plan_size": (_i, [_i, _i, _psz]),
+    "smlm_plan_build": (_i, [_vp, _sz, _vp, _vp, _i, _i, _i, _vp]),
+    "smlm_gemm_workspace_size": (_i, [_i, _i, _i, _i, _psz]),
+    "smlm_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
+    "smlm_lora_fwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _psz]),
+    "smlm_lora_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
+                           _f, _vp, _vp]),
+    "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
+    "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i,
+                           _i, _i, _i, _i, _i, _vp, _vp]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the HIP library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m loquetier_amd.build` "
+                "(hipcc, gfx950). There is no fallback path.")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return load().smlm_strerror(code).decode()
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        raise RuntimeError(f"{what}: {strerror(code)} (code {code})")
+
+
+def size_query(fn_name: str, *args: int) -> int:
+    out = C.c_size_t(0)
+    check(getattr(load(), fn_name)(*args, C.byref(out)), fn_name)
+    return out.value

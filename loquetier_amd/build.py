@@ -1,0 +1,52 @@
+"""Builds libsmlm_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
+
+Usage: python -m loquetier_amd.build
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC_DIR = os.path.join(PKG_DIR, "csrc")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libsmlm_hip.so")
+SOURCES = ["smlm_api.hip"]
+HEADERS = ["smlm_common.hpp", "smlm_plan.hpp", "smlm_forward.hpp", "smlm_backward.hpp"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+    # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    return "hipcc"
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile every HIP source into loquetier_amd/lib/libsmlm_hip.so (always recompiles)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC_DIR,
+           *[os.path.join(CSRC_DIR, s) for s in SOURCES], "-o", LIB_PATH + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass warns that it does not know the packed-fp32 feature: harmless
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
+    if err.strip() and verbose:
+        print(err, file=sys.stderr)
+    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

@@ -1,0 +1,144 @@
+// Shared device helpers for the SMLM kernels (gfx950 / CDNA4 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "smlm.h"
+
+namespace smlm {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTileRows = 16;     // rows of one MFMA tile = tokens per plan tile
+constexpr int kWaveSize = 64;
+constexpr int kSegBits = 20;      // segment index bits inside a sort key
+constexpr int kMaxSegments = 1 << kSegBits;
+
+// Element-type traits: one v_mfma_f32_16x16x32 step and the 16-bit <-> fp32
+// conversions (round to nearest even on the way down).
+template <int DT>
+struct Num;
+
+template <>
+struct Num<SMLM_DTYPE_F16> {
+  static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t bits(float f) {
+    _Float16 h = (_Float16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, h);
+  }
+  static __device__ __forceinline__ float lo(uint32_t u) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(u & 0xffffu));
+  }
+  static __device__ __forceinline__ float hi(uint32_t u) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(u >> 16));
+  }
+};
+
+template <>
+struct Num<SMLM_DTYPE_BF16> {
+  static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t bits(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7f800000u) == 0x7f800000u) {          // inf / nan: truncate, keep nan a nan
+      if (u & 0x007fffffu) u |= 0x00400000u;
+      return u >> 16;
+    }
+    u += 0x7fffu + ((u >> 16) & 1u);                 // round to nearest even
+    return u >> 16;
+  }
+  static __device__ __forceinline__ float lo(uint32_t u) {
+    return __builtin_bit_cast(float, u << 16);
+  }
+  static __device__ __forceinline__ float hi(uint32_t u) {
+    return __builtin_bit_cast(float, u & 0xffff0000u);
+  }
+};
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return Num<DT>::bits(lo) | (Num<DT>::bits(hi) << 16);
+}
+
+__device__ __forceinline__ u32x4 ldg16(const uint16_t* p) {
+  return *reinterpret_cast<const u32x4*>(p);
+}
+__device__ __forceinline__ void stg16(uint16_t* p, u32x4 v) {
+  *reinterpret_cast<u32x4*>(p) = v;
+}
+__device__ __forceinline__ f32x4 ldg_f4(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+
+// Eight 16-bit elements with a stride (the slow gather used for the weight
+// layout the reference never passes).
+__device__ __forceinline__ u32x4 ldg_strided8(const uint16_t* p, long stride) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t a = p[(2 * i) * stride];
+    uint32_t b = p[(2 * i + 1) * stride];
+    r[i] = a | (b << 16);
+  }
+  return r;
+}
+
+// Views into a plan buffer (all int32).  Sizes are functions of (T, S) only.
+struct PlanView {
+  int32_t* hdr;         // [16]: 0 n_tiles, 1 n_groups, 2 rows covered, 3 key kind used
+  int32_t* sorted_seg;  // [S]   segment at sorted position p
+  int32_t* rowpos;      // [S+1] first gathered-row index of sorted position p
+  int32_t* grp_tile;    // [S+1] first tile of group G (exclusive scan), [NG] = n_tiles
+  int32_t* grp_row;     // [S+1] first gathered-row index of group G, [NG] = rows covered
+  int32_t* grp_seg;     // [S]   representative (first) segment of group G
+  int32_t* grp_id;      // [S]   int32 key of group G (adapter id for SMLM_KEY_I32)
+  int32_t* tile_row;    // [nt_max*16] row index of each tile slot, -1 = empty
+  int32_t* tile_rseg;   // [nt_max*16] segment of each tile slot, -1 = empty
+  uint64_t* sort_keys;  // [pow2 >= S] scratch for sorts that do not fit in LDS
+  int nt_max;
+};
+
+inline int plan_nt_max(int T, int S) { return T / kTileRows + S + 1; }
+inline int next_pow2(int v) {
+  int n = 1;
+  while (n < v) n <<= 1;
+  return n;
+}
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Carves the views out of `base`; returns the bytes used (base may be null to size).
+inline size_t plan_carve(void* base, int T, int S, PlanView* pv) {
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off = align_up(off + bytes, 256);
+    return base ? reinterpret_cast<char*>(base) + o : nullptr;
+  };
+  const int nt_max = plan_nt_max(T, S);
+  PlanView v;
+  v.hdr = reinterpret_cast<int32_t*>(take(16 * 4));
+  v.sorted_seg = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.rowpos = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.grp_tile = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.grp_row = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.grp_seg = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.grp_id = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.tile_row = reinterpret_cast<int32_t*>(take((size_t)nt_max * kTileRows * 4));
+  v.tile_rseg = reinterpret_cast<int32_t*>(take((size_t)nt_max * kTileRows * 4));
+  v.sort_keys = reinterpret_cast<uint64_t*>(take((size_t)next_pow2(S > 0 ? S : 1) * 8));
+  v.nt_max = nt_max;
+  if (pv) *pv = v;
+  return off;
+}
+
+}  // namespace smlm

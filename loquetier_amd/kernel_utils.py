@@ -1,0 +1,189 @@
+"""Host-side mirror of src/loquetier_src/kernel_utils.py for the SMLM path:
+`BatchLenInfo` (row layout of the flat batch) and the `add_lora` autograd
+Function, with the reference's positional arguments and `None`-padded backward
+tuple, running on the HIP kernels.
+"""
+from __future__ import annotations
+
+from collections.abc import Sequence
+from typing import List, Optional, Tuple
+
+import numpy as np
+import torch
+from torch.autograd.function import Function, FunctionCtx
+
+from .ops import _kernels as kernel
+
+
+class BatchLenInfo:
+    """Row layout [train | eval | prefill | decode] of one flat batch
+    (reference: src/loquetier_src/kernel_utils.py:11-98, same properties)."""
+
+    def __init__(self, trains: List[Tuple[int, ...]], prefills: List[int], decode: int,
+                 evals: List[Tuple[int, ...]], indptr_device: torch.device,
+                 indptr_dtype: torch.dtype = torch.int32):
+        self._train_batches = trains
+        tlen = [t[0] * t[1] for t in trains]
+        if tlen:
+            self._train_partition = np.cumsum([0] + tlen)
+            self._tlen = int(self._train_partition[-1])
+        else:
+            self._train_partition = []
+            self._tlen = 0
+        self._eval_batches = evals
+        if evals:
+            self._eval_partition = np.cumsum([self._tlen] + [e[0] * e[1] for e in evals])
+        else:
+            self._eval_partition = []
+        self._prefills = list(prefills)
+        self._decode = decode
+        if prefills:
+            cumsum = np.cumsum([0] + list(prefills))
+            self._indptr = torch.tensor(cumsum, dtype=indptr_dtype, device=indptr_device)
+            self._doff = int(cumsum[-1]) + self._tlen
+        else:
+            self._indptr = None
+            self._doff = self._tlen
+
+    @property
+    def train_batches(self) -> List[Tuple[int, ...]]:
+        return self._train_batches
+
+    @property
+    def train_partition(self) -> Sequence[int]:
+        return self._train_partition
+
+    @property
+    def eval_batches(self) -> List[Tuple[int, ...]]:
+        return self._eval_batches
+
+    @property
+    def eval_partition(self) -> Sequence[int]:
+        return self._eval_partition
+
+    @property
+    def prefills(self) -> List[int]:
+        return self._prefills
+
+    @property
+    def decode(self) -> int:
+        return self._decode
+
+    @property
+    def tlen(self) -> int:
+        return self._tlen
+
+    @property
+    def doff(self) -> int:
+        return self._doff
+
+    @property
+    def indptr(self) -> Optional[torch.Tensor]:
+        return self._indptr
+
+
+def _ptr_table(tensors: Sequence[torch.Tensor], device: torch.device) -> torch.Tensor:
+    return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, device=device)
+
+
+def _unique_adapters(weight_list: Sequence[torch.Tensor]):
+    """Train partitions -> indices into the list of distinct (A, B) pairs."""
+    pairs, index, part_adapter = [], {}, []
+    for wa, wb in zip(weight_list[::2], weight_list[1::2]):
+        key = (wa.data_ptr(), wb.data_ptr())
+        if key not in index:
+            index[key] = len(pairs)
+            pairs.append((wa, wb))
+        part_adapter.append(index[key])
+    return pairs, part_adapter
+
+
+def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Optional[torch.Tensor],
+                  weight_list: Sequence[torch.Tensor], tp: Sequence[int], lora_rank: int,
+                  part_scale: Optional[torch.Tensor] = None):
+    """Shared backward: returns (grad_x [T, h_in], [grad per weight occurrence]).
+
+    Partitions that train the same adapter contribute to one summed gradient,
+    returned for the first occurrence of that adapter; later occurrences get
+    None (autograd adds per-occurrence gradients, so the total is the same as
+    the reference's, src/loquetier_src/models/mixed_lora.py:201-204)."""
+    dev, dt = grad_output.device, grad_output.dtype
+    T = grad_output.size(0)
+    h_in = x_train.size(1)
+    n_parts = min(len(weight_list) // 2, len(tp) - 1)
+    tp = [int(t) for t in tp][: n_parts + 1]
+    tl = tp[-1]
+    grad_x = torch.empty((T, h_in), dtype=dt, device=dev)
+    if tl < T:
+        grad_x[tl:].zero_()
+    if tp[0] > 0:
+        grad_x[: tp[0]].zero_()
+    pairs, part_adapter = _unique_adapters(weight_list[: 2 * n_parts])
+    da = [torch.empty_like(wa) for wa, _ in pairs]
+    db = [torch.empty_like(wb) for _, wb in pairs]
+    if tl > 0:
+        g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
+        part_indptr = torch.tensor(tp, dtype=torch.int32, device=dev)
+        part_ad = torch.tensor(part_adapter, dtype=torch.int32, device=dev)
+        plan = kernel.SegmentPlan(part_indptr, part_ad, tl)
+        kernel.smlm_lora_backward(
+            grad_x, _ptr_table(da, dev), _ptr_table(db, dev), g, x_train, v_train,
+            _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
+            part_ad, plan, lora_rank, part_scale)
+    else:
+        for t in da + db:
+            t.zero_()
+    grads: List[Optional[torch.Tensor]] = []
+    seen = set()
+    for ad in part_adapter:
+        if ad in seen:
+            grads += [None, None]
+        else:
+            seen.add(ad)
+            grads += [da[ad], db[ad]]
+    grads += [None] * (len(weight_list) - len(grads))
+    return grad_x, grads
+
+
+class add_lora(Function):
+    """Reference: src/loquetier_src/kernel_utils.py:101-147.
+
+    forward(y_shape, x, wa_ptr, wb_ptr, s, lora_rank, train_len, train_partition, *weights)
+    returns y = (x @ A_seg^T) @ B_seg^T per segment (A [r,h_in], B [h_out,r]).
+    The two grouped GEMMs of the reference run as one fused call; v (rounded to
+    x's dtype, as the reference materialises it) is kept for backward instead
+    of being recomputed.  backward returns gradients for x and for each
+    trainable weight, written for the layout the forward uses.
+    """
+
+    @staticmethod
+    def forward(ctx: FunctionCtx, y_shape, x, wa_ptr, wb_ptr, s, lora_rank, train_len,
+                train_partition, *args):
+        y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
+        plan = kernel.SegmentPlan(s, wa_ptr, x.size(0))
+        need_v = len(args) > 0 and train_len > 0
+        v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
+        kernel.smlm_lora_forward(y, x, wa_ptr, wb_ptr, plan, lora_rank, v_out=v)
+        # what the reference's setup_context keeps (kernel_utils.py:122-126), plus v
+        ctx.tp = train_partition
+        ctx.rank = lora_rank
+        ctx.has_v = v is not None
+        if v is not None:
+            ctx.save_for_backward(x[:train_len, ...], v[:train_len, ...], *args)
+        else:
+            ctx.save_for_backward(x[:train_len, ...], *args)
+        return y
+
+    @staticmethod
+    def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
+        if ctx.has_v:
+            x, v, *weight_list = ctx.saved_tensors
+        else:
+            x, *weight_list = ctx.saved_tensors
+            v = None
+        if len(weight_list) == 0:
+            return None, None, None, None, None, None, None, None
+        assert len(weight_list) % 2 == 0
+        grad_x, grads = lora_backward(grad_output, x, v, weight_list, ctx.tp, ctx.rank)
+        return (None, grad_x, None, None, None, None, None, None, *grads)
+
