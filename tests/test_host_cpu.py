@@ -1,0 +1,142 @@
+"""CPU-only checks of the boundary and the host logic: the C-ABI library loads
+and exports every symbol include/smlm.h declares, argument validation returns
+the documented codes before any GPU work, and the Python mirrors of the
+reference's host-side helpers agree with the oracle.  No kernel is launched.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from loquetier_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from loquetier_amd.build import build_library
+        build_library()
+    return _lib
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    header = open(os.path.join(ROOT, "include", "smlm.h")).read()
+    declared = set(re.findall(r"SMLM_API\s+[\w\s\*]+?\b(smlm_\w+)\s*\(", header))
+    assert len(declared) >= 11
+    handle = ctypes.CDLL(lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), f"{name} is declared in smlm.h but not exported"
+    assert declared == set(lib.SIGNATURES), "ctypes binding and header disagree"
+    assert lib.load().smlm_abi_version() == 1
+
+
+def test_missing_library_fails_loudly(lib, monkeypatch):
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "LIB_PATH", "/nonexistent/libsmlm_hip.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        lib.load()
+
+
+def test_size_queries(lib):
+    assert lib.size_query("smlm_tmp_size", 0) == 0
+    assert lib.size_query("smlm_tmp_size", 256) == 64 * 256
+    small = lib.size_query("smlm_plan_size", 256, 256)
+    big = lib.size_query("smlm_plan_size", 8192, 1075)
+    assert 0 < small < big
+    # the plan must hold a row and a segment index for every slot of every possible tile
+    assert big >= (8192 // 16 + 1075 + 1) * 16 * 8
+    assert lib.size_query("smlm_gemm_workspace_size", 4224, 132, 4096, 16) > \
+        lib.size_query("smlm_plan_size", 4224, 132)
+    assert lib.size_query("smlm_lora_fwd_workspace_size", 4224, 132, 4096, 4096, 16) >= 4224 * 16 * 4
+    assert lib.size_query("smlm_lora_bwd_workspace_size", 4096, 4, 4, 4096, 4096, 16) > 0
+    out = ctypes.c_size_t(0)
+    assert lib.load().smlm_plan_size(-1, 4, ctypes.byref(out)) == -1
+    assert lib.load().smlm_plan_size(16, 1 << 20, ctypes.byref(out)) == -6
+
+
+def test_argument_validation_codes(lib):
+    L = lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 255) // 256 * 256  # 16-byte aligned fake "device" address; never dereferenced
+    big = 1 << 30
+    gemm = lambda **k: L.smlm_gemm(k.get("y", p), p, p, p, p, k.get("ws", big), k.get("T", 16), 2,
+                                   k.get("d_in", 64), k.get("d_out", 8), k.get("ld", 64), 0,
+                                   k.get("dtype", 0), 0.0, None, None)
+    assert gemm(dtype=2) == -2                      # fp32 etc.: "No suitable kernel."
+    assert lib.strerror(-2) == "No suitable kernel."
+    assert gemm(d_in=60, ld=60) == -3               # not a multiple of 8
+    assert gemm(y=p + 2) == -3                      # misaligned matrix
+    assert gemm(y=None) == -1
+    assert gemm(ws=128) == -4                       # workspace too small
+    assert gemm(T=-1) == -1
+    assert gemm(T=0) == 0                           # empty batch: nothing to do, no launch
+    assert L.smlm_plan_build(p, big, p, None, 2, 16, 2, None) == -1   # key kind needs keys
+    assert L.smlm_plan_build(p, big, p, p, 9, 16, 2, None) == -1      # unknown key kind
+    assert L.smlm_plan_build(p, 64, p, None, 0, 16, 2, None) == -4
+    assert L.smlm_lora_fwd(p, p, None, p, p, None, p, p, p, big, 16, 2, 64, 64, 12, 0, 0.0, None, None) == -3
+    assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, p, p, big, 16, 1, 1, 64, 64, 128, 1,
+                           None, None) == -6        # rank above the backward kernels' limit
+    assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, p, p, 16, 16, 1, 1, 64, 64, 8, 1,
+                           None, None) == -4
+
+
+def test_python_surface_rejects_host_tensors(lib):
+    from loquetier_amd.ops import _kernels as K
+    y, x = torch.zeros(4, 8, dtype=torch.float16), torch.zeros(4, 16, dtype=torch.float16)
+    w, s = torch.zeros(1, dtype=torch.int64), torch.tensor([0, 4], dtype=torch.int32)
+    tmp = torch.zeros(K.smlm_forward_cutlass_tmp_size(1), dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        K.smlm_forward_cutlass(y, x, w, s, tmp, False)
+
+
+def test_batch_len_info_mirror(oracle):
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    cases = [([(2, 8), (1, 5)], [3, 4], 6, []), ([], [7], 2, []), ([(1, 1024)], [], 128, [(1, 4)]),
+             ([], [], 5, [])]
+    for trains, prefills, decode, evals in cases:
+        b = BatchLenInfo(trains, prefills, decode, evals, torch.device("cpu"))
+        tp, tlen, doff = oracle.batch_len_info(trains, prefills)
+        assert list(b.train_partition) == (tp.tolist() if trains else [])
+        assert b.tlen == tlen and b.doff == doff and b.decode == decode
+        if prefills:
+            assert b.indptr.dtype == torch.int32
+            assert b.indptr.tolist() == np.concatenate([[0], np.cumsum(prefills)]).tolist()
+        else:
+            assert b.indptr is None
+        if evals:
+            assert list(b.eval_partition) == np.cumsum([tlen] + [e[0] * e[1] for e in evals]).tolist()
+
+
+def test_build_segments_mirror(oracle):
+    from loquetier_amd.segments import build_segments
+    rng = np.random.default_rng(0)
+    for _ in range(30):
+        n = int(rng.integers(1, 40))
+        ids = rng.integers(0, 5, n).tolist()
+        lens = rng.integers(1, 20, n).tolist()
+        lora_ids, lora_len, segment = build_segments(ids, lens, "cpu")
+        o_ids, o_len, o_seg = oracle.build_segments(ids, lens)
+        assert lora_ids == o_ids
+        assert lora_len.dtype == torch.int32 and segment.dtype == torch.int32
+        assert lora_len.tolist() == o_len.tolist() and segment.tolist() == o_seg.tolist()
+    with pytest.raises(IndexError):
+        build_segments([], [], "cpu")
+
+
+def test_prepare_weight_mirror(oracle):
+    from loquetier_amd.mixed_lora import prepare_weight
+    rng = np.random.default_rng(1)
+    w = rng.standard_normal((8, 32)).astype(np.float32)
+    for dt, tdt in (("fp16", torch.float16), ("bf16", torch.bfloat16)):
+        for scaling in (None, 2.0):
+            got = prepare_weight(torch.from_numpy(w), 16, tdt, "cpu", 0, scaling).float().numpy()
+            assert np.array_equal(got, oracle.prepare_weight(w, 0, 16, scaling, dt))
+            got = prepare_weight(torch.from_numpy(w.T.copy()), 16, tdt, "cpu", 1, scaling).float().numpy()
+            assert np.array_equal(got, oracle.prepare_weight(w.T.copy(), 1, 16, scaling, dt))
+        same = prepare_weight(torch.from_numpy(w), 8, tdt, "cpu", 0, None)
+        assert same.shape == (8, 32)
