@@ -1,0 +1,330 @@
+#!/usr/bin/env python3
+"""Benchmark of the SMLM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5]
+
+A step is one pass of the hot path over one synthetic batch: the tile plan is
+built from the batch's (segment, adapter-id) arrays, then every projection of
+the workload runs the fused LoRA forward (shrink + expand, accumulating in
+place into a base-layer output); configs with training rows add the backward
+(dX, dA, dB).  The default workload is the decode-heavy batch BASELINE.json's
+metric is quoted on (configs[1]); the other configs are selectable for
+profiling.  Steps are HIP-graph replays so the GPU, not Python, sets the pace;
+consecutive steps use different buffer sets, more than the 256 MB Infinity
+Cache holds in total, so weights and activations come from HBM.
+
+Prints one JSON line (see the keys below); `roofline` is for the dominant
+kernel measured alone with HIP events on the launch stream, `cpu_baseline` is
+the per-segment torch restatement of the reference timed on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "SMLM tokens/s + HBM GB/s (% of 8 TB/s), Llama-2-7B shapes, 1 GPU"
+
+
+def workload(name: str):
+    """Shapes and routing of BASELINE.json's configs 2-5 (seeds = config number)."""
+    if name == "cfg2":
+        ids = np.random.default_rng(2).integers(0, 32, 256).tolist()
+        return dict(name="cfg2: 256 single-token segments over 32 adapters, r=16, q/k/v/o 4096->4096, "
+                         "fp16, forward", dtype="fp16", r=16, NA=32, seg=list(range(257)), ids=ids,
+                    proj=[("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096)],
+                    n_train_parts=0)
+    if name == "cfg3":
+        return dict(name="cfg3: 4x512 prefill + 64 decode, 16 adapters, r=32, gate/up 4096->11008, "
+                         "down 11008->4096, fp16, forward", dtype="fp16", r=32, NA=16,
+                    seg=[0, 512, 1024, 1536, 2048] + list(range(2049, 2113)),
+                    ids=[i % 16 for i in range(68)],
+                    proj=[("gate", 4096, 11008), ("up", 4096, 11008), ("down", 11008, 4096)],
+                    n_train_parts=0)
+    if name == "cfg4":
+        return dict(name="cfg4: 4x1024 training rows (fwd+bwd) + 128 decode, 36 adapters, r=16, "
+                         "4096->4096, bf16", dtype="bf16", r=16, NA=36,
+                    seg=[0, 1024, 2048, 3072, 4096] + list(range(4097, 4225)),
+                    ids=[0, 1, 2, 3] + [4 + i % 32 for i in range(128)],
+                    proj=[("h", 4096, 4096)], n_train_parts=4)
+    if name == "cfg5":
+        rng = np.random.default_rng(5)
+        lens = []
+        while sum(lens) < 8192:
+            lens.append(int(np.clip(rng.geometric(1 / 8), 1, 2048)))
+        lens[-1] -= sum(lens) - 8192
+        seg = np.concatenate([[0], np.cumsum(lens)]).tolist()
+        S = len(lens)
+        return dict(name="cfg5: 64 adapters, ranks {8,16,32,64} padded to 64, geometric segments, 8192 "
+                         "rows, Llama-3-8B shapes, bf16, fwd + bwd on first quarter of segments",
+                    dtype="bf16", r=64, NA=64, seg=seg, ids=[i % 64 for i in range(S)],
+                    proj=[("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024),
+                          ("gate", 4096, 14336), ("up", 4096, 14336), ("down", 14336, 4096)],
+                    n_train_parts=S // 4, true_ranks=[8, 16, 32, 64])
+    raise SystemExit(f"unknown config {name}")
+
+
+def algorithmic_bytes(w, h_in, h_out, accumulate=True):
+    """Forward bytes of one projection: x and y once (y read too when accumulating),
+    A and B of each distinct active adapter once, v written and read once at I/O width."""
+    T = w["seg"][-1]
+    active = sorted(set(w["ids"]))
+    ranks = w.get("true_ranks")
+    rsum = sum((ranks[a % 4] if ranks else w["r"]) for a in active)
+    vbytes = 0
+    for i, a in enumerate(w["ids"]):
+        n = w["seg"][i + 1] - w["seg"][i]
+        vbytes += 2 * n * (ranks[a % 4] if ranks else w["r"]) * 2
+    return (T * h_in + T * h_out * (2 if accumulate else 1)) * 2 + rsum * (h_in + h_out) * 2 + vbytes
+
+
+def backward_bytes(w, h_in, h_out):
+    """dY and x read once, dX written, A/B read and dA/dB written per training adapter, v and dV."""
+    P = w["n_train_parts"]
+    n = w["seg"][P]
+    train = sorted(set(w["ids"][:P]))
+    ranks = w.get("true_ranks")
+    rsum = sum((ranks[a % 4] if ranks else w["r"]) for a in train)
+    return n * (h_out + 2 * h_in) * 2 + 2 * rsum * (h_in + h_out) * 2 + 3 * n * w["r"] * 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="cfg2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; every box has one MI355X and no collective, "
+              "sharding or rank code exists in it. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
+    from loquetier_amd import _lib
+    from loquetier_amd.ops import _kernels as K
+    _lib.load()  # no fallback: raises when the HIP library is missing
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = workload(args.config)
+    tdt = torch.float16 if w["dtype"] == "fp16" else torch.bfloat16
+    T, S, r, NA = w["seg"][-1], len(w["ids"]), w["r"], w["NA"]
+    P = w["n_train_parts"]
+    n_train = w["seg"][P] if P else 0
+
+    fwd_bytes = sum(algorithmic_bytes(w, hi, ho) for _, hi, ho in w["proj"])
+    bwd_bytes = sum(backward_bytes(w, hi, ho) for _, hi, ho in w["proj"]) if P else 0
+    footprint = sum((T * (hi + ho) + NA * r * (hi + ho)) * 2 for _, hi, ho in w["proj"])
+    if P:
+        footprint += sum(n_train * (hi + ho) * 2 for _, hi, ho in w["proj"])
+    R = 1 if args.no_rotate else max(2, math.ceil(640e6 / footprint))
+    R = min(R, 16)
+
+    gen = torch.Generator(device="cpu").manual_seed(int(args.config[-1]))
+    seg_t = torch.tensor(w["seg"], dtype=torch.int32, device=dev)
+    ids_t = torch.tensor(w["ids"], dtype=torch.int32, device=dev)
+    scale_t = torch.full((S,), 2.0, device=dev)
+
+    def randn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=gen) * std).to(dev).to(tdt)
+
+    ranks = w.get("true_ranks")
+    sets = []
+    for _ in range(R):
+        projs = []
+        for _, hi, ho in w["proj"]:
+            A = randn(NA, r, hi, std=hi ** -0.5)
+            B = randn(NA, ho, r, std=r ** -0.5)
+            if ranks:  # true rank below the padded rank: zero the padding (mixed_lora.py:501-521)
+                for a in range(NA):
+                    A[a, ranks[a % 4]:] = 0
+                    B[a, :, ranks[a % 4]:] = 0
+            d = dict(x=randn(T, hi), y=randn(T, ho), A=A, B=B,
+                     a_tab=torch.tensor([A[a].data_ptr() for a in range(NA)], dtype=torch.int64, device=dev),
+                     b_tab=torch.tensor([B[a].data_ptr() for a in range(NA)], dtype=torch.int64, device=dev))
+            if P:
+                train = sorted(set(w["ids"][:P]))
+                d.update(g=randn(n_train, ho), dx=torch.empty(n_train, hi, dtype=tdt, device=dev),
+                         v=torch.empty(T, r, dtype=tdt, device=dev),
+                         dA=torch.empty(len(train), r, hi, dtype=tdt, device=dev),
+                         dB=torch.empty(len(train), ho, r, dtype=tdt, device=dev))
+                d["ta_tab"] = torch.tensor([A[a].data_ptr() for a in train], dtype=torch.int64, device=dev)
+                d["tb_tab"] = torch.tensor([B[a].data_ptr() for a in train], dtype=torch.int64, device=dev)
+                d["da_tab"] = torch.tensor([d["dA"][i].data_ptr() for i in range(len(train))],
+                                           dtype=torch.int64, device=dev)
+                d["db_tab"] = torch.tensor([d["dB"][i].data_ptr() for i in range(len(train))],
+                                           dtype=torch.int64, device=dev)
+            projs.append(d)
+        sets.append(dict(proj=projs,
+                         plan_buf=torch.empty(K.SegmentPlan.nbytes(T, S), dtype=torch.uint8, device=dev),
+                         bplan_buf=torch.empty(K.SegmentPlan.nbytes(max(n_train, 1), max(P, 1)),
+                                               dtype=torch.uint8, device=dev)))
+    if P:
+        train = sorted(set(w["ids"][:P]))
+        part_indptr = torch.tensor(w["seg"][:P + 1], dtype=torch.int32, device=dev)
+        part_ad = torch.tensor([train.index(a) for a in w["ids"][:P]], dtype=torch.int32, device=dev)
+        part_scale = torch.full((P,), 2.0, device=dev)
+
+    def step(st):
+        plan = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
+        pr = st["proj"]
+        K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
+                                  [d["b_tab"] for d in pr], plan, r, seg_scale=scale_t, beta=1.0,
+                                  v_out=[d["v"] for d in pr] if P else None)
+        if P:
+            bplan = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
+            for d in st["proj"]:
+                K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
+                                     d["ta_tab"], d["tb_tab"], bplan, r, part_scale)
+
+    # eager once on the capture stream (sizes its workspace outside any capture), then one
+    # graph per buffer set
+    cap_stream = torch.cuda.Stream()
+    with torch.cuda.stream(cap_stream):
+        for st in sets:
+            step(st)
+    torch.cuda.synchronize()
+    graphs = []
+    for st in sets:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=cap_stream):
+            step(st)
+        graphs.append(g)
+    torch.cuda.synchronize()
+
+    def run(n):
+        for i in range(n):
+            graphs[i % R].replay()
+
+    run(args.warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    run(args.steps)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    tokens_per_s = T / (ms_per_step * 1e-3)
+    step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel alone: the expand kernel of one projection (y += s * v B^T), launched
+    # back to back from a graph over the rotating buffer sets, timed with HIP events on its stream
+    _, hi0, ho0 = max(w["proj"], key=lambda p: p[2])
+    pidx = [p[2] for p in w["proj"]].index(ho0)
+    v16 = [torch.randn(T, r, generator=gen).to(dev).to(tdt) for _ in range(R)]
+    plans = [K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"]) for st in sets]
+    reps = max(4, 48 // R)
+
+    def expand_only():
+        for _ in range(reps):
+            for i, st in enumerate(sets):
+                d = st["proj"][pidx]
+                K.smlm_gemm_planned(d["y"], v16[i], d["b_tab"], plans[i], seg_scale=scale_t, beta=1.0)
+
+    def shrink_only():
+        for _ in range(reps):
+            for i, st in enumerate(sets):
+                d = st["proj"][pidx]
+                K.smlm_gemm_planned(v16[i], d["x"], d["a_tab"], plans[i])
+
+    def time_graph(fn, launches):
+        with torch.cuda.stream(cap_stream):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=cap_stream):
+            fn()
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n_rep = 10
+        a.record()
+        for _ in range(n_rep):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / (n_rep * launches)  # us per launch
+
+    n_act = len(set(w["ids"]))
+    rsum = sum((ranks[a % 4] if ranks else r) for a in set(w["ids"]))
+    expand_us = time_graph(expand_only, reps * R)
+    expand_bytes = T * ho0 * 2 * 2 + rsum * ho0 * 2 + T * r * 2
+    shrink_us = time_graph(shrink_only, reps * R)
+    shrink_bytes = T * hi0 * 2 + rsum * hi0 * 2 + T * r * 2
+    traffic = None
+    tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(args.config, {}).get("expand_bytes_per_launch")
+    achieved = expand_bytes / (expand_us * 1e-6) / 1e9
+    roofline = dict(kernel="expand_kernel", bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
+                    unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
+                    us_per_launch=round(expand_us, 3), algorithmic_bytes=expand_bytes,
+                    projection=f"{hi0}->{ho0}")
+
+    # ---- CPU baseline: per-segment torch matmuls on the host cores (bounded sample)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import torch_segments as ref
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        cores = torch.get_num_threads()
+        st = sets[0]
+        host = [dict(x=d["x"].cpu(), y=d["y"].cpu(), A=[a.cpu() for a in d["A"]],
+                     B=[b.cpu() for b in d["B"]], g=d["g"].cpu() if P else None) for d in st["proj"]]
+        seg, ids = w["seg"], w["ids"]
+
+        def cpu_step():
+            for h in host:
+                ref.add_lora_forward(h["x"], [h["A"][a] for a in ids], [h["B"][a] for a in ids], seg,
+                                     y=h["y"], beta=1.0, seg_scale=[2.0] * S)
+                if P:
+                    ref.add_lora_backward(h["g"], h["x"][:n_train], h["A"], h["B"], seg[:P + 1], ids[:P])
+
+        cpu_step()
+        n, t_begin = 0, time.perf_counter()
+        while True:
+            cpu_step()
+            n += 1
+            el = time.perf_counter() - t_begin
+            if el > 12.0 or n >= 200:
+                break
+        cpu = dict(value=round(T * n / el, 1), unit="tokens/s", cores=cores, kind="port",
+                   sample=f"{n} whole steps of the same workload ({el:.1f} s), per-segment torch.matmul "
+                          f"in fp32 on {w['dtype']} data (oracle/torch_segments.py)")
+
+    out = {
+        "metric": METRIC, "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if w["dtype"] == "fp16" else "bf16", "data": "synthetic",
+        "config": {"workload": w["name"], "tokens_per_step": T, "segments": S, "adapters": NA, "rank": r,
+                   "projections": [f"{n}:{a}->{b}" for n, a, b in w["proj"]],
+                   "buffer_sets_rotated": R, "step_includes": "plan build + fused forward per projection"
+                   + (" + backward" if P else ""), "graph_replay": True},
+        "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
+        "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
+        "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "roofline": roofline,
+        "kernels": {"shrink_us": round(shrink_us, 3),
+                    "shrink_gbps": round(shrink_bytes / (shrink_us * 1e-6) / 1e9, 1),
+                    "expand_us": round(expand_us, 3), "expand_gbps": round(achieved, 1)},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

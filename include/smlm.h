@@ -76,10 +76,16 @@ SMLM_API int smlm_tmp_size(int num_problems, size_t* bytes);
  * (seg_indptr, keys): one plan serves every layer and projection of a batch.
  *   seg_key: NULL for SMLM_KEY_NONE, const int32_t* [S] for SMLM_KEY_I32,
  *            const void* const* [S] for SMLM_KEY_PTR (device memory).
+ * The key kind also fixes how the GEMM entry points below index their weight
+ * tables: a plan built with SMLM_KEY_I32 makes them read w_ptrs[key] (the
+ * table has one entry per adapter -- the gather wa_ptrs[lora_ids] of
+ * src/loquetier_src/models/mixed_lora.py:182 done inside the kernel); any other
+ * plan makes them read w_ptrs[i] for segment i (one entry per segment).
+ * Segments that share a key must share their weights.
  */
 SMLM_API int smlm_plan_size(int T, int S, size_t* bytes);
 SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr,
-                    const void* seg_key, int key_kind, int T, int S, void* stream);
+                             const void* seg_key, int key_kind, int T, int S, void* stream);
 
 /*
  * Grouped GEMM  Y_i = beta*Y_i + scale_i * X_i W_i  over the segments.
@@ -93,9 +99,22 @@ SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_i
  */
 SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes);
 SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const int32_t* seg_indptr,
-              void* workspace, size_t workspace_bytes, int T, int S, int d_in, int d_out,
-              int w_ld, int w_row_major, int dtype, float beta, const float* seg_scale,
-              void* stream);
+                       void* workspace, size_t workspace_bytes, int T, int S, int d_in, int d_out,
+                       int w_ld, int w_row_major, int dtype, float beta, const float* seg_scale,
+                       void* stream);
+
+/*
+ * The same grouped GEMM with a plan built beforehand by smlm_plan_build for
+ * (seg_indptr, T, S): nothing but the GEMM kernels is launched, so a caller
+ * that issues many GEMMs over one batch (every layer and projection of a
+ * model step) pays for the plan once.  No counterpart in the reference, which
+ * rebuilds its problem table inside every call (smlm_forward_cutlass.cuh:76-79).
+ */
+SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t* bytes);
+SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs, const void* plan,
+                               void* workspace, size_t workspace_bytes, int T, int S, int d_in,
+                               int d_out, int w_ld, int w_row_major, int dtype, float beta,
+                               const float* seg_scale, void* stream);
 
 /*
  * Fused LoRA forward  y = beta*y + scale_i * round16(x A^T) B^T.
@@ -103,19 +122,34 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
  * (src/loquetier_src/kernel_utils.py:115-119) plus, with beta = 1 and
  * seg_scale, the scale multiply and residual add of MixedLoraLinear.forward
  * (src/loquetier_src/models/mixed_lora.py:214-217).
- *   a_ptrs / b_ptrs: device arrays of device addresses.  With seg_adapter
- *     (int32 [S], device) they are per-adapter tables indexed by
- *     seg_adapter[i] -- the gather wa_ptrs[lora_ids] of mixed_lora.py:182
- *     done inside the kernel; with seg_adapter = NULL they are per-segment.
- *   plan: built by smlm_plan_build for the same (seg_indptr, T, S).
+ *   a_ptrs / b_ptrs: device arrays of device addresses, indexed as the plan's
+ *     key kind says (see smlm_plan_build).
+ *   plan: built by smlm_plan_build for the batch's (seg_indptr, T, S).
  *   v_out: NULL, or [T, r] receiving the rounded intermediate for backward.
  */
 SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes);
 SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* const* a_ptrs,
-                  const void* const* b_ptrs, const int32_t* seg_adapter,
-                  const int32_t* seg_indptr, const void* plan, void* workspace,
-                  size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
-                  float beta, const float* seg_scale, void* stream);
+                           const void* const* b_ptrs, const void* plan, void* workspace,
+                           size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
+                           float beta, const float* seg_scale, void* stream);
+
+/*
+ * The fused forward for up to 8 projections of one batch in two launches (one
+ * shrink, one expand): q/k/v/o or gate/up/down of a layer share the plan, the
+ * rank and the segment routing, and in the decode regime a launch costs as much
+ * as the data movement of one projection.  y, x, v_out, a_ptrs, b_ptrs, h_in,
+ * h_out are HOST arrays of n_proj entries (v_out may be NULL or hold NULLs);
+ * projections may differ in h_in / h_out.  No counterpart in the reference,
+ * which calls its kernel once per linear layer (mixed_lora.py:198-205).
+ */
+SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_in, int r,
+                                                size_t* bytes);
+SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* x,
+                                 void* const* v_out, const void* const* const* a_ptrs,
+                                 const void* const* const* b_ptrs, const int* h_in,
+                                 const int* h_out, const void* plan, void* workspace,
+                                 size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
+                                 const float* seg_scale, void* stream);
 
 /*
  * LoRA backward for fine-tuning rows.  Replaces add_lora.backward
@@ -130,18 +164,19 @@ SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* cons
  * is fixed, no atomics.  dx rows [0, n_rows) covered by a partition are
  * overwritten, others untouched.
  *   plan: built by smlm_plan_build(part_indptr, part_adapter, SMLM_KEY_I32,
- *         n_rows, P).   v: NULL (recomputed from x and A) or [n_rows, r].
+ *         n_rows, P); it carries the partitions and their adapters.
+ *   a_ptrs, b_ptrs, da_ptrs, db_ptrs: device arrays of NA device addresses.
+ *   v: NULL (recomputed from x and A) or [n_rows, r].
  *   part_scale: NULL or float [P] (device), the forward's seg_scale.
  * Needs n_rows >= 1, P >= 1, NA >= 1 and r <= 64.
  */
 SMLM_API int smlm_lora_bwd_workspace_size(int n_rows, int P, int NA, int h_in, int h_out, int r,
-                                 size_t* bytes);
+                                          size_t* bytes);
 SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs, const void* dy,
-                  const void* x, const void* v, const void* const* a_ptrs,
-                  const void* const* b_ptrs, const int32_t* part_adapter,
-                  const int32_t* part_indptr, const void* plan, void* workspace,
-                  size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out, int r,
-                  int dtype, const float* part_scale, void* stream);
+                           const void* x, const void* v, const void* const* a_ptrs,
+                           const void* const* b_ptrs, const void* plan, void* workspace,
+                           size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out,
+                           int r, int dtype, const float* part_scale, void* stream);
 
 #ifdef __cplusplus
 }

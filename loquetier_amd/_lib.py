@@ -17,6 +17,8 @@ SMLM_ERR_DTYPE = -2
 
 _vp, _i, _sz, _f = C.c_void_p, C.c_int, C.c_size_t, C.c_float
 _psz = C.POINTER(C.c_size_t)
+_pi = C.POINTER(C.c_int)
+_pvp = C.POINTER(C.c_void_p)
 
 # name -> (restype, argtypes); must list every symbol include/smlm.h declares
 SIGNATURES = {
@@ -27,12 +29,16 @@ SIGNATURES = {
     "smlm_plan_build": (_i, [_vp, _sz, _vp, _vp, _i, _i, _i, _vp]),
     "smlm_gemm_workspace_size": (_i, [_i, _i, _i, _i, _psz]),
     "smlm_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
+    "smlm_gemm_planned_workspace_size": (_i, [_i, _i, _i, _psz]),
+    "smlm_gemm_planned": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_lora_fwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _psz]),
-    "smlm_lora_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
-                           _f, _vp, _vp]),
+    "smlm_lora_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
+    "smlm_lora_fwd_multi_workspace_size": (_i, [_i, _i, _pi, _i, _psz]),
+    "smlm_lora_fwd_multi": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _pi, _pi, _vp, _vp, _sz, _i, _i, _i,
+                                 _i, _f, _vp, _vp]),
     "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
-    "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i,
-                           _i, _i, _i, _i, _i, _vp, _vp]),
+    "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
+                           _i, _vp, _vp]),
 }
 
 _lib = None
@@ -46,6 +52,12 @@ def load() -> C.CDLL:
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build it with `python -m loquetier_amd.build` "
                 "(hipcc, gfx950). There is no fallback path.")
+        # torch ships its own copy of the HIP runtime (soname libamdhip64.so.7) and
+        # hands out streams and device pointers that belong to that copy.  Importing
+        # torch first makes the loader resolve this library's libamdhip64.so.7 to the
+        # copy already in the process; the other order would put two runtimes in one
+        # process and every launch on a torch stream would fail.
+        import torch  # noqa: F401
         lib = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)

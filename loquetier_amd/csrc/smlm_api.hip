@@ -17,12 +17,31 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int round_up(int a, int b) { return ceil_div(a, b) * b; }
 
-int launch_status() { return hipGetLastError() == hipSuccess ? SMLM_OK : SMLM_ERR_LAUNCH; }
+// Every kernel takes one argument struct.  hipLaunchKernel hands back the
+// status of this launch itself; the thread's "last error" slot is shared with
+// every other HIP user in the process (torch leaves benign codes there), so it
+// is neither read nor cleared here.
+template <typename A>
+int launch(void (*kernel)(A), dim3 grid, dim3 block, hipStream_t st, const A& a) {
+  void* params[] = {const_cast<A*>(&a)};
+  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, params, 0, st) ==
+                 hipSuccess
+             ? SMLM_OK
+             : SMLM_ERR_LAUNCH;
+}
 
 // ---- launch shapes: functions of (T, d_in, d_out) only, never of the
 // segmentation, so re-segmenting a batch cannot change a bit of any row. ----
+inline int tiles_per_wave(int T) { return T >= 1024 ? kBlkTiles : 1; }
+
+// upper bound of the number of work units along the tile axis
+inline int tile_units(int T, int S, int mt) {
+  const int nt_max = plan_nt_max(T, S);
+  return mt == 1 ? nt_max : nt_max / kBlkTiles + S + 2;
+}
+
 struct ShrinkCfg {
-  int NB, U, ksplit, k_per_wave, zblocks;
+  int NB, U, MT, ksplit, k_per_wave, zblocks;
 };
 
 ShrinkCfg shrink_cfg(int T, int d_in, int d_out) {
@@ -31,70 +50,84 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out) {
   const int cols = d_out >= 64 ? 64 : d_out;
   c.NB = cols <= 16 ? 1 : (cols <= 32 ? 2 : 4);
   c.U = c.NB == 4 ? 2 : 4;
+  c.MT = tiles_per_wave(T);
   const int kq = 32 * c.U;
-  const int tiles = ceil_div(T > 0 ? T : 1, kTileRows);
-  const int want = ceil_div(1024, tiles);
+  const int units = ceil_div(T > 0 ? T : 1, kTileRows * c.MT);
+  const int want = ceil_div(1024, units);
   int max_split = d_in / (kFwdWaves * kq);
   if (max_split < 1) max_split = 1;
   if (max_split > 16) max_split = 16;
-  int ks = want < 1 ? 1 : (want > max_split ? max_split : want);
+  const int ks = want < 1 ? 1 : (want > max_split ? max_split : want);
   c.k_per_wave = round_up(ceil_div(d_in, kFwdWaves * ks), kq);
   c.ksplit = ceil_div(d_in, kFwdWaves * c.k_per_wave);
   return c;
 }
 
 int expand_nq(int T, int d_out) {
-  const int tiles = ceil_div(T > 0 ? T : 1, kTileRows);
-  return ((long)tiles * ceil_div(d_out, 512) >= 512) ? 4 : 2;
+  const int units = ceil_div(T > 0 ? T : 1, kTileRows * tiles_per_wave(T));
+  return ((long)units * ceil_div(d_out, 512) >= 512) ? 4 : 2;
 }
 
-TileArgs tile_args(const PlanView& pv) { return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg}; }
-
-template <int DT, bool RM>
-void launch_shrink_dt(const ShrinkCfg& c, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
-  if (c.NB == 1) hipLaunchKernelGGL((shrink_kernel<DT, 1, 4, RM>), grid, dim3(kFwdThreads), 0, st, a);
-  else if (c.NB == 2) hipLaunchKernelGGL((shrink_kernel<DT, 2, 4, RM>), grid, dim3(kFwdThreads), 0, st, a);
-  else hipLaunchKernelGGL((shrink_kernel<DT, 4, 2, RM>), grid, dim3(kFwdThreads), 0, st, a);
+TileArgs tile_args(const PlanView& pv) {
+  return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
 }
 
-int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int nt_max, hipStream_t st,
-                  const ShrinkArgs& a) {
-  dim3 grid(nt_max, c.ksplit, c.zblocks);
-  if (dtype == SMLM_DTYPE_F16) {
-    if (row_major) launch_shrink_dt<SMLM_DTYPE_F16, true>(c, grid, st, a);
-    else launch_shrink_dt<SMLM_DTYPE_F16, false>(c, grid, st, a);
-  } else {
-    if (row_major) launch_shrink_dt<SMLM_DTYPE_BF16, true>(c, grid, st, a);
-    else launch_shrink_dt<SMLM_DTYPE_BF16, false>(c, grid, st, a);
-  }
-  return launch_status();
+template <int DT, int MT, bool RM>
+int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, MT, RM>, grid, dim3(kFwdThreads), st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, MT, RM>, grid, dim3(kFwdThreads), st, a);
+  return launch(shrink_kernel<DT, 4, 2, MT, RM>, grid, dim3(kFwdThreads), st, a);
+}
+
+template <int DT>
+int launch_shrink_dt(bool row_major, int NB, int MT, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
+  if (row_major) return launch_shrink_nb<DT, 1, true>(NB, grid, st, a);  // the slow layout: one tile per wave
+  if (MT == 1) return launch_shrink_nb<DT, 1, false>(NB, grid, st, a);
+  return launch_shrink_nb<DT, kBlkTiles, false>(NB, grid, st, a);
+}
+
+// all projections of one launch share NB / U / MT (same rank, same T)
+int launch_shrink(int dtype, bool row_major, int NB, int MT, int S, hipStream_t st, ShrinkArgs& a) {
+  if (row_major) MT = 1;
+  a.gx = tile_units(a.T, S, MT);
+  dim3 grid((unsigned)((long)a.gx * a.gy * a.nproj));
+  if (dtype == SMLM_DTYPE_F16) return launch_shrink_dt<SMLM_DTYPE_F16>(row_major, NB, MT, grid, st, a);
+  return launch_shrink_dt<SMLM_DTYPE_BF16>(row_major, NB, MT, grid, st, a);
 }
 
 int launch_reduce(int dtype, int nt_max, hipStream_t st, const ReduceArgs& a) {
   if (dtype == SMLM_DTYPE_F16)
-    hipLaunchKernelGGL((reduce_kernel<SMLM_DTYPE_F16>), dim3(nt_max), dim3(256), 0, st, a);
-  else
-    hipLaunchKernelGGL((reduce_kernel<SMLM_DTYPE_BF16>), dim3(nt_max), dim3(256), 0, st, a);
-  return launch_status();
+    return launch(reduce_kernel<SMLM_DTYPE_F16>, dim3(nt_max), dim3(256), st, a);
+  return launch(reduce_kernel<SMLM_DTYPE_BF16>, dim3(nt_max), dim3(256), st, a);
 }
 
-template <int DT, bool RM>
-void launch_expand_dt(int nq, dim3 grid, hipStream_t st, const ExpandArgs& a) {
-  if (nq == 4) hipLaunchKernelGGL((expand_kernel<DT, 4, RM>), grid, dim3(kFwdThreads), 0, st, a);
-  else hipLaunchKernelGGL((expand_kernel<DT, 2, RM>), grid, dim3(kFwdThreads), 0, st, a);
+template <int DT, int NQ, int MT>
+int launch_expand_ks(int KS, dim3 grid, hipStream_t st, const ExpandArgs& a) {
+  if (KS == 1) return launch(expand_kernel<DT, NQ, 1, MT, false>, grid, dim3(kFwdThreads), st, a);
+  if (KS == 2) return launch(expand_kernel<DT, NQ, 2, MT, false>, grid, dim3(kFwdThreads), st, a);
+  return launch(expand_kernel<DT, NQ, 0, MT, false>, grid, dim3(kFwdThreads), st, a);
 }
 
-int launch_expand(int dtype, bool row_major, int nq, int nt_max, hipStream_t st,
-                  const ExpandArgs& a) {
-  dim3 grid(nt_max, ceil_div(a.d_out, kFwdWaves * 32 * nq));
-  if (dtype == SMLM_DTYPE_F16) {
-    if (row_major) launch_expand_dt<SMLM_DTYPE_F16, true>(nq, grid, st, a);
-    else launch_expand_dt<SMLM_DTYPE_F16, false>(nq, grid, st, a);
-  } else {
-    if (row_major) launch_expand_dt<SMLM_DTYPE_BF16, true>(nq, grid, st, a);
-    else launch_expand_dt<SMLM_DTYPE_BF16, false>(nq, grid, st, a);
-  }
-  return launch_status();
+template <int DT>
+int launch_expand_dt(bool row_major, int nq, int KS, int MT, dim3 grid, hipStream_t st,
+                     const ExpandArgs& a) {
+  if (row_major) return launch(expand_kernel<DT, 2, 0, 1, true>, grid, dim3(kFwdThreads), st, a);
+  if (MT == 1)
+    return nq == 4 ? launch_expand_ks<DT, 4, 1>(KS, grid, st, a) : launch_expand_ks<DT, 2, 1>(KS, grid, st, a);
+  return nq == 4 ? launch_expand_ks<DT, 4, kBlkTiles>(KS, grid, st, a)
+                 : launch_expand_ks<DT, 2, kBlkTiles>(KS, grid, st, a);
+}
+
+// all projections of one launch share the rank (d_in); d_out may differ
+int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int max_d_in, int max_d_out,
+                  hipStream_t st, ExpandArgs& a) {
+  if (row_major) { MT = 1; nq = 2; }
+  const int KS = max_d_in <= 32 ? 1 : (max_d_in <= 64 ? 2 : 0);
+  a.gx = tile_units(a.T, S, MT);
+  a.gy = ceil_div(max_d_out, kFwdWaves * 32 * nq);
+  dim3 grid((unsigned)((long)a.gx * a.gy * a.nproj));
+  if (dtype == SMLM_DTYPE_F16) return launch_expand_dt<SMLM_DTYPE_F16>(row_major, nq, KS, MT, grid, st, a);
+  return launch_expand_dt<SMLM_DTYPE_BF16>(row_major, nq, KS, MT, grid, st, a);
 }
 
 int check_common(int T, int S, int dtype) {
@@ -107,18 +140,43 @@ int check_common(int T, int S, int dtype) {
 int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* seg_key,
                     int key_kind, int S, hipStream_t st) {
   const int N = next_pow2(S);
-  if (N <= kPlanLdsKeys)
-    hipLaunchKernelGGL(plan_sort_kernel<true>, dim3(1), dim3(kPlanThreads), 0, st, pv, seg_indptr,
-                       seg_key, key_kind, S, N);
-  else
-    hipLaunchKernelGGL(plan_sort_kernel<false>, dim3(1), dim3(kPlanThreads), 0, st, pv, seg_indptr,
-                       seg_key, key_kind, S, N);
-  int rc = launch_status();
+  const PlanSortArgs sa{pv, seg_indptr, seg_key, key_kind, S, N};
+  if (S <= kPlanSmallSegs && pv.nt_max <= kPlanSmallTiles)
+    return launch(plan_small_kernel, dim3(1), dim3(kPlanThreads), st, sa);
+  int rc = (N <= kPlanLdsKeys)
+               ? launch(plan_sort_kernel<true>, dim3(1), dim3(kPlanThreads), st, sa)
+               : launch(plan_sort_kernel<false>, dim3(1), dim3(kPlanThreads), st, sa);
   if (rc) return rc;
   const long slots = (long)pv.nt_max * kTileRows;
-  hipLaunchKernelGGL(plan_fill_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, st, pv,
-                     seg_indptr, S);
-  return launch_status();
+  const PlanFillArgs fa{pv, seg_indptr, S};
+  return launch(plan_fill_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), st, fa);
+}
+
+// shrink of one or more projections that share x-row routing and rank
+int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int nproj,
+               const void* const* x, const void* const* const* w_ptrs, float* const* partial,
+               void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
+               const float* seg_scale, hipStream_t st, ShrinkCfg* cfgs) {
+  ShrinkArgs a{};
+  a.plan = tile_args(pv);
+  a.seg_scale = seg_scale;
+  a.beta = beta;
+  a.T = T;
+  a.nproj = nproj;
+  a.gy = 1;
+  for (int i = 0; i < nproj; ++i) {
+    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out);
+    cfgs[i] = c;
+    ShrinkProj& P = a.p[i];
+    P.x = reinterpret_cast<const uint16_t*>(x[i]);
+    P.w_ptrs = w_ptrs[i];
+    P.partial = partial[i];
+    P.out = reinterpret_cast<uint16_t*>(out[i]);
+    P.d_in = d_in[i]; P.d_out = d_out; P.ldw = ldw[i];
+    P.k_per_wave = c.k_per_wave; P.ksplit = c.ksplit; P.zblocks = c.zblocks;
+    if (c.ksplit * c.zblocks > a.gy) a.gy = c.ksplit * c.zblocks;
+  }
+  return launch_shrink(dtype, row_major, cfgs[0].NB, cfgs[0].MT, S, st, a);
 }
 
 struct BwdLayout {
@@ -184,8 +242,8 @@ SMLM_API int smlm_plan_size(int T, int S, size_t* bytes) {
   return SMLM_OK;
 }
 
-SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr, const void* seg_key,
-                    int key_kind, int T, int S, void* stream) {
+SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr,
+                             const void* seg_key, int key_kind, int T, int S, void* stream) {
   if (T < 0 || S < 0) return SMLM_ERR_ARG;
   if (S >= kMaxSegments || T > (1 << 30)) return SMLM_ERR_LIMIT;
   if (key_kind != SMLM_KEY_NONE && key_kind != SMLM_KEY_I32 && key_kind != SMLM_KEY_PTR)
@@ -198,21 +256,83 @@ SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_i
   return plan_build_impl(pv, seg_indptr, seg_key, key_kind, S, (hipStream_t)stream);
 }
 
-SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes) {
-  if (T < 0 || S < 0 || d_in <= 0 || d_out <= 0 || !bytes) return SMLM_ERR_ARG;
-  if (S >= kMaxSegments || T > (1 << 30)) return SMLM_ERR_LIMIT;
-  size_t n = plan_carve(nullptr, T, S, nullptr);
+SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t* bytes) {
+  if (T < 0 || d_in <= 0 || d_out <= 0 || !bytes) return SMLM_ERR_ARG;
+  if (T > (1 << 30)) return SMLM_ERR_LIMIT;
+  size_t n = 256;
   if (d_in >= d_out) {
     const ShrinkCfg c = shrink_cfg(T, d_in, d_out);
-    if (c.ksplit > 1) n += align_up((size_t)c.ksplit * T * d_out * 4, 256);
+    if (c.ksplit > 1) n = align_up((size_t)c.ksplit * T * d_out * 4, 256);
   }
   *bytes = n;
   return SMLM_OK;
 }
 
+SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs, const void* plan,
+                               void* workspace, size_t workspace_bytes, int T, int S, int d_in,
+                               int d_out, int w_ld, int w_row_major, int dtype, float beta,
+                               const float* seg_scale, void* stream) {
+  int rc = check_common(T, S, dtype);
+  if (rc) return rc;
+  if (d_in <= 0 || d_out <= 0 || w_ld <= 0) return SMLM_ERR_ARG;
+  if ((d_in & 7) || (d_out & 7) || (w_ld & 7)) return SMLM_ERR_ALIGN;
+  if (w_ld < (w_row_major ? d_out : d_in)) return SMLM_ERR_ARG;
+  if (T == 0 || S == 0) return SMLM_OK;
+  if (!y || !x || !w_ptrs || !plan || !workspace) return SMLM_ERR_ARG;
+  if (!aligned16(y) || !aligned16(x) || !aligned16(workspace) || !aligned16(plan))
+    return SMLM_ERR_ALIGN;
+  size_t need = 0;
+  rc = smlm_gemm_planned_workspace_size(T, d_in, d_out, &need);
+  if (rc) return rc;
+  if (workspace_bytes < need) return SMLM_ERR_WORKSPACE;
+
+  hipStream_t st = (hipStream_t)stream;
+  PlanView pv;
+  plan_carve(const_cast<void*>(plan), T, S, &pv);
+
+  if (d_in < d_out) {  // the reference's "expand" branch (smlm_forward_cutlass.cuh:82)
+    ExpandArgs a{};
+    a.plan = tile_args(pv);
+    a.seg_scale = seg_scale;
+    a.beta = beta;
+    a.T = T; a.nproj = 1; a.nt_max = pv.nt_max;
+    ExpandProj& P = a.p[0];
+    P.y = reinterpret_cast<uint16_t*>(y);
+    P.v = reinterpret_cast<const uint16_t*>(x);
+    P.w_ptrs = w_ptrs;
+    P.d_in = d_in; P.d_out = d_out; P.ldw = w_ld; P.ksplit = 1;
+    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T), S, d_in,
+                         d_out, st, a);
+  }
+  float* partial = reinterpret_cast<float*>(workspace);
+  ShrinkCfg c;
+  rc = run_shrink(dtype, w_row_major != 0, pv, T, S, 1, &x, &w_ptrs, &partial, &y, &d_in, d_out, &w_ld,
+                  beta, seg_scale, st, &c);
+  if (rc || c.ksplit == 1) return rc;
+  ReduceArgs ra{};
+  ra.plan = tile_args(pv);
+  ra.partial = partial;
+  ra.out = reinterpret_cast<uint16_t*>(y);
+  ra.seg_scale = seg_scale;
+  ra.beta = beta;
+  ra.T = T; ra.d_out = d_out; ra.ksplit = c.ksplit;
+  return launch_reduce(dtype, pv.nt_max, st, ra);
+}
+
+SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes) {
+  if (T < 0 || S < 0 || d_in <= 0 || d_out <= 0 || !bytes) return SMLM_ERR_ARG;
+  if (S >= kMaxSegments || T > (1 << 30)) return SMLM_ERR_LIMIT;
+  size_t extra = 0;
+  int rc = smlm_gemm_planned_workspace_size(T, d_in, d_out, &extra);
+  if (rc) return rc;
+  *bytes = plan_carve(nullptr, T, S, nullptr) + extra;
+  return SMLM_OK;
+}
+
 SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const int32_t* seg_indptr,
-              void* workspace, size_t workspace_bytes, int T, int S, int d_in, int d_out, int w_ld,
-              int w_row_major, int dtype, float beta, const float* seg_scale, void* stream) {
+                       void* workspace, size_t workspace_bytes, int T, int S, int d_in, int d_out,
+                       int w_ld, int w_row_major, int dtype, float beta, const float* seg_scale,
+                       void* stream) {
   int rc = check_common(T, S, dtype);
   if (rc) return rc;
   if (d_in <= 0 || d_out <= 0 || w_ld <= 0) return SMLM_ERR_ARG;
@@ -231,98 +351,106 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
   const size_t plan_bytes = plan_carve(workspace, T, S, &pv);
   rc = plan_build_impl(pv, seg_indptr, w_ptrs, SMLM_KEY_PTR, S, st);
   if (rc) return rc;
-
-  if (d_in < d_out) {  // the reference's "expand" branch (smlm_forward_cutlass.cuh:82)
-    ExpandArgs a{};
-    a.plan = tile_args(pv);
-    a.y = reinterpret_cast<uint16_t*>(y);
-    a.v = reinterpret_cast<const uint16_t*>(x);
-    a.w_ptrs = w_ptrs;
-    a.seg_scale = seg_scale;
-    a.beta = beta;
-    a.T = T; a.d_in = d_in; a.d_out = d_out; a.ldw = w_ld; a.ksplit = 1; a.nt_max = pv.nt_max;
-    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), pv.nt_max, st, a);
-  }
-  const ShrinkCfg c = shrink_cfg(T, d_in, d_out);
-  ShrinkArgs a{};
-  a.plan = tile_args(pv);
-  a.x = reinterpret_cast<const uint16_t*>(x);
-  a.w_ptrs = w_ptrs;
-  a.partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan_bytes);
-  a.out = reinterpret_cast<uint16_t*>(y);
-  a.seg_scale = seg_scale;
-  a.beta = beta;
-  a.T = T; a.d_in = d_in; a.d_out = d_out; a.ldw = w_ld;
-  a.k_per_wave = c.k_per_wave; a.ksplit = c.ksplit;
-  rc = launch_shrink(dtype, w_row_major != 0, c, pv.nt_max, st, a);
-  if (rc || c.ksplit == 1) return rc;
-  ReduceArgs ra{};
-  ra.plan = a.plan;
-  ra.partial = a.partial;
-  ra.out = a.out;
-  ra.seg_scale = seg_scale;
-  ra.beta = beta;
-  ra.T = T; ra.d_out = d_out; ra.ksplit = c.ksplit;
-  return launch_reduce(dtype, pv.nt_max, st, ra);
+  return smlm_gemm_planned(y, x, w_ptrs, workspace, reinterpret_cast<char*>(workspace) + plan_bytes,
+                           workspace_bytes - plan_bytes, T, S, d_in, d_out, w_ld, w_row_major, dtype,
+                           beta, seg_scale, stream);
 }
 
-SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes) {
-  if (T < 0 || S < 0 || h_in <= 0 || h_out <= 0 || r <= 0 || !bytes) return SMLM_ERR_ARG;
-  const ShrinkCfg c = shrink_cfg(T, h_in, r);
-  *bytes = align_up((size_t)c.ksplit * (T > 0 ? T : 1) * r * 4, 256);
+SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_in, int r,
+                                                size_t* bytes) {
+  if (n_proj < 1 || n_proj > kMaxProj || T < 0 || !h_in || r <= 0 || !bytes) return SMLM_ERR_ARG;
+  size_t n = 0;
+  for (int i = 0; i < n_proj; ++i) {
+    if (h_in[i] <= 0) return SMLM_ERR_ARG;
+    const ShrinkCfg c = shrink_cfg(T, h_in[i], r);
+    n += align_up((size_t)c.ksplit * (T > 0 ? T : 1) * r * 4, 256);
+  }
+  *bytes = n;
   return SMLM_OK;
 }
 
-SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* const* a_ptrs,
-                  const void* const* b_ptrs, const int32_t* seg_adapter, const int32_t* seg_indptr,
-                  const void* plan, void* workspace, size_t workspace_bytes, int T, int S, int h_in,
-                  int h_out, int r, int dtype, float beta, const float* seg_scale, void* stream) {
+SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* x,
+                                 void* const* v_out, const void* const* const* a_ptrs,
+                                 const void* const* const* b_ptrs, const int* h_in,
+                                 const int* h_out, const void* plan, void* workspace,
+                                 size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
+                                 const float* seg_scale, void* stream) {
   int rc = check_common(T, S, dtype);
   if (rc) return rc;
-  if (h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
-  if ((h_in & 7) || (h_out & 7) || (r & 7)) return SMLM_ERR_ALIGN;
+  if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
+    return SMLM_ERR_ARG;
+  if (r & 7) return SMLM_ERR_ALIGN;
+  int max_h_out = 0;
+  for (int i = 0; i < n_proj; ++i) {
+    if (h_in[i] <= 0 || h_out[i] <= 0) return SMLM_ERR_ARG;
+    if ((h_in[i] & 7) || (h_out[i] & 7)) return SMLM_ERR_ALIGN;
+    if (h_out[i] > max_h_out) max_h_out = h_out[i];
+  }
   if (T == 0 || S == 0) return SMLM_OK;
-  if (!y || !x || !a_ptrs || !b_ptrs || !seg_indptr || !plan || !workspace) return SMLM_ERR_ARG;
-  if (!aligned16(y) || !aligned16(x) || !aligned16(workspace) || !aligned16(plan) ||
-      (v_out && !aligned16(v_out)))
-    return SMLM_ERR_ALIGN;
+  if (!plan || !workspace) return SMLM_ERR_ARG;
+  if (!aligned16(workspace) || !aligned16(plan)) return SMLM_ERR_ALIGN;
+  for (int i = 0; i < n_proj; ++i) {
+    if (!y[i] || !x[i] || !a_ptrs[i] || !b_ptrs[i]) return SMLM_ERR_ARG;
+    if (!aligned16(y[i]) || !aligned16(x[i]) || (v_out && v_out[i] && !aligned16(v_out[i])))
+      return SMLM_ERR_ALIGN;
+  }
   size_t need = 0;
-  smlm_lora_fwd_workspace_size(T, S, h_in, h_out, r, &need);
+  rc = smlm_lora_fwd_multi_workspace_size(n_proj, T, h_in, r, &need);
+  if (rc) return rc;
   if (workspace_bytes < need) return SMLM_ERR_WORKSPACE;
 
   hipStream_t st = (hipStream_t)stream;
   PlanView pv;
   plan_carve(const_cast<void*>(plan), T, S, &pv);
-  const ShrinkCfg c = shrink_cfg(T, h_in, r);
 
-  ShrinkArgs sa{};
-  sa.plan = tile_args(pv);
-  sa.x = reinterpret_cast<const uint16_t*>(x);
-  sa.w_ptrs = a_ptrs;
-  sa.seg_adapter = seg_adapter;
-  sa.partial = reinterpret_cast<float*>(workspace);
-  sa.out = reinterpret_cast<uint16_t*>(workspace);  // 16-bit v when ksplit == 1
-  sa.beta = 0.0f;
-  sa.T = T; sa.d_in = h_in; sa.d_out = r; sa.ldw = h_in;
-  sa.k_per_wave = c.k_per_wave; sa.ksplit = c.ksplit;
-  rc = launch_shrink(dtype, false, c, pv.nt_max, st, sa);
+  // shrink: every projection's v as k-split fp32 partial sums (or 16-bit when not split)
+  float* partial[kMaxProj];
+  void* out16[kMaxProj];
+  ShrinkCfg cfgs[kMaxProj];
+  {
+    char* w = reinterpret_cast<char*>(workspace);
+    for (int i = 0; i < n_proj; ++i) {
+      const ShrinkCfg c = shrink_cfg(T, h_in[i], r);
+      partial[i] = reinterpret_cast<float*>(w);
+      out16[i] = w;
+      w += align_up((size_t)c.ksplit * T * r * 4, 256);
+    }
+  }
+  rc = run_shrink(dtype, false, pv, T, S, n_proj, x, a_ptrs, partial, out16, h_in, r, h_in, 0.0f,
+                  nullptr, st, cfgs);
   if (rc) return rc;
 
   ExpandArgs ea{};
-  ea.plan = sa.plan;
-  ea.y = reinterpret_cast<uint16_t*>(y);
-  if (c.ksplit > 1) ea.partial = sa.partial; else ea.v = sa.out;
-  ea.w_ptrs = b_ptrs;
-  ea.seg_adapter = seg_adapter;
+  ea.plan = tile_args(pv);
   ea.seg_scale = seg_scale;
-  ea.v_out = reinterpret_cast<uint16_t*>(v_out);
   ea.beta = beta;
-  ea.T = T; ea.d_in = r; ea.d_out = h_out; ea.ldw = r; ea.ksplit = c.ksplit; ea.nt_max = pv.nt_max;
-  return launch_expand(dtype, false, expand_nq(T, h_out), pv.nt_max, st, ea);
+  ea.T = T; ea.nproj = n_proj; ea.nt_max = pv.nt_max;
+  for (int i = 0; i < n_proj; ++i) {
+    ExpandProj& P = ea.p[i];
+    P.y = reinterpret_cast<uint16_t*>(y[i]);
+    if (cfgs[i].ksplit > 1) P.partial = partial[i]; else P.v = reinterpret_cast<const uint16_t*>(out16[i]);
+    P.w_ptrs = b_ptrs[i];
+    P.v_out = v_out ? reinterpret_cast<uint16_t*>(v_out[i]) : nullptr;
+    P.d_in = r; P.d_out = h_out[i]; P.ldw = r; P.ksplit = cfgs[i].ksplit;
+  }
+  return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, r, max_h_out, st, ea);
+}
+
+SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes) {
+  if (S < 0 || h_out <= 0) return SMLM_ERR_ARG;
+  return smlm_lora_fwd_multi_workspace_size(1, T, &h_in, r, bytes);
+}
+
+SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* const* a_ptrs,
+                           const void* const* b_ptrs, const void* plan, void* workspace,
+                           size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
+                           float beta, const float* seg_scale, void* stream) {
+  return smlm_lora_fwd_multi(1, &y, &x, v_out ? &v_out : nullptr, &a_ptrs, &b_ptrs, &h_in, &h_out, plan,
+                             workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale, stream);
 }
 
 SMLM_API int smlm_lora_bwd_workspace_size(int n_rows, int P, int NA, int h_in, int h_out, int r,
-                                 size_t* bytes) {
+                                          size_t* bytes) {
   if (n_rows < 0 || P < 0 || NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0 || !bytes)
     return SMLM_ERR_ARG;
   *bytes = bwd_layout(n_rows > 0 ? n_rows : 1, P, NA > 0 ? NA : 1, h_in, h_out, r).total;
@@ -330,11 +458,10 @@ SMLM_API int smlm_lora_bwd_workspace_size(int n_rows, int P, int NA, int h_in, i
 }
 
 SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs, const void* dy,
-                  const void* x, const void* v, const void* const* a_ptrs,
-                  const void* const* b_ptrs, const int32_t* part_adapter,
-                  const int32_t* part_indptr, const void* plan, void* workspace,
-                  size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out, int r,
-                  int dtype, const float* part_scale, void* stream) {
+                           const void* x, const void* v, const void* const* a_ptrs,
+                           const void* const* b_ptrs, const void* plan, void* workspace,
+                           size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out,
+                           int r, int dtype, const float* part_scale, void* stream) {
   int rc = check_common(n_rows, P, dtype);
   if (rc) return rc;
   if (NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
@@ -342,7 +469,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   if (r > 64) return SMLM_ERR_LIMIT;
   if (NA == 0 || n_rows == 0 || P == 0) return SMLM_ERR_ARG;
   if (!da_ptrs || !db_ptrs || !a_ptrs || !b_ptrs || !workspace) return SMLM_ERR_ARG;
-  if (!dx || !dy || !x || !part_adapter || !part_indptr || !plan) return SMLM_ERR_ARG;
+  if (!dx || !dy || !x || !plan) return SMLM_ERR_ARG;
   if (!aligned16(dx) || !aligned16(dy) || !aligned16(x) || !aligned16(v) || !aligned16(workspace) ||
       !aligned16(plan))
     return SMLM_ERR_ALIGN;
@@ -356,74 +483,65 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   const void** at_ptrs = reinterpret_cast<const void**>(ws + L.at_ptrs);
   const void** bt_ptrs = reinterpret_cast<const void**>(ws + L.bt_ptrs);
   float* partial = reinterpret_cast<float*>(ws + L.partial);
-  uint16_t* dv16 = reinterpret_cast<uint16_t*>(ws + L.dv16);
-  uint16_t* v16 = reinterpret_cast<uint16_t*>(ws + L.v16);
+  void* dv16 = ws + L.dv16;
+  void* v16 = ws + L.v16;
   uint16_t* pt_a = reinterpret_cast<uint16_t*>(ws + L.pt_a);
   uint16_t* pt_b = reinterpret_cast<uint16_t*>(ws + L.pt_b);
 
   PlanView pv{};
   plan_carve(const_cast<void*>(plan), n_rows, P, &pv);
-  {
 
-    // 1. transposed copies of the training adapters' weights: At [h_in, r], Bt [r, h_out]
-    TransposeArgs ta{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
-    hipLaunchKernelGGL(transpose_kernel, dim3(ceil_div(h_in, 32), ceil_div(r, 32), NA), dim3(256), 0,
-                       st, ta);
-    TransposeArgs tb{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
-    hipLaunchKernelGGL(transpose_kernel, dim3(ceil_div(r, 32), ceil_div(h_out, 32), NA), dim3(256), 0,
-                       st, tb);
-    if ((rc = launch_status())) return rc;
+  // 1. transposed copies of the training adapters' weights: At [h_in, r], Bt [r, h_out]
+  TransposeArgs ta{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
+  if ((rc = launch(transpose_kernel, dim3(ceil_div(h_in, 32), ceil_div(r, 32), NA), dim3(256), st, ta)))
+    return rc;
+  TransposeArgs tb{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
+  if ((rc = launch(transpose_kernel, dim3(ceil_div(r, 32), ceil_div(h_out, 32), NA), dim3(256), st, tb)))
+    return rc;
 
-    // 2. v = round16(x A^T) unless the forward saved it
-    const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
-    if (!vv) {
-      ShrinkArgs sa{};
-      sa.plan = tile_args(pv);
-      sa.x = reinterpret_cast<const uint16_t*>(x);
-      sa.w_ptrs = a_ptrs;
-      sa.seg_adapter = part_adapter;
-      sa.partial = partial;
-      sa.out = v16;
-      sa.T = n_rows; sa.d_in = h_in; sa.d_out = r; sa.ldw = h_in;
-      sa.k_per_wave = L.cfg_v.k_per_wave; sa.ksplit = L.cfg_v.ksplit;
-      if ((rc = launch_shrink(dtype, false, L.cfg_v, pv.nt_max, st, sa))) return rc;
-      if (L.cfg_v.ksplit > 1) {
-        ReduceArgs ra{};
-        ra.plan = sa.plan; ra.partial = partial; ra.out = v16;
-        ra.T = n_rows; ra.d_out = r; ra.ksplit = L.cfg_v.ksplit;
-        if ((rc = launch_reduce(dtype, pv.nt_max, st, ra))) return rc;
-      }
-      vv = v16;
+  // 2. v = round16(x A^T) unless the forward saved it
+  const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
+  ShrinkCfg c;
+  if (!vv) {
+    if ((rc = run_shrink(dtype, false, pv, n_rows, P, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
+                         0.0f, nullptr, st, &c)))
+      return rc;
+    if (c.ksplit > 1) {
+      ReduceArgs ra{};
+      ra.plan = tile_args(pv);
+      ra.partial = partial;
+      ra.out = reinterpret_cast<uint16_t*>(v16);
+      ra.T = n_rows; ra.d_out = r; ra.ksplit = c.ksplit;
+      if ((rc = launch_reduce(dtype, pv.nt_max, st, ra))) return rc;
     }
-
-    // 3. dV = dY B  (k-split partial sums, or 16-bit when not split)
-    ShrinkArgs sd{};
-    sd.plan = tile_args(pv);
-    sd.x = reinterpret_cast<const uint16_t*>(dy);
-    sd.w_ptrs = bt_ptrs;
-    sd.seg_adapter = part_adapter;
-    sd.partial = partial;
-    sd.out = dv16;
-    sd.T = n_rows; sd.d_in = h_out; sd.d_out = r; sd.ldw = h_out;
-    sd.k_per_wave = L.cfg_dv.k_per_wave; sd.ksplit = L.cfg_dv.ksplit;
-    if ((rc = launch_shrink(dtype, false, L.cfg_dv, pv.nt_max, st, sd))) return rc;
-
-    // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
-    ExpandArgs ea{};
-    ea.plan = sd.plan;
-    ea.y = reinterpret_cast<uint16_t*>(dx);
-    if (L.cfg_dv.ksplit > 1) ea.partial = partial; else ea.v = dv16;
-    ea.w_ptrs = at_ptrs;
-    ea.seg_adapter = part_adapter;
-    ea.seg_scale = part_scale;
-    ea.pt_a = pt_a;
-    ea.pt_b = pt_b;
-    ea.v2 = vv;
-    ea.beta = 0.0f;
-    ea.T = n_rows; ea.d_in = r; ea.d_out = h_in; ea.ldw = r; ea.ksplit = L.cfg_dv.ksplit;
-    ea.nt_max = pv.nt_max;
-    if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), pv.nt_max, st, ea))) return rc;
+    vv = reinterpret_cast<const uint16_t*>(v16);
   }
+
+  // 3. dV = dY B  (k-split partial sums, or 16-bit when not split)
+  const void* const* btp = bt_ptrs;
+  if ((rc = run_shrink(dtype, false, pv, n_rows, P, 1, &dy, &btp, &partial, &dv16, &h_out, r, &h_out,
+                       0.0f, nullptr, st, &c)))
+    return rc;
+
+  // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
+  ExpandArgs ea{};
+  ea.plan = tile_args(pv);
+  ea.seg_scale = part_scale;
+  ea.pt_a = pt_a;
+  ea.pt_b = pt_b;
+  ea.v2 = vv;
+  ea.beta = 0.0f;
+  ea.T = n_rows; ea.nproj = 1; ea.nt_max = pv.nt_max;
+  {
+    ExpandProj& E = ea.p[0];
+    E.y = reinterpret_cast<uint16_t*>(dx);
+    if (c.ksplit > 1) E.partial = partial; else E.v = reinterpret_cast<const uint16_t*>(dv16);
+    E.w_ptrs = at_ptrs;
+    E.d_in = r; E.d_out = h_in; E.ldw = r; E.ksplit = c.ksplit;
+  }
+  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, r, h_in, st,
+                          ea)))
+    return rc;
 
   // 5. dA_a, dB_a for every adapter (zeros when it has no rows)
   WgradArgs wa{};
@@ -443,15 +561,13 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA);
   const int nbj = ceil_div(r, 16);
   if (dtype == SMLM_DTYPE_F16) {
-    if (nbj == 1) hipLaunchKernelGGL((wgrad_kernel<SMLM_DTYPE_F16, 1>), grid, dim3(256), 0, st, wa);
-    else if (nbj == 2) hipLaunchKernelGGL((wgrad_kernel<SMLM_DTYPE_F16, 2>), grid, dim3(256), 0, st, wa);
-    else hipLaunchKernelGGL((wgrad_kernel<SMLM_DTYPE_F16, 4>), grid, dim3(256), 0, st, wa);
-  } else {
-    if (nbj == 1) hipLaunchKernelGGL((wgrad_kernel<SMLM_DTYPE_BF16, 1>), grid, dim3(256), 0, st, wa);
-    else if (nbj == 2) hipLaunchKernelGGL((wgrad_kernel<SMLM_DTYPE_BF16, 2>), grid, dim3(256), 0, st, wa);
-    else hipLaunchKernelGGL((wgrad_kernel<SMLM_DTYPE_BF16, 4>), grid, dim3(256), 0, st, wa);
+    if (nbj == 1) return launch(wgrad_kernel<SMLM_DTYPE_F16, 1>, grid, dim3(256), st, wa);
+    if (nbj == 2) return launch(wgrad_kernel<SMLM_DTYPE_F16, 2>, grid, dim3(256), st, wa);
+    return launch(wgrad_kernel<SMLM_DTYPE_F16, 4>, grid, dim3(256), st, wa);
   }
-  return launch_status();
+  if (nbj == 1) return launch(wgrad_kernel<SMLM_DTYPE_BF16, 1>, grid, dim3(256), st, wa);
+  if (nbj == 2) return launch(wgrad_kernel<SMLM_DTYPE_BF16, 2>, grid, dim3(256), st, wa);
+  return launch(wgrad_kernel<SMLM_DTYPE_BF16, 4>, grid, dim3(256), st, wa);
 }
 
 }  // extern "C"

@@ -15,6 +15,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTileRows = 16;     // rows of one MFMA tile = tokens per plan tile
+constexpr int kBlkTiles = 4;      // a tile block = up to this many consecutive tiles of one group
 constexpr int kWaveSize = 64;
 constexpr int kSegBits = 20;      // segment index bits inside a sort key
 constexpr int kMaxSegments = 1 << kSegBits;
@@ -70,24 +71,29 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return Num<DT>::bits(lo) | (Num<DT>::bits(hi) << 16);
 }
 
+// Global-memory accessors.  Addresses read from pointer tables carry no address
+// space, and a generic pointer makes the compiler emit flat instructions; every
+// pointer that reaches these helpers is device global memory, so say so.
+#define SMLM_GLOBAL __attribute__((address_space(1)))
 __device__ __forceinline__ u32x4 ldg16(const uint16_t* p) {
-  return *reinterpret_cast<const u32x4*>(p);
+  return *(const SMLM_GLOBAL u32x4*)(p);
 }
 __device__ __forceinline__ void stg16(uint16_t* p, u32x4 v) {
-  *reinterpret_cast<u32x4*>(p) = v;
+  *(SMLM_GLOBAL u32x4*)(p) = v;
 }
 __device__ __forceinline__ f32x4 ldg_f4(const float* p) {
-  return *reinterpret_cast<const f32x4*>(p);
+  return *(const SMLM_GLOBAL f32x4*)(p);
 }
 
 // Eight 16-bit elements with a stride (the slow gather used for the weight
 // layout the reference never passes).
 __device__ __forceinline__ u32x4 ldg_strided8(const uint16_t* p, long stride) {
+  const SMLM_GLOBAL uint16_t* q = (const SMLM_GLOBAL uint16_t*)p;
   u32x4 r;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    uint32_t a = p[(2 * i) * stride];
-    uint32_t b = p[(2 * i + 1) * stride];
+    uint32_t a = q[(2 * i) * stride];
+    uint32_t b = q[(2 * i + 1) * stride];
     r[i] = a | (b << 16);
   }
   return r;
@@ -95,15 +101,19 @@ __device__ __forceinline__ u32x4 ldg_strided8(const uint16_t* p, long stride) {
 
 // Views into a plan buffer (all int32).  Sizes are functions of (T, S) only.
 struct PlanView {
-  int32_t* hdr;         // [16]: 0 n_tiles, 1 n_groups, 2 rows covered, 3 key kind used
+  int32_t* hdr;         // [16]: 0 n_tiles, 1 n_groups, 2 rows covered, 3 key kind used, 4 n_blocks
   int32_t* sorted_seg;  // [S]   segment at sorted position p
   int32_t* rowpos;      // [S+1] first gathered-row index of sorted position p
   int32_t* grp_tile;    // [S+1] first tile of group G (exclusive scan), [NG] = n_tiles
   int32_t* grp_row;     // [S+1] first gathered-row index of group G, [NG] = rows covered
   int32_t* grp_seg;     // [S]   representative (first) segment of group G
   int32_t* grp_id;      // [S]   int32 key of group G (adapter id for SMLM_KEY_I32)
+  int32_t* grp_blk;     // [S+1] first tile block of group G, [NG] = n_blocks
   int32_t* tile_row;    // [nt_max*16] row index of each tile slot, -1 = empty
   int32_t* tile_rseg;   // [nt_max*16] segment of each tile slot, -1 = empty
+  int32_t* tile_wid;    // [nt_max] index into the caller's weight table: the int32 key for
+                        //          SMLM_KEY_I32 plans, else the group's first segment
+  int32_t* blk;         // [nt_max] tile block b: (first tile << 3) | number of tiles (1..4)
   uint64_t* sort_keys;  // [pow2 >= S] scratch for sorts that do not fit in LDS
   int nt_max;
 };
@@ -133,8 +143,11 @@ inline size_t plan_carve(void* base, int T, int S, PlanView* pv) {
   v.grp_row = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
   v.grp_seg = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
   v.grp_id = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
+  v.grp_blk = reinterpret_cast<int32_t*>(take((size_t)(S + 1) * 4));
   v.tile_row = reinterpret_cast<int32_t*>(take((size_t)nt_max * kTileRows * 4));
   v.tile_rseg = reinterpret_cast<int32_t*>(take((size_t)nt_max * kTileRows * 4));
+  v.tile_wid = reinterpret_cast<int32_t*>(take((size_t)nt_max * 4));
+  v.blk = reinterpret_cast<int32_t*>(take((size_t)nt_max * 4));
   v.sort_keys = reinterpret_cast<uint64_t*>(take((size_t)next_pow2(S > 0 ? S : 1) * 8));
   v.nt_max = nt_max;
   if (pv) *pv = v;

@@ -5,16 +5,30 @@
 // thread per segment writes a GEMM problem; here segments that share a key are
 // laid end to end (stable in segment order) and cut into 16-row tiles, so a
 // tile never mixes adapters and an adapter's rows share tiles.
+//
+// Two routes: batches of up to 1024 segments are planned by ONE workgroup in
+// one launch with every intermediate array in LDS (the decode regime, where a
+// second launch would cost as much as the GEMM); larger batches use a sort /
+// scan launch followed by a grid-wide fill launch.
 #pragma once
 #include "smlm_common.hpp"
 
 namespace smlm {
 
 constexpr int kPlanThreads = 1024;
-constexpr int kPlanLdsKeys = 4096;  // sorts up to this many keys stay in LDS
+constexpr int kPlanLdsKeys = 4096;   // two-launch route: sorts up to this many keys stay in LDS
+constexpr int kPlanSmallSegs = 1024; // one-launch route: at most this many segments ...
+constexpr int kPlanSmallTiles = 4096; // ... and at most this many possible tiles
+
+struct PlanSortArgs {
+  PlanView pv;
+  const int32_t* s;  // [S+1] segment boundaries
+  const void* key;   // per-segment keys, see SMLM_KEY_*
+  int key_kind, S, N;  // N = power of two >= S
+};
 
 // Inclusive scan of one 64-bit value per thread over a 1024-thread block.
-// `wave_tot` is LDS scratch of 16 entries.  Returns the inclusive prefix; the
+// `wave_tot` is LDS scratch of 17 entries.  Returns the inclusive prefix; the
 // block total is left in wave_tot[16].
 __device__ __forceinline__ uint64_t block_scan_incl(uint64_t v, uint64_t* wave_tot) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -39,67 +53,203 @@ __device__ __forceinline__ uint64_t block_scan_incl(uint64_t v, uint64_t* wave_t
   return v + wave_tot[wave];
 }
 
-// USE_LDS is a template parameter, not a run-time choice, so that the key array
-// is addressed with LDS instructions: a generic pointer that may point into LDS
-// makes the compiler emit flat accesses with folded immediate offsets, and a
-// flat access whose base register sits just below the LDS aperture (K[p-1] at
-// p = 0) is routed by the hardware on the base alone and faults.
+// Sort key of segment i: group key in the high bits, segment index in the low
+// kSegBits, so equal keys keep their segment order and no two keys are equal.
+__device__ __forceinline__ uint64_t make_key(const void* key, int kind, int i) {
+  if (kind == SMLM_KEY_I32)
+    return ((uint64_t)(uint32_t) reinterpret_cast<const int32_t*>(key)[i] << kSegBits) | (uint32_t)i;
+  if (kind == SMLM_KEY_PTR)
+    return ((reinterpret_cast<const uint64_t*>(key)[i] >> 4) << kSegBits) | (uint32_t)i;
+  return ((uint64_t)i << kSegBits) | (uint32_t)i;
+}
+
+// A 16-byte aligned address below 2^48 packs into 44 bits; anything else
+// cannot be a sort key, so such a batch is planned segment by segment.
+__device__ __forceinline__ int usable_kind(const void* key, int key_kind, int S, int* bad_key) {
+  if (threadIdx.x == 0) *bad_key = 0;
+  __syncthreads();
+  if (key_kind == SMLM_KEY_PTR) {
+    const uint64_t* pk = reinterpret_cast<const uint64_t*>(key);
+    for (int i = threadIdx.x; i < S; i += kPlanThreads)
+      if ((pk[i] >> 48) != 0 || (pk[i] & 15) != 0) *bad_key = 1;
+  }
+  __syncthreads();
+  return *bad_key ? SMLM_KEY_NONE : key_kind;
+}
+
+// Bitonic sort, ascending.  K must be addressed by the caller's own address
+// space (LDS array or global pointer), never through a pointer that could be
+// either: a generic pointer into LDS makes the compiler emit flat accesses
+// with folded immediate offsets, and a flat access whose base register sits
+// just below the LDS aperture is routed by the hardware on the base alone and
+// faults.
+template <typename KeyArray>
+__device__ __forceinline__ void bitonic_sort(KeyArray K, int N) {
+  for (int size = 2; size <= N; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = threadIdx.x; i < (N >> 1); i += kPlanThreads) {
+        const int lo = 2 * i - (i & (stride - 1));
+        const int hi = lo + stride;
+        const bool asc = (lo & size) == 0;
+        const uint64_t a = K[lo], b = K[hi];
+        if ((a > b) == asc) {
+          K[lo] = b;
+          K[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// last index i in [0, n) with a[i] <= q, given a[0] <= q < a[n]
+template <typename Arr>
+__device__ __forceinline__ int last_le(Arr a, int n, int q) {
+  int lo = 0, hi = n;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (a[mid] <= q) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// ---------------------------------------------------------------- one launch
+__global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs args) {
+  __shared__ uint64_t K[kPlanSmallSegs];
+  __shared__ int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];
+  __shared__ int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
+  __shared__ int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
+  __shared__ uint64_t wave_tot[17];
+  __shared__ int bad_key;
+  const PlanView pv = args.pv;
+  const int32_t* __restrict__ s = args.s;
+  const int S = args.S, N = args.N, tid = threadIdx.x;
+  const int kind = usable_kind(args.key, args.key_kind, S, &bad_key);
+
+  K[tid] = tid < S ? make_key(args.key, kind, tid) : ~0ull;
+  __syncthreads();
+  if (kind != SMLM_KEY_NONE) bitonic_sort(K, N);
+
+  // gathered-row position of every sorted segment, group heads
+  constexpr uint64_t kRowMask = (1ull << 40) - 1;
+  int seg = 0, len = 0;
+  uint64_t gk = 0;
+  bool head = false;
+  if (tid < S) {
+    const uint64_t k = K[tid];
+    seg = (int)(k & (kMaxSegments - 1));
+    gk = k >> kSegBits;
+    len = s[seg + 1] - s[seg];
+    if (len < 0) len = 0;
+    head = true;
+    if (tid > 0) head = (K[tid - 1] >> kSegBits) != gk;
+  }
+  const uint64_t v = (uint64_t)len | ((uint64_t)(head ? 1 : 0) << 40);
+  const uint64_t incl = block_scan_incl(v, wave_tot);
+  const uint64_t total = wave_tot[16];
+  const int rows_total = (int)(total & kRowMask), NG = (int)(total >> 40);
+  if (tid < S) {
+    const int rows_before = (int)((incl - v) & kRowMask);
+    sseg[tid] = seg;
+    rowpos[tid] = rows_before;
+    pv.sorted_seg[tid] = seg;
+    pv.rowpos[tid] = rows_before;
+    if (head) {
+      const int G = (int)(incl >> 40) - 1;
+      grow[G] = rows_before;
+      gseg[G] = seg;
+      gid[G] = (int32_t)(uint32_t)gk;
+    }
+  }
+  if (tid == 0) {
+    rowpos[S] = rows_total;
+    grow[NG] = rows_total;
+    pv.rowpos[S] = rows_total;
+  }
+  __syncthreads();
+
+  // tiles per group -> first tile of each group
+  uint64_t nt = 0;
+  if (tid < NG) nt = (uint64_t)((grow[tid + 1] - grow[tid] + kTileRows - 1) / kTileRows);
+  const uint64_t tincl = block_scan_incl(nt, wave_tot);
+  const int n_tiles = (int)wave_tot[16];
+  if (tid < NG) {
+    gtile[tid] = (int)(tincl - nt);
+    pv.grp_tile[tid] = (int)(tincl - nt);
+    pv.grp_row[tid] = grow[tid];
+    pv.grp_seg[tid] = gseg[tid];
+    pv.grp_id[tid] = gid[tid];
+  }
+  // tile blocks per group -> first block of each group
+  const uint64_t nb = (nt + kBlkTiles - 1) / kBlkTiles;
+  const uint64_t bincl = block_scan_incl(nb, wave_tot);
+  const int n_blocks = (int)wave_tot[16];
+  if (tid < NG) {
+    gblk[tid] = (int)(bincl - nb);
+    pv.grp_blk[tid] = (int)(bincl - nb);
+  }
+  if (tid == 0) {
+    gtile[NG] = n_tiles;
+    gblk[NG] = n_blocks;
+    pv.grp_tile[NG] = n_tiles;
+    pv.grp_blk[NG] = n_blocks;
+    pv.grp_row[NG] = rows_total;
+    pv.hdr[0] = n_tiles;
+    pv.hdr[1] = NG;
+    pv.hdr[2] = rows_total;
+    pv.hdr[3] = kind;
+    pv.hdr[4] = n_blocks;
+  }
+  __syncthreads();
+
+  for (int b = tid; b < n_blocks; b += kPlanThreads) {
+    const int G = last_le(gblk, NG, b);
+    const int tile0 = gtile[G] + (b - gblk[G]) * kBlkTiles;
+    const int left = gtile[G + 1] - tile0;
+    pv.blk[b] = (tile0 << 3) | (left < kBlkTiles ? left : kBlkTiles);
+  }
+
+  // fill: one thread per tile slot
+  for (int slot = tid; slot < n_tiles * kTileRows; slot += kPlanThreads) {
+    const int tile = slot / kTileRows, c = slot % kTileRows;
+    const int G = last_le(gtile, NG, tile);
+    const int q = grow[G] + (tile - gtile[G]) * kTileRows + c;
+    int row = -1, rseg = -1;
+    if (q < grow[G + 1]) {
+      const int a = last_le(rowpos, S, q);
+      rseg = sseg[a];
+      row = s[rseg] + (q - rowpos[a]);
+    }
+    pv.tile_row[slot] = row;
+    pv.tile_rseg[slot] = rseg;
+    if (c == 0) pv.tile_wid[tile] = (kind == SMLM_KEY_I32) ? gid[G] : gseg[G];
+  }
+}
+
+// --------------------------------------------------------------- two launches
 template <bool USE_LDS>
-__global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanView pv,
-                                                                 const int32_t* __restrict__ s,
-                                                                 const void* key, int key_kind,
-                                                                 int S, int N) {
+__global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs args) {
   __shared__ uint64_t lds_keys[USE_LDS ? kPlanLdsKeys : 1];
   __shared__ uint64_t wave_tot[17];
   __shared__ int bad_key;
   __shared__ uint64_t carry;
-  const int tid = threadIdx.x;
-  uint64_t* K = USE_LDS ? lds_keys : pv.sort_keys;
+  const PlanView pv = args.pv;
+  const int32_t* __restrict__ s = args.s;
+  const int S = args.S, N = args.N, tid = threadIdx.x;
+  const int kind = usable_kind(args.key, args.key_kind, S, &bad_key);
 
-  if (tid == 0) bad_key = 0;
-  __syncthreads();
-  if (key_kind == SMLM_KEY_PTR) {
-    // A 16-byte aligned address below 2^48 packs into 44 bits; anything else
-    // cannot be a sort key, so such a batch is planned segment by segment.
-    const uint64_t* pk = reinterpret_cast<const uint64_t*>(key);
-    for (int i = tid; i < S; i += kPlanThreads)
-      if ((pk[i] >> 48) != 0 || (pk[i] & 15) != 0) bad_key = 1;
+  if (USE_LDS) {
+    for (int i = tid; i < N; i += kPlanThreads) lds_keys[i] = i < S ? make_key(args.key, kind, i) : ~0ull;
     __syncthreads();
-  }
-  const int kind = bad_key ? SMLM_KEY_NONE : key_kind;
-
-  for (int i = tid; i < N; i += kPlanThreads) {
-    uint64_t k;
-    if (i >= S) {
-      k = ~0ull;
-    } else if (kind == SMLM_KEY_I32) {
-      k = ((uint64_t)(uint32_t) reinterpret_cast<const int32_t*>(key)[i] << kSegBits) | (uint32_t)i;
-    } else if (kind == SMLM_KEY_PTR) {
-      k = ((reinterpret_cast<const uint64_t*>(key)[i] >> 4) << kSegBits) | (uint32_t)i;
-    } else {
-      k = ((uint64_t)i << kSegBits) | (uint32_t)i;
-    }
-    K[i] = k;
+    if (kind != SMLM_KEY_NONE) bitonic_sort(lds_keys, N);
+    for (int i = tid; i < S; i += kPlanThreads) pv.sort_keys[i] = lds_keys[i];
+  } else {
+    for (int i = tid; i < N; i += kPlanThreads) pv.sort_keys[i] = i < S ? make_key(args.key, kind, i) : ~0ull;
+    __syncthreads();
+    if (kind != SMLM_KEY_NONE) bitonic_sort(pv.sort_keys, N);
   }
   __syncthreads();
-
-  if (kind != SMLM_KEY_NONE) {  // bitonic sort, ascending; ties impossible (segment index inside)
-    for (int size = 2; size <= N; size <<= 1) {
-      for (int stride = size >> 1; stride > 0; stride >>= 1) {
-        for (int i = tid; i < (N >> 1); i += kPlanThreads) {
-          const int lo = 2 * i - (i & (stride - 1));
-          const int hi = lo + stride;
-          const bool asc = (lo & size) == 0;
-          const uint64_t a = K[lo], b = K[hi];
-          if ((a > b) == asc) {
-            K[lo] = b;
-            K[hi] = a;
-          }
-        }
-        __syncthreads();
-      }
-    }
-  }
+  const uint64_t* K = pv.sort_keys;  // global from here on
 
   // Pass A: gathered-row position of every sorted segment, group heads.
   if (tid == 0) carry = 0;
@@ -166,38 +316,63 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanView pv,
     pv.grp_tile[NG] = (int)carry;
     pv.hdr[0] = (int)carry;
   }
+  __syncthreads();
+
+  // Pass C: tile blocks per group -> first block of each group.
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < NG; base += kPlanThreads) {
+    const int G = base + tid;
+    uint64_t nb = 0;
+    if (G < NG) nb = (uint64_t)((pv.grp_tile[G + 1] - pv.grp_tile[G] + kBlkTiles - 1) / kBlkTiles);
+    const uint64_t incl = block_scan_incl(nb, wave_tot) + carry;
+    if (G < NG) pv.grp_blk[G] = (int)(incl - nb);
+    __syncthreads();
+    if (tid == 0) carry += wave_tot[16];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    pv.grp_blk[NG] = (int)carry;
+    pv.hdr[4] = (int)carry;
+  }
 }
 
+struct PlanFillArgs {
+  PlanView pv;
+  const int32_t* s;
+  int S;
+};
+
 // One thread per tile slot: which row (and segment) sits there.
-__global__ __launch_bounds__(256) void plan_fill_kernel(PlanView pv, const int32_t* __restrict__ s,
-                                                        int S) {
+__global__ __launch_bounds__(256) void plan_fill_kernel(PlanFillArgs args) {
+  const PlanView pv = args.pv;
+  const int32_t* __restrict__ s = args.s;
+  const int S = args.S;
   const long slot = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int tile = (int)(slot / kTileRows), c = (int)(slot % kTileRows);
   if (tile >= pv.nt_max) return;
-  const int n_tiles = pv.hdr[0];
-  if (tile >= n_tiles) return;
   const int NG = pv.hdr[1];
+  if (slot < pv.hdr[4]) {  // the first n_blocks threads also write the tile-block table
+    const int b = (int)slot;
+    const int Gb = last_le(pv.grp_blk, NG, b);
+    const int tile0 = pv.grp_tile[Gb] + (b - pv.grp_blk[Gb]) * kBlkTiles;
+    const int left = pv.grp_tile[Gb + 1] - tile0;
+    pv.blk[b] = (tile0 << 3) | (left < kBlkTiles ? left : kBlkTiles);
+  }
+  if (tile >= pv.hdr[0]) return;
   // last group whose first tile is <= tile (empty groups share a first tile
   // with their successor, so "last" lands on the one that owns the tile)
-  int lo = 0, hi = NG;  // invariant: grp_tile[lo] <= tile < grp_tile[hi]
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (pv.grp_tile[mid] <= tile) lo = mid; else hi = mid;
-  }
-  const int G = lo;
+  const int G = last_le(pv.grp_tile, NG, tile);
   const int q = pv.grp_row[G] + (tile - pv.grp_tile[G]) * kTileRows + c;
   int row = -1, rseg = -1;
   if (q < pv.grp_row[G + 1]) {
-    int a = 0, b = S;  // invariant: rowpos[a] <= q < rowpos[b]
-    while (b - a > 1) {
-      const int mid = (a + b) >> 1;
-      if (pv.rowpos[mid] <= q) a = mid; else b = mid;
-    }
+    const int a = last_le(pv.rowpos, S, q);
     rseg = pv.sorted_seg[a];
     row = s[rseg] + (q - pv.rowpos[a]);
   }
   pv.tile_row[slot] = row;
   pv.tile_rseg[slot] = rseg;
+  if (c == 0) pv.tile_wid[tile] = (pv.hdr[3] == SMLM_KEY_I32) ? pv.grp_id[G] : pv.grp_seg[G];
 }
 
 }  // namespace smlm

@@ -129,7 +129,7 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
         kernel.smlm_lora_backward(
             grad_x, _ptr_table(da, dev), _ptr_table(db, dev), g, x_train, v_train,
             _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
-            part_ad, plan, lora_rank, part_scale)
+            plan, lora_rank, part_scale)
     else:
         for t in da + db:
             t.zero_()

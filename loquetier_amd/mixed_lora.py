@@ -106,18 +106,19 @@ def prepare_weight(weight: torch.Tensor, rank: int, dtype: torch.dtype, device, 
 class fused_add_lora(Function):
     """result <- result + scale_seg * (x A_seg^T) B_seg^T, in place, one call.
 
-    Arguments: (result, x, wa_table, wb_table, seg_adapter, seg_scale, plan,
-    lora_rank, train_len, train_partition, *weights).  Returns `result`.
+    Arguments: (result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
+    train_len, train_partition, *weights); the tables hold one address per
+    adapter and the plan is keyed by adapter id.  Returns `result`.
     Gradients: result -> passed through, x -> dX on train rows (zero elsewhere),
     each trainable weight -> its summed gradient (None when not training)."""
 
     @staticmethod
-    def forward(ctx: FunctionCtx, result, x, wa_table, wb_table, seg_adapter, seg_scale, plan,
-                lora_rank, train_len, train_partition, *weights):
+    def forward(ctx: FunctionCtx, result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
+                train_len, train_partition, *weights):
         need_v = len(weights) > 0 and train_len > 0
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
-        kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank,
-                                 seg_adapter=seg_adapter, seg_scale=seg_scale, beta=1.0, v_out=v)
+        kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
+                                 beta=1.0, v_out=v)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
@@ -137,7 +138,7 @@ class fused_add_lora(Function):
 
     @staticmethod
     def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
-        n_fixed = 10
+        n_fixed = 9
         if not ctx.has_v:
             return (grad_output, None) + (None,) * (n_fixed - 2) + (None,) * (2 * ctx.n_parts)
         x, v, *weight_list = ctx.saved_tensors
@@ -212,7 +213,7 @@ class MixedLoraLinear(nn.Module):
             result = result.to(self.dtype).contiguous()
             if not x.is_contiguous():
                 x = x.contiguous()
-            result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_adapter, seg_scale,
+            result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale,
                                           ctx.plan(self.device, x.size(0)), self.rank, blen.tlen,
                                           blen.train_partition, *weights)
             return result.to(torch_result_dtype)

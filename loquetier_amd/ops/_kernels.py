@@ -8,6 +8,7 @@ torch's current stream of that device.  Nothing here computes on the host.
 """
 from __future__ import annotations
 
+import ctypes as C
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -111,7 +112,8 @@ class SegmentPlan:
     per-problem table inside every kernel call,
     smlm_forward_cutlass.cuh:76-79)."""
 
-    def __init__(self, segment: torch.Tensor, seg_key: Optional[torch.Tensor], T: int):
+    def __init__(self, segment: torch.Tensor, seg_key: Optional[torch.Tensor], T: int,
+                 buf: Optional[torch.Tensor] = None):
         _check_input(segment, "segment")
         if segment.dtype != torch.int32 or segment.dim() != 1:
             raise RuntimeError("segment must be a 1D int32 tensor")
@@ -131,13 +133,22 @@ class SegmentPlan:
             _check_input(seg_key, "seg_key")
             if seg_key.dim() != 1 or seg_key.size(0) != self.S:
                 raise RuntimeError("seg_key must have one entry per segment")
+        self.kind = kind
         dev = segment.device
         nbytes = _lib.size_query("smlm_plan_size", self.T, self.S)
-        self.buf = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+        if buf is None:
+            buf = torch.empty(max(nbytes, 64), dtype=torch.uint8, device=dev)
+        elif buf.dtype != torch.uint8 or buf.numel() < nbytes or buf.device != dev:
+            raise RuntimeError(f"plan buffer must be a uint8 tensor of >= {nbytes} bytes on {dev}")
+        self.buf = buf
         with torch.cuda.device(dev):
             rc = _lib.load().smlm_plan_build(self.buf.data_ptr(), self.buf.numel(), segment.data_ptr(),
                                              _ptr(seg_key), kind, self.T, self.S, _stream(dev))
         _lib.check(rc, "smlm_plan_build")
+
+    @staticmethod
+    def nbytes(T: int, S: int) -> int:
+        return _lib.size_query("smlm_plan_size", int(T), int(S))
 
     def header(self) -> Tuple[int, int, int, int]:
         """(n_tiles, n_groups, rows covered, key kind used) -- synchronises; for tests."""
@@ -145,58 +156,117 @@ class SegmentPlan:
         return int(h[0]), int(h[1]), int(h[2]), int(h[3])
 
 
-def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_ptrs: torch.Tensor,
-                      plan: SegmentPlan, rank: int, seg_adapter: Optional[torch.Tensor] = None,
-                      seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
-                      v_out: Optional[torch.Tensor] = None) -> None:
-    """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call."""
-    for t, n in ((y, "y"), (x, "x"), (a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs")):
+def _check_table(t: torch.Tensor, plan: SegmentPlan, name: str) -> None:
+    _check_input(t, name)
+    if t.dtype != torch.int64 or t.dim() != 1:
+        raise RuntimeError(f"{name} must be a 1D int64 tensor of device addresses")
+    if plan.kind != _lib.SMLM_KEY_I32 and t.size(0) != plan.S:
+        raise RuntimeError(f"{name} needs one entry per segment unless the plan is keyed by adapter id")
+
+
+def _check_scale(seg_scale: Optional[torch.Tensor], plan: SegmentPlan) -> None:
+    if seg_scale is not None and (seg_scale.dtype != torch.float32 or seg_scale.dim() != 1
+                                  or seg_scale.size(0) != plan.S or not seg_scale.is_cuda):
+        raise RuntimeError("seg_scale must be a device float32 tensor with one entry per segment")
+
+
+def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, plan: SegmentPlan,
+                      is_row_major: bool = False, seg_scale: Optional[torch.Tensor] = None,
+                      beta: float = 0.0) -> None:
+    """Grouped GEMM over a prebuilt plan: y[seg] = beta*y[seg] + scale*x[seg] @ W_seg.
+    w_ptrs is indexed by adapter id when the plan was built from int32 adapter ids,
+    by segment otherwise."""
+    for t, n in ((y, "y"), (x, "x")):
         _check_input(t, n)
     _check_dim(2, y, "y")
     _check_dim(2, x, "x")
+    _check_table(w_ptrs, plan, "w_ptrs")
+    _check_scale(seg_scale, plan)
     if y.dtype != x.dtype or y.size(0) != x.size(0) or x.size(0) != plan.T:
-        raise RuntimeError("x [T,h_in] and y [T,h_out] must share dtype and T with the plan")
-    if a_ptrs.dtype != torch.int64 or b_ptrs.dtype != torch.int64:
-        raise RuntimeError("pointer tables must be int64")
-    if seg_adapter is None and (a_ptrs.size(0) != plan.S or b_ptrs.size(0) != plan.S):
-        raise RuntimeError("per-segment pointer tables must have one entry per segment")
-    if seg_adapter is not None and (seg_adapter.dtype != torch.int32 or seg_adapter.size(0) != plan.S
-                                    or not seg_adapter.is_cuda):
-        raise RuntimeError("seg_adapter must be a device int32 tensor with one entry per segment")
-    if seg_scale is not None and (seg_scale.dtype != torch.float32 or seg_scale.size(0) != plan.S
-                                  or not seg_scale.is_cuda):
-        raise RuntimeError("seg_scale must be a device float32 tensor with one entry per segment")
-    if v_out is not None and (v_out.dtype != x.dtype or tuple(v_out.shape) != (x.size(0), rank)
-                              or not v_out.is_contiguous()):
-        raise RuntimeError("v_out must be a contiguous [T, rank] tensor of x's dtype")
+        raise RuntimeError("x [T,d_in] and y [T,d_out] must share dtype and T with the plan")
     code = _dtype_code(x)
-    T, h_in, h_out = x.size(0), x.size(1), y.size(1)
+    T, d_in, d_out = x.size(0), x.size(1), y.size(1)
+    w_ld = d_out if is_row_major else d_in
     dev = x.device
     with torch.cuda.device(dev):
-        need = _lib.size_query("smlm_lora_fwd_workspace_size", T, plan.S, h_in, h_out, rank)
+        need = _lib.size_query("smlm_gemm_planned_workspace_size", T, d_in, d_out)
         ws = _workspace(dev, need)
-        rc = _lib.load().smlm_lora_fwd(y.data_ptr(), x.data_ptr(), _ptr(v_out), a_ptrs.data_ptr(),
-                                       b_ptrs.data_ptr(), _ptr(seg_adapter), plan.segment.data_ptr(),
-                                       plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), T, plan.S, h_in,
-                                       h_out, rank, code, float(beta), _ptr(seg_scale), _stream(dev))
+        rc = _lib.load().smlm_gemm_planned(y.data_ptr(), x.data_ptr(), w_ptrs.data_ptr(),
+                                           plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), T, plan.S,
+                                           d_in, d_out, w_ld, int(bool(is_row_major)), code,
+                                           float(beta), _ptr(seg_scale), _stream(dev))
+    _lib.check(rc, "smlm_gemm_planned")
+
+
+def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_ptrs: torch.Tensor,
+                      plan: SegmentPlan, rank: int, seg_scale: Optional[torch.Tensor] = None,
+                      beta: float = 0.0, v_out: Optional[torch.Tensor] = None) -> None:
+    """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call (two launches).
+    a_ptrs / b_ptrs are indexed by adapter id when the plan was built from int32
+    adapter ids, by segment otherwise."""
+    smlm_lora_forward_multi([y], [x], [a_ptrs], [b_ptrs], plan, rank, seg_scale=seg_scale, beta=beta,
+                            v_out=None if v_out is None else [v_out])
+
+
+def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
+                            seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
+                            v_out=None) -> None:
+    """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
+    in two launches.  Lists of equal length; entries of xs may be the same tensor."""
+    n = len(ys)
+    if not (1 <= n <= 8) or len(xs) != n or len(a_ptrs) != n or len(b_ptrs) != n or \
+            (v_out is not None and len(v_out) != n):
+        raise RuntimeError("between 1 and 8 projections, all lists of one length")
+    _check_scale(seg_scale, plan)
+    for i in range(n):
+        _check_input(ys[i], "y")
+        _check_input(xs[i], "x")
+        _check_dim(2, ys[i], "y")
+        _check_dim(2, xs[i], "x")
+        _check_table(a_ptrs[i], plan, "a_ptrs")
+        _check_table(b_ptrs[i], plan, "b_ptrs")
+        if ys[i].dtype != xs[0].dtype or xs[i].dtype != xs[0].dtype or ys[i].size(0) != plan.T \
+                or xs[i].size(0) != plan.T or ys[i].device != xs[0].device:
+            raise RuntimeError("x [T,h_in] and y [T,h_out] must share dtype, device and T with the plan")
+        if v_out is not None and v_out[i] is not None:
+            vo = v_out[i]
+            if vo.dtype != xs[0].dtype or tuple(vo.shape) != (plan.T, rank) or not vo.is_contiguous():
+                raise RuntimeError("v_out must be a contiguous [T, rank] tensor of x's dtype")
+    code = _dtype_code(xs[0])
+    dev = xs[0].device
+    VP, CI = C.c_void_p * n, C.c_int * n
+    h_in = CI(*[x.size(1) for x in xs])
+    h_out = CI(*[y.size(1) for y in ys])
+    vo_arr = None if v_out is None else VP(*[_ptr(t) for t in v_out])
+    with torch.cuda.device(dev):
+        need = C.c_size_t(0)
+        _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(n, plan.T, h_in, rank, C.byref(need)),
+                   "smlm_lora_fwd_multi_workspace_size")
+        ws = _workspace(dev, need.value)
+        rc = _lib.load().smlm_lora_fwd_multi(
+            n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
+            VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]), h_in, h_out,
+            plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
+            _ptr(seg_scale), _stream(dev))
     _lib.check(rc, "smlm_lora_forward")
 
 
 def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.Tensor,
                        dy: torch.Tensor, x: torch.Tensor, v: Optional[torch.Tensor],
-                       a_ptrs: torch.Tensor, b_ptrs: torch.Tensor, part_adapter: torch.Tensor,
-                       plan: SegmentPlan, rank: int, part_scale: Optional[torch.Tensor] = None) -> None:
-    """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h)."""
+                       a_ptrs: torch.Tensor, b_ptrs: torch.Tensor, plan: SegmentPlan, rank: int,
+                       part_scale: Optional[torch.Tensor] = None) -> None:
+    """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
+    `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows)."""
     for t, n in ((dx, "dx"), (dy, "dy"), (x, "x"), (da_ptrs, "da_ptrs"), (db_ptrs, "db_ptrs"),
-                 (a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs"), (part_adapter, "part_adapter")):
+                 (a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs")):
         _check_input(t, n)
+    if plan.kind != _lib.SMLM_KEY_I32:
+        raise RuntimeError("the backward plan must be built from int32 adapter ids")
     n_rows = plan.T
     if dy.size(0) < n_rows or x.size(0) < n_rows or dx.size(0) < n_rows:
         raise RuntimeError("dy, x and dx need at least plan.T rows")
     if dx.dtype != dy.dtype or x.dtype != dy.dtype or (v is not None and v.dtype != dy.dtype):
         raise RuntimeError("dx, dy, x, v must share one dtype")
-    if part_adapter.dtype != torch.int32 or part_adapter.size(0) != plan.S:
-        raise RuntimeError("part_adapter must be int32 with one entry per partition")
     NA = a_ptrs.size(0)
     if b_ptrs.size(0) != NA or da_ptrs.size(0) != NA or db_ptrs.size(0) != NA:
         raise RuntimeError("pointer tables must all have one entry per adapter")
@@ -210,8 +280,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
         ws = _workspace(dev, need)
         rc = _lib.load().smlm_lora_bwd(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
                                        dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
-                                       b_ptrs.data_ptr(), part_adapter.data_ptr(),
-                                       plan.segment.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
+                                       b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
                                        ws.numel(), n_rows, plan.S, NA, h_in, h_out, rank, code,
                                        _ptr(part_scale), _stream(dev))
     _lib.check(rc, "smlm_lora_backward")

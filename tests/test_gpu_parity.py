@@ -143,7 +143,7 @@ def test_fused_forward_accumulate(K, oracle, gpu_device, case, dt):
     ids_t = torch.tensor(ids, dtype=torch.int32, device=d)
     plan = K.SegmentPlan(s, ids_t, T)
     v = torch.zeros(T, r, dtype=TDT[dt], device=d)
-    K.smlm_lora_forward(yd, xd, ptrs(Ad, d), ptrs(Bd, d), plan, r, seg_adapter=ids_t,
+    K.smlm_lora_forward(yd, xd, ptrs(Ad, d), ptrs(Bd, d), plan, r,
                         seg_scale=torch.from_numpy(scale).to(d), beta=1.0, v_out=v)
     yo, vo = oracle.lora_fused(base, x, [A[i] for i in ids], [B[i] for i in ids], seg, scale, 1.0, dt)
     covered = np.zeros(T, bool)
@@ -186,7 +186,9 @@ def test_routing_bit_exact_small_integers(K, oracle, gpu_device, dt):
         plan = K.SegmentPlan(s, key, T)
         y = torch.zeros(T, h_out, dtype=TDT[dt], device=d)
         v = torch.zeros(T, r, dtype=TDT[dt], device=d)
-        K.smlm_lora_forward(y, xd, ptrs(Ad, d), ptrs(Bd, d), plan, r, seg_adapter=ids_t, v_out=v)
+        tabs = (ptrs(Ad, d), ptrs(Bd, d)) if key is ids_t else \
+            (ptrs([Ad[i] for i in ids], d), ptrs([Bd[i] for i in ids], d))
+        K.smlm_lora_forward(y, xd, tabs[0], tabs[1], plan, r, v_out=v)
         assert np.array_equal(to_np(v), vo)
         assert np.array_equal(to_np(y), yo)
 
@@ -208,7 +210,10 @@ def test_resegmenting_changes_no_bit(K, oracle, gpu_device, dt):
         ids_t = torch.tensor(ids, dtype=torch.int32, device=d)
         plan = K.SegmentPlan(s, ids_t if key_kind else None, T)
         y = torch.zeros(T, h_out, dtype=TDT[dt], device=d)
-        K.smlm_lora_forward(y, xd, ptrs(Ad, d), ptrs(Bd, d), plan, r, seg_adapter=ids_t)
+        if key_kind:
+            K.smlm_lora_forward(y, xd, ptrs(Ad, d), ptrs(Bd, d), plan, r)
+        else:
+            K.smlm_lora_forward(y, xd, ptrs([Ad[i] for i in ids], d), ptrs([Bd[i] for i in ids], d), plan, r)
         return y
 
     per_row = run(list(range(T + 1)), row_ad.tolist(), 1)                  # one segment per row
@@ -311,7 +316,7 @@ def _bwd_exact(K, oracle, d, dt, x, A, B, g, tp, part_ad, r, scale=None):
     dx = torch.empty(n_rows, x.shape[1], dtype=TDT[dt], device=d)
     pi = torch.tensor(tp, dtype=torch.int32, device=d)
     pa = torch.tensor(part_ad, dtype=torch.int32, device=d)
-    K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, None, ptrs(Ad, d), ptrs(Bd, d), pa,
+    K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, None, ptrs(Ad, d), ptrs(Bd, d),
                          K.SegmentPlan(pi, pa, n_rows), r)
     gx, ga, gb = oracle.add_lora_backward(g, x, A, B, tp, part_ad, dt)
     covered = np.zeros(n_rows, bool)
@@ -332,7 +337,7 @@ def _fwd_exact(K, oracle, d, dt, x, A, B, seg, ids, r, base, scale_val=2.0):
     v = torch.zeros(T, r, dtype=TDT[dt], device=d)
     sc = torch.full((len(ids),), scale_val, device=d)
     K.smlm_lora_forward(yd, xd, ptrs(Ad, d), ptrs(Bd, d), K.SegmentPlan(s, ids_t, T), r,
-                        seg_adapter=ids_t, seg_scale=sc, beta=1.0, v_out=v)
+                        seg_scale=sc, beta=1.0, v_out=v)
     yo, vo = oracle.lora_fused(base, x, [A[i] for i in ids], [B[i] for i in ids], seg,
                                [scale_val] * len(ids), 1.0, dt)
     assert np.array_equal(to_np(v), vo), "v differs"
@@ -350,10 +355,73 @@ def test_forward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
 
 
+def _ragged_segments(rng, T, S):
+    cuts = np.sort(rng.choice(np.arange(1, T), S - 1, replace=False))
+    return [0] + cuts.tolist() + [T]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [
+    # T, S, NA, h_in, h_out, r: tile blocks of four (T >= 1024), ragged groups
+    (1500, 40, 7, 512, 768, 32),
+    (2048, 300, 5, 256, 264, 16),
+    (1100, 3, 3, 128, 1024, 64),
+    # more than 1024 segments: two-launch plan with the sort in LDS
+    (3000, 1500, 37, 128, 160, 8),
+    # more than 4096 segments: the sort runs in global memory
+    (5000, 5000, 61, 64, 128, 8),
+], ids=["blocks-ragged", "blocks-many-segs", "blocks-long", "plan-two-launch", "plan-global-sort"])
+def test_forward_dyadic_bit_exact_larger(K, oracle, gpu_device, shape, dt):
+    T, S, NA, h_in, h_out, r = shape
+    rng = np.random.default_rng(31)
+    seg = list(range(T + 1)) if S == T else _ragged_segments(rng, T, S)
+    ids = rng.integers(0, NA, S).tolist()
+    x, A, B = make_case(oracle, 202, T, seg, ids, NA, h_in, h_out, r, dt, dy=True)
+    base = dyadic(rng, (T, h_out), 16, 8)
+    _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
+
+
+def test_multi_projection_equals_single_calls(K, oracle, gpu_device):
+    """q/k/v/o-style batched launch: bit-identical to one call per projection,
+    with different widths per projection and a shared x for three of them."""
+    d, dt = gpu_device, "bf16"
+    T, r, NA = 300, 16, 6
+    rng = np.random.default_rng(32)
+    seg = _ragged_segments(rng, T, 25)
+    ids = rng.integers(0, NA, 25).tolist()
+    dims = [(512, 512), (512, 128), (512, 128), (384, 640)]
+    s = torch.tensor(seg, dtype=torch.int32, device=d)
+    ids_t = torch.tensor(ids, dtype=torch.int32, device=d)
+    plan = K.SegmentPlan(s, ids_t, T)
+    sc = torch.full((25,), 0.5, device=d)
+    xs_np = {512: oracle.round_to(rng.standard_normal((T, 512)), dt),
+             384: oracle.round_to(rng.standard_normal((T, 384)), dt)}
+    xs_dev = {k: dev_t(v, dt, d) for k, v in xs_np.items()}
+    projs = []
+    for hi, ho in dims:
+        A = [dev_t(oracle.round_to(rng.standard_normal((r, hi)) / np.sqrt(hi), dt), dt, d) for _ in range(NA)]
+        B = [dev_t(oracle.round_to(rng.standard_normal((ho, r)) / 4, dt), dt, d) for _ in range(NA)]
+        y0 = dev_t(oracle.round_to(rng.standard_normal((T, ho)), dt), dt, d)
+        projs.append(dict(x=xs_dev[hi], A=A, B=B, a=ptrs(A, d), b=ptrs(B, d), y0=y0))
+    single, single_v = [], []
+    for p in projs:
+        y, v = p["y0"].clone(), torch.zeros(T, r, dtype=TDT[dt], device=d)
+        K.smlm_lora_forward(y, p["x"], p["a"], p["b"], plan, r, seg_scale=sc, beta=1.0, v_out=v)
+        single.append(y)
+        single_v.append(v)
+    ys = [p["y0"].clone() for p in projs]
+    vs = [torch.zeros(T, r, dtype=TDT[dt], device=d) for _ in projs]
+    K.smlm_lora_forward_multi(ys, [p["x"] for p in projs], [p["a"] for p in projs],
+                              [p["b"] for p in projs], plan, r, seg_scale=sc, beta=1.0, v_out=vs)
+    for a, b in zip(single + single_v, ys + vs):
+        assert torch.equal(a, b)
+
+
 # --------------------------------------------------------------- backward ---
 BWD_CASES = [
     # name, tp, part_ad, NA, n_infer_rows, h_in, h_out, r
     ("two-parts", [0, 5, 12], [0, 1], 2, 3, 64, 96, 8),
+    ("blocks", [0, 500, 520, 1300], [2, 0, 2], 3, 7, 256, 192, 16),
     ("shared-adapter", [0, 40, 70, 100], [1, 0, 1], 2, 5, 128, 256, 16),
     ("empty-part", [0, 17, 17, 50], [0, 1, 2], 3, 0, 256, 128, 32),
     ("rank64", [0, 33, 90], [0, 1], 2, 4, 192, 320, 64),
@@ -385,7 +453,7 @@ def test_backward_against_oracle(K, oracle, gpu_device, case, dt, with_v):
         _, vo = oracle.add_lora_forward(x[:n_rows], [A[a] for a in part_ad], [B[a] for a in part_ad],
                                         tp, h_out, dt)
         v = dev_t(vo, dt, d)
-    K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, v, ptrs(Ad, d), ptrs(Bd, d), pa, plan, r)
+    K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, v, ptrs(Ad, d), ptrs(Bd, d), plan, r)
     gx, ga, gb = oracle.add_lora_backward(g[:n_rows], x[:n_rows], A, B, tp, part_ad, dt)
     # bf16: dV (|dV| up to ~8) is rounded to 8 bits inside the op; one element
     # rounding the other way moves a dX row by 2^-8 |dV| |A| ~ 4e-3
@@ -421,7 +489,7 @@ def test_backward_is_deterministic(K, oracle, gpu_device):
         dx = torch.empty(tp[-1], h_in, dtype=TDT[dt], device=d)
         pi = torch.tensor(tp, dtype=torch.int32, device=d)
         pa = torch.tensor(part_ad, dtype=torch.int32, device=d)
-        K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, None, ptrs(Ad, d), ptrs(Bd, d), pa,
+        K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, None, ptrs(Ad, d), ptrs(Bd, d),
                              K.SegmentPlan(pi, pa, tp[-1]), r)
         outs.append([dx] + dA + dB)
     for o in outs[1:]:
@@ -542,12 +610,11 @@ def _permutation_invariance(K, d, dt, x, A, B, seg, ids, r, y):
     y2 = torch.zeros_like(y)
     s2 = torch.tensor(seg2, dtype=torch.int32, device=d)
     ids2 = torch.tensor([ids[i] for i in order], dtype=torch.int32, device=d)
-    K.smlm_lora_forward(y2, xd[perm].contiguous(), ptrs(Ad, d), ptrs(Bd, d), K.SegmentPlan(s2, ids2, T), r,
-                        seg_adapter=ids2)
+    K.smlm_lora_forward(y2, xd[perm].contiguous(), ptrs(Ad, d), ptrs(Bd, d), K.SegmentPlan(s2, ids2, T), r)
     y1 = torch.zeros_like(y)
     s1 = torch.tensor(seg, dtype=torch.int32, device=d)
     ids1 = torch.tensor(ids, dtype=torch.int32, device=d)
-    K.smlm_lora_forward(y1, xd, ptrs(Ad, d), ptrs(Bd, d), K.SegmentPlan(s1, ids1, T), r, seg_adapter=ids1)
+    K.smlm_lora_forward(y1, xd, ptrs(Ad, d), ptrs(Bd, d), K.SegmentPlan(s1, ids1, T), r)
     assert torch.equal(y2, y1[perm])
 
 
@@ -635,8 +702,7 @@ def test_full_size_gaussian_tolerance(K, gpu_device, cfg):
     ids_t = torch.tensor(ids, dtype=torch.int32, device=d)
     y = torch.zeros(T, 4096, dtype=dt, device=d)
     v = torch.zeros(T, r, dtype=dt, device=d)
-    K.smlm_lora_forward(y, x, ptrs(A, d), ptrs(B, d), K.SegmentPlan(s, ids_t, T), r, seg_adapter=ids_t,
-                        v_out=v)
+    K.smlm_lora_forward(y, x, ptrs(A, d), ptrs(B, d), K.SegmentPlan(s, ids_t, T), r, v_out=v)
     for i in range(len(ids)):
         a, b = seg[i], seg[i + 1]
         v_ref = x[a:b].float() @ A[ids[i]].float().t()
