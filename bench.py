@@ -102,6 +102,7 @@ def main():
     ap.add_argument("--config", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
+    ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; every box has one MI355X and no collective, "
@@ -176,104 +177,95 @@ def main():
         part_ad = torch.tensor([train.index(a) for a in w["ids"][:P]], dtype=torch.int32, device=dev)
         part_scale = torch.full((P,), 2.0, device=dev)
 
-    def step(st):
-        plan = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
+    def fwd(st, stages=3):
         pr = st["proj"]
         K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
-                                  [d["b_tab"] for d in pr], plan, r, seg_scale=scale_t, beta=1.0,
-                                  v_out=[d["v"] for d in pr] if P else None)
+                                  [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
+                                  v_out=[d["v"] for d in pr] if P else None, stages=stages)
+
+    def step(st):
+        st["plan"] = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
+        fwd(st)
         if P:
             bplan = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
             for d in st["proj"]:
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
                                      d["ta_tab"], d["tb_tab"], bplan, r, part_scale)
 
-    # eager once on the capture stream (sizes its workspace outside any capture), then one
-    # graph per buffer set
+    # eager once on the capture stream (sizes its workspace outside any capture)
     cap_stream = torch.cuda.Stream()
     with torch.cuda.stream(cap_stream):
         for st in sets:
             step(st)
     torch.cuda.synchronize()
-    graphs = []
-    for st in sets:
+
+    def capture(fn):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, stream=cap_stream):
-            step(st)
-        graphs.append(g)
+            fn()
+        return g
+
+    def timed(graph_runs):
+        """graph_runs: list of (graph, times).  Returns elapsed ms between HIP events
+        recorded on the stream the graphs are launched on."""
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for g, n in graph_runs:
+            for _ in range(n):
+                g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b)
+
+    # One graph holds one step on each of the R buffer sets (launching a graph costs the host
+    # tens of microseconds, more than a decode step takes on the GPU); a second graph holds the
+    # K mod R steps left over, so that exactly K steps are timed.
+    def steps_graph(n):
+        return capture(lambda: [step(sets[i % R]) for i in range(n)])
+
+    g_round = steps_graph(R)
+    g_rest = steps_graph(args.steps % R) if args.steps % R else None
+    g_warm = steps_graph(args.warmup % R) if args.warmup % R else None
     torch.cuda.synchronize()
 
-    def run(n):
-        for i in range(n):
-            graphs[i % R].replay()
-
-    run(args.warmup)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    timed([(g_round, args.warmup // R)] + ([(g_warm, 1)] if g_warm else []))
     t0 = time.perf_counter()
-    e0.record()
-    run(args.steps)
-    e1.record()
-    torch.cuda.synchronize()
+    ms = timed([(g_round, args.steps // R)] + ([(g_rest, 1)] if g_rest else []))
     wall_ms = (time.perf_counter() - t0) * 1e3
-    ms_per_step = e0.elapsed_time(e1) / args.steps
+    ms_per_step = ms / args.steps
     tokens_per_s = T / (ms_per_step * 1e-3)
     step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
 
-    # ---- dominant kernel alone: the expand kernel of one projection (y += s * v B^T), launched
-    # back to back from a graph over the rotating buffer sets, timed with HIP events on its stream
-    _, hi0, ho0 = max(w["proj"], key=lambda p: p[2])
-    pidx = [p[2] for p in w["proj"]].index(ho0)
-    v16 = [torch.randn(T, r, generator=gen).to(dev).to(tdt) for _ in range(R)]
-    plans = [K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"]) for st in sets]
-    reps = max(4, 48 // R)
+    if args.step_only:
+        print(json.dumps({"config": args.config, "ms_per_step": round(ms_per_step, 5),
+                          "step_hbm_gbps": round(step_gbps, 1)}), flush=True)
+        return
 
-    def expand_only():
-        for _ in range(reps):
-            for i, st in enumerate(sets):
-                d = st["proj"][pidx]
-                K.smlm_gemm_planned(d["y"], v16[i], d["b_tab"], plans[i], seg_scale=scale_t, beta=1.0)
-
-    def shrink_only():
-        for _ in range(reps):
-            for i, st in enumerate(sets):
-                d = st["proj"][pidx]
-                K.smlm_gemm_planned(v16[i], d["x"], d["a_tab"], plans[i])
-
-    def time_graph(fn, launches):
-        with torch.cuda.stream(cap_stream):
-            fn()
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=cap_stream):
-            fn()
-        for _ in range(3):
-            g.replay()
-        torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        n_rep = 10
-        a.record()
-        for _ in range(n_rep):
-            g.replay()
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) * 1e3 / (n_rep * launches)  # us per launch
-
-    n_act = len(set(w["ids"]))
+    # ---- dominant kernel alone: the expand launch of the step (all projections of the batch,
+    # y += s * v B^T), launched back to back from a graph over the rotating buffer sets and timed
+    # with HIP events on its stream.  The shrink launch is timed the same way.
+    reps = max(2, 48 // R)
+    ranks = w.get("true_ranks")
     rsum = sum((ranks[a % 4] if ranks else r) for a in set(w["ids"]))
-    expand_us = time_graph(expand_only, reps * R)
-    expand_bytes = T * ho0 * 2 * 2 + rsum * ho0 * 2 + T * r * 2
-    shrink_us = time_graph(shrink_only, reps * R)
-    shrink_bytes = T * hi0 * 2 + rsum * hi0 * 2 + T * r * 2
+
+    def stage_us(stages):
+        g = capture(lambda: [fwd(st, stages) for _ in range(reps) for st in sets])
+        timed([(g, 2)])
+        return timed([(g, 10)]) * 1e3 / (10 * reps * R)  # us per launch
+
+    expand_us = stage_us(2)
+    shrink_us = stage_us(1)
+    expand_bytes = sum(T * ho * 2 * 2 + rsum * ho * 2 + T * r * 2 for _, hi, ho in w["proj"])
+    shrink_bytes = sum(T * hi * 2 + rsum * hi * 2 + T * r * 2 for _, hi, ho in w["proj"])
     traffic = None
     tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get(args.config, {}).get("expand_bytes_per_launch")
     achieved = expand_bytes / (expand_us * 1e-6) / 1e9
-    roofline = dict(kernel="expand_kernel", bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
-                    unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
-                    us_per_launch=round(expand_us, 3), algorithmic_bytes=expand_bytes,
-                    projection=f"{hi0}->{ho0}")
+    roofline = dict(kernel="expand kernel, one launch for all projections of the step", bound="hbm",
+                    achieved=round(achieved, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
+                    us_per_launch=round(expand_us, 3), algorithmic_bytes=expand_bytes)
 
     # ---- CPU baseline: per-segment torch matmuls on the host cores (bounded sample)
     cpu = None
@@ -318,9 +310,10 @@ def main():
         "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
         "roofline": roofline,
-        "kernels": {"shrink_us": round(shrink_us, 3),
+        "kernels": {"shrink_us": round(shrink_us, 3), "shrink_bytes": shrink_bytes,
                     "shrink_gbps": round(shrink_bytes / (shrink_us * 1e-6) / 1e9, 1),
-                    "expand_us": round(expand_us, 3), "expand_gbps": round(achieved, 1)},
+                    "expand_us": round(expand_us, 3), "expand_bytes": expand_bytes,
+                    "expand_gbps": round(achieved, 1)},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

@@ -46,6 +46,10 @@ extern "C" {
 #define SMLM_KEY_I32 1  /* int32 adapter id per segment                      */
 #define SMLM_KEY_PTR 2  /* 64-bit weight address per segment                 */
 
+/* stages of the fused forward (smlm_lora_fwd_multi) */
+#define SMLM_STAGE_SHRINK 1 /* v = x A^T, left in the workspace                */
+#define SMLM_STAGE_EXPAND 2 /* y = beta*y + scale * v B^T from that workspace  */
+
 #define SMLM_OK 0
 #define SMLM_ERR_ARG (-1)       /* null pointer, negative size, bad enum      */
 #define SMLM_ERR_DTYPE (-2)     /* "No suitable kernel." (loquetier_ops.cc:318) */
@@ -139,8 +143,12 @@ SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* cons
  * rank and the segment routing, and in the decode regime a launch costs as much
  * as the data movement of one projection.  y, x, v_out, a_ptrs, b_ptrs, h_in,
  * h_out are HOST arrays of n_proj entries (v_out may be NULL or hold NULLs);
- * projections may differ in h_in / h_out.  No counterpart in the reference,
- * which calls its kernel once per linear layer (mixed_lora.py:198-205).
+ * projections may differ in h_in / h_out.  `stages` is SMLM_STAGE_SHRINK |
+ * SMLM_STAGE_EXPAND for the whole forward; a caller may also issue the two
+ * stages as separate calls with the same arguments and workspace (the expand
+ * stage reads what the shrink stage left there).  No counterpart in the
+ * reference, which calls its kernel once per linear layer
+ * (mixed_lora.py:198-205).
  */
 SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_in, int r,
                                                 size_t* bytes);
@@ -149,7 +157,7 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
                                  const void* const* const* b_ptrs, const int* h_in,
                                  const int* h_out, const void* plan, void* workspace,
                                  size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
-                                 const float* seg_scale, void* stream);
+                                 const float* seg_scale, int stages, void* stream);
 
 /*
  * LoRA backward for fine-tuning rows.  Replaces add_lora.backward

@@ -9,11 +9,13 @@ import ctypes as C
 import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, "lib", "libsmlm_hip.so")
+# SMLM_HIP_LIBRARY selects another build of the same library (e.g. one made with -DSMLM_TUNING)
+LIB_PATH = os.environ.get("SMLM_HIP_LIBRARY") or os.path.join(_PKG_DIR, "lib", "libsmlm_hip.so")
 
 SMLM_DTYPE_F16, SMLM_DTYPE_BF16 = 0, 1
 SMLM_KEY_NONE, SMLM_KEY_I32, SMLM_KEY_PTR = 0, 1, 2
 SMLM_ERR_DTYPE = -2
+SMLM_STAGE_SHRINK, SMLM_STAGE_EXPAND = 1, 2
 
 _vp, _i, _sz, _f = C.c_void_p, C.c_int, C.c_size_t, C.c_float
 _psz = C.POINTER(C.c_size_t)
@@ -35,7 +37,7 @@ SIGNATURES = {
     "smlm_lora_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_lora_fwd_multi_workspace_size": (_i, [_i, _i, _pi, _i, _psz]),
     "smlm_lora_fwd_multi": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _pi, _pi, _vp, _vp, _sz, _i, _i, _i,
-                                 _i, _f, _vp, _vp]),
+                                 _i, _f, _vp, _i, _vp]),
     "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
     "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
                            _i, _vp, _vp]),

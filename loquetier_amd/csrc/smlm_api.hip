@@ -3,6 +3,8 @@
 // synchronisation, no state.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "smlm.h"
 #include "smlm_backward.hpp"
 #include "smlm_common.hpp"
@@ -32,39 +34,71 @@ int launch(void (*kernel)(A), dim3 grid, dim3 block, hipStream_t st, const A& a)
 
 // ---- launch shapes: functions of (T, d_in, d_out) only, never of the
 // segmentation, so re-segmenting a batch cannot change a bit of any row. ----
-inline int tiles_per_wave(int T) { return T >= 1024 ? kBlkTiles : 1; }
+// Tuning overrides (only in builds with -DSMLM_TUNING): SMLM_TUNE_<NAME>=value.
+inline int tune(const char* name, int dflt) {
+#ifdef SMLM_TUNING
+  const char* e = getenv(name);
+  if (e && *e) return atoi(e);
+#else
+  (void)name;
+#endif
+  return dflt;
+}
+
+inline int tiles_per_wave(int T) { return tune("SMLM_TUNE_MT", T >= 1024 ? kBlkTiles : 1); }
 
 // upper bound of the number of work units along the tile axis
-inline int tile_units(int T, int S, int mt) {
+inline int tile_units_max(int T, int S, int mt) {
   const int nt_max = plan_nt_max(T, S);
   return mt == 1 ? nt_max : nt_max / kBlkTiles + S + 2;
 }
 
+// persistent 1-D grid: a multiple of the XCD count, no larger than the work bound
+constexpr int kMaxGrid = 2048;
+inline dim3 work_grid(long bound) {
+  const long cap = tune("SMLM_TUNE_GRID", kMaxGrid);
+  long g = bound < cap ? bound : cap;
+  g = (g + kNumXcd - 1) / kNumXcd * kNumXcd;
+  return dim3((unsigned)g);
+}
+
 struct ShrinkCfg {
-  int NB, U, MT, ksplit, k_per_wave, zblocks;
+  int NB, U, MT, NW, ksplit, k_per_wave, zblocks;
 };
 
-ShrinkCfg shrink_cfg(int T, int d_in, int d_out) {
+// waves per shrink workgroup, one choice for all projections of a launch: small
+// batches whose every projection has a long enough k use sixteen waves that
+// cover all of k, so nothing is left to fold afterwards
+int shrink_waves(int T, int nproj, const int* d_in, int d_out) {
+  const int kq = 32 * (d_out > 32 ? 4 : 8);  // k per wave and load batch of the sixteen-wave kernels
+  bool all_long = tiles_per_wave(T) == 1;
+  for (int i = 0; i < nproj; ++i) all_long = all_long && d_in[i] >= 16 * kq;
+  return tune("SMLM_TUNE_NW", all_long ? 16 : kFwdWaves);
+}
+
+ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   ShrinkCfg c;
   c.zblocks = ceil_div(d_out, 64);
   const int cols = d_out >= 64 ? 64 : d_out;
   c.NB = cols <= 16 ? 1 : (cols <= 32 ? 2 : 4);
-  c.U = c.NB == 4 ? 2 : 4;
+  c.U = (c.NB == 4 ? 2 : 4) * (nw == 16 ? 2 : 1);  // one batch of loads covers a sixteenth of k
   c.MT = tiles_per_wave(T);
   const int kq = 32 * c.U;
+  c.NW = nw;
   const int units = ceil_div(T > 0 ? T : 1, kTileRows * c.MT);
-  const int want = ceil_div(1024, units);
-  int max_split = d_in / (kFwdWaves * kq);
+  const int want = c.NW == 16 ? 1 : ceil_div(1024, units);
+  int max_split = d_in / (c.NW * kq);
   if (max_split < 1) max_split = 1;
   if (max_split > 16) max_split = 16;
   const int ks = want < 1 ? 1 : (want > max_split ? max_split : want);
-  c.k_per_wave = round_up(ceil_div(d_in, kFwdWaves * ks), kq);
-  c.ksplit = ceil_div(d_in, kFwdWaves * c.k_per_wave);
+  c.k_per_wave = round_up(ceil_div(d_in, c.NW * ks), kq);
+  c.ksplit = ceil_div(d_in, c.NW * c.k_per_wave);
   return c;
 }
 
 int expand_nq(int T, int d_out) {
-  const int units = ceil_div(T > 0 ? T : 1, kTileRows * tiles_per_wave(T));
+  if (tiles_per_wave(T) > 1) return 4;  // block kernel: a 128-column chunk per workgroup
+  const int units = ceil_div(T > 0 ? T : 1, kTileRows);
   return ((long)units * ceil_div(d_out, 512) >= 512) ? 4 : 2;
 }
 
@@ -72,62 +106,77 @@ TileArgs tile_args(const PlanView& pv) {
   return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
 }
 
-template <int DT, int MT, bool RM>
+template <int DT, int MT, int NW, bool RM>
 int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
-  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, MT, RM>, grid, dim3(kFwdThreads), st, a);
-  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, MT, RM>, grid, dim3(kFwdThreads), st, a);
-  return launch(shrink_kernel<DT, 4, 2, MT, RM>, grid, dim3(kFwdThreads), st, a);
+  const dim3 block(NW * kWaveSize);
+  constexpr int UF = NW == 16 ? 2 : 1;  // must match shrink_cfg
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4 * UF, MT, NW, RM>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4 * UF, MT, NW, RM>, grid, block, st, a);
+  return launch(shrink_kernel<DT, 4, 2 * UF, MT, NW, RM>, grid, block, st, a);
 }
 
 template <int DT>
-int launch_shrink_dt(bool row_major, int NB, int MT, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
-  if (row_major) return launch_shrink_nb<DT, 1, true>(NB, grid, st, a);  // the slow layout: one tile per wave
-  if (MT == 1) return launch_shrink_nb<DT, 1, false>(NB, grid, st, a);
-  return launch_shrink_nb<DT, kBlkTiles, false>(NB, grid, st, a);
+int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStream_t st,
+                     const ShrinkArgs& a) {
+  if (row_major) return launch_shrink_nb<DT, 1, kFwdWaves, true>(NB, grid, st, a);  // the slow layout
+  if (MT == 1)
+    return NW == 16 ? launch_shrink_nb<DT, 1, 16, false>(NB, grid, st, a)
+                    : launch_shrink_nb<DT, 1, kFwdWaves, false>(NB, grid, st, a);
+  return launch_shrink_nb<DT, kBlkTiles, kFwdWaves, false>(NB, grid, st, a);
 }
 
-// all projections of one launch share NB / U / MT (same rank, same T)
-int launch_shrink(int dtype, bool row_major, int NB, int MT, int S, hipStream_t st, ShrinkArgs& a) {
-  if (row_major) MT = 1;
-  a.gx = tile_units(a.T, S, MT);
-  dim3 grid((unsigned)((long)a.gx * a.gy * a.nproj));
-  if (dtype == SMLM_DTYPE_F16) return launch_shrink_dt<SMLM_DTYPE_F16>(row_major, NB, MT, grid, st, a);
-  return launch_shrink_dt<SMLM_DTYPE_BF16>(row_major, NB, MT, grid, st, a);
+// all projections of one launch share NB / U / MT / NW (same rank, same T)
+int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, hipStream_t st, ShrinkArgs& a) {
+  const int MT = row_major ? 1 : c.MT;
+  a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 1);
+  const dim3 grid = work_grid((long)tile_units_max(a.T, S, MT) * a.items.row_start[a.items.nproj]);
+  if (dtype == SMLM_DTYPE_F16)
+    return launch_shrink_dt<SMLM_DTYPE_F16>(row_major, c.NB, MT, c.NW, grid, st, a);
+  return launch_shrink_dt<SMLM_DTYPE_BF16>(row_major, c.NB, MT, c.NW, grid, st, a);
 }
 
 int launch_reduce(int dtype, int nt_max, hipStream_t st, const ReduceArgs& a) {
-  if (dtype == SMLM_DTYPE_F16)
-    return launch(reduce_kernel<SMLM_DTYPE_F16>, dim3(nt_max), dim3(256), st, a);
-  return launch(reduce_kernel<SMLM_DTYPE_BF16>, dim3(nt_max), dim3(256), st, a);
+  const dim3 grid = work_grid((long)nt_max * a.nproj);
+  if (dtype == SMLM_DTYPE_F16) return launch(reduce_kernel<SMLM_DTYPE_F16>, grid, dim3(256), st, a);
+  return launch(reduce_kernel<SMLM_DTYPE_BF16>, grid, dim3(256), st, a);
 }
 
-template <int DT, int NQ, int MT>
-int launch_expand_ks(int KS, dim3 grid, hipStream_t st, const ExpandArgs& a) {
-  if (KS == 1) return launch(expand_kernel<DT, NQ, 1, MT, false>, grid, dim3(kFwdThreads), st, a);
-  if (KS == 2) return launch(expand_kernel<DT, NQ, 2, MT, false>, grid, dim3(kFwdThreads), st, a);
-  return launch(expand_kernel<DT, NQ, 0, MT, false>, grid, dim3(kFwdThreads), st, a);
+template <int DT, int NQ>
+int launch_expand_wave(int KS, dim3 grid, hipStream_t st, const ExpandArgs& a) {
+  if (KS == 1) return launch(expand_wave_kernel<DT, NQ, 1, false>, grid, dim3(kFwdThreads), st, a);
+  if (KS == 2) return launch(expand_wave_kernel<DT, NQ, 2, false>, grid, dim3(kFwdThreads), st, a);
+  return launch(expand_wave_kernel<DT, NQ, 0, false>, grid, dim3(kFwdThreads), st, a);
 }
 
 template <int DT>
-int launch_expand_dt(bool row_major, int nq, int KS, int MT, dim3 grid, hipStream_t st,
+int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipStream_t st,
                      const ExpandArgs& a) {
-  if (row_major) return launch(expand_kernel<DT, 2, 0, 1, true>, grid, dim3(kFwdThreads), st, a);
-  if (MT == 1)
-    return nq == 4 ? launch_expand_ks<DT, 4, 1>(KS, grid, st, a) : launch_expand_ks<DT, 2, 1>(KS, grid, st, a);
-  return nq == 4 ? launch_expand_ks<DT, 4, kBlkTiles>(KS, grid, st, a)
-                 : launch_expand_ks<DT, 2, kBlkTiles>(KS, grid, st, a);
+  if (row_major) return launch(expand_wave_kernel<DT, 2, 0, true>, grid, dim3(kFwdThreads), st, a);
+  if (block)
+    return KS == 1 ? launch(expand_block_kernel<DT, 4, 1>, grid, dim3(kFwdThreads), st, a)
+                   : launch(expand_block_kernel<DT, 4, 2>, grid, dim3(kFwdThreads), st, a);
+  return nq == 4 ? launch_expand_wave<DT, 4>(KS, grid, st, a) : launch_expand_wave<DT, 2>(KS, grid, st, a);
 }
 
 // all projections of one launch share the rank (d_in); d_out may differ
-int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int max_d_in, int max_d_out,
+int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int nproj, int max_d_in,
                   hipStream_t st, ExpandArgs& a) {
-  if (row_major) { MT = 1; nq = 2; }
   const int KS = max_d_in <= 32 ? 1 : (max_d_in <= 64 ? 2 : 0);
-  a.gx = tile_units(a.T, S, MT);
-  a.gy = ceil_div(max_d_out, kFwdWaves * 32 * nq);
-  dim3 grid((unsigned)((long)a.gx * a.gy * a.nproj));
-  if (dtype == SMLM_DTYPE_F16) return launch_expand_dt<SMLM_DTYPE_F16>(row_major, nq, KS, MT, grid, st, a);
-  return launch_expand_dt<SMLM_DTYPE_BF16>(row_major, nq, KS, MT, grid, st, a);
+  const bool block = !row_major && MT > 1 && KS > 0;  // tile blocks with the weights staged in LDS
+  if (row_major) nq = 2;
+  if (block) nq = 4;
+  nq = tune("SMLM_TUNE_NQ", nq);
+  if (block) nq = 4;
+  const int chunk = block ? 32 * nq : kFwdWaves * 32 * nq;  // columns per workgroup
+  a.items.nproj = nproj;
+  a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 0);
+  a.items.row_start[0] = 0;
+  for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);
+  const dim3 grid =
+      work_grid((long)tile_units_max(a.T, S, block ? kBlkTiles : 1) * a.items.row_start[nproj]);
+  if (dtype == SMLM_DTYPE_F16)
+    return launch_expand_dt<SMLM_DTYPE_F16>(row_major, block, nq, KS, grid, st, a);
+  return launch_expand_dt<SMLM_DTYPE_BF16>(row_major, block, nq, KS, grid, st, a);
 }
 
 int check_common(int T, int S, int dtype) {
@@ -142,7 +191,7 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
   const int N = next_pow2(S);
   const PlanSortArgs sa{pv, seg_indptr, seg_key, key_kind, S, N};
   if (S <= kPlanSmallSegs && pv.nt_max <= kPlanSmallTiles)
-    return launch(plan_small_kernel, dim3(1), dim3(kPlanThreads), st, sa);
+    return launch(plan_small_kernel, dim3(1), dim3(round_up(S < 256 ? 256 : S, 64)), st, sa);
   int rc = (N <= kPlanLdsKeys)
                ? launch(plan_sort_kernel<true>, dim3(1), dim3(kPlanThreads), st, sa)
                : launch(plan_sort_kernel<false>, dim3(1), dim3(kPlanThreads), st, sa);
@@ -152,21 +201,27 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
   return launch(plan_fill_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), st, fa);
 }
 
-// shrink of one or more projections that share x-row routing and rank
+// shrink of one or more projections that share row routing and output width:
+// out[i] = beta*out[i] + scale * x[i] W_i^T in 16 bits, via k-split fp32 partial
+// sums folded by a second launch when the split is wider than one workgroup
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
-               const float* seg_scale, hipStream_t st, ShrinkCfg* cfgs) {
+               const float* seg_scale, hipStream_t st) {
   ShrinkArgs a{};
   a.plan = tile_args(pv);
   a.seg_scale = seg_scale;
   a.beta = beta;
   a.T = T;
-  a.nproj = nproj;
-  a.gy = 1;
+  a.items.nproj = nproj;
+  a.items.row_start[0] = 0;
+  ReduceArgs ra{};
+  bool need_reduce = false;
+  ShrinkCfg c0{};
+  const int nw = row_major ? kFwdWaves : shrink_waves(T, nproj, d_in, d_out);
   for (int i = 0; i < nproj; ++i) {
-    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out);
-    cfgs[i] = c;
+    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw);
+    if (i == 0) c0 = c;
     ShrinkProj& P = a.p[i];
     P.x = reinterpret_cast<const uint16_t*>(x[i]);
     P.w_ptrs = w_ptrs[i];
@@ -174,9 +229,17 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
     P.out = reinterpret_cast<uint16_t*>(out[i]);
     P.d_in = d_in[i]; P.d_out = d_out; P.ldw = ldw[i];
     P.k_per_wave = c.k_per_wave; P.ksplit = c.ksplit; P.zblocks = c.zblocks;
-    if (c.ksplit * c.zblocks > a.gy) a.gy = c.ksplit * c.zblocks;
+    a.items.row_start[i + 1] = a.items.row_start[i] + c.ksplit * c.zblocks;
+    ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit};
+    need_reduce = need_reduce || c.ksplit > 1;
   }
-  return launch_shrink(dtype, row_major, cfgs[0].NB, cfgs[0].MT, S, st, a);
+  int rc = launch_shrink(dtype, row_major, c0, S, st, a);
+  if (rc || !need_reduce) return rc;
+  ra.plan = a.plan;
+  ra.seg_scale = seg_scale;
+  ra.beta = beta;
+  ra.T = T; ra.d_out = d_out; ra.nproj = nproj;
+  return launch_reduce(dtype, pv.nt_max, st, ra);
 }
 
 struct BwdLayout {
@@ -193,8 +256,8 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
     off = align_up(off + bytes, 256);
     return o;
   };
-  L.cfg_dv = shrink_cfg(n_rows, h_out, r);
-  L.cfg_v = shrink_cfg(n_rows, h_in, r);
+  L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves);
+  L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves);
   const int ks = L.cfg_dv.ksplit > L.cfg_v.ksplit ? L.cfg_dv.ksplit : L.cfg_v.ksplit;
   L.pitch = (long)plan_nt_max(n_rows, P) * kTileRows;
   L.at = take((size_t)NA * h_in * r * 2);
@@ -261,7 +324,8 @@ SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t
   if (T > (1 << 30)) return SMLM_ERR_LIMIT;
   size_t n = 256;
   if (d_in >= d_out) {
-    const ShrinkCfg c = shrink_cfg(T, d_in, d_out);
+    // sized for the four-wave split, which never needs less than the sixteen-wave one
+    const ShrinkCfg c = shrink_cfg(T, d_in, d_out, kFwdWaves);
     if (c.ksplit > 1) n = align_up((size_t)c.ksplit * T * d_out * 4, 256);
   }
   *bytes = n;
@@ -295,28 +359,18 @@ SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs
     a.plan = tile_args(pv);
     a.seg_scale = seg_scale;
     a.beta = beta;
-    a.T = T; a.nproj = 1; a.nt_max = pv.nt_max;
+    a.T = T; a.nt_max = pv.nt_max;
     ExpandProj& P = a.p[0];
     P.y = reinterpret_cast<uint16_t*>(y);
     P.v = reinterpret_cast<const uint16_t*>(x);
     P.w_ptrs = w_ptrs;
-    P.d_in = d_in; P.d_out = d_out; P.ldw = w_ld; P.ksplit = 1;
-    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T), S, d_in,
-                         d_out, st, a);
+    P.d_in = d_in; P.d_out = d_out; P.ldw = w_ld;
+    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T), S, 1, d_in,
+                         st, a);
   }
   float* partial = reinterpret_cast<float*>(workspace);
-  ShrinkCfg c;
-  rc = run_shrink(dtype, w_row_major != 0, pv, T, S, 1, &x, &w_ptrs, &partial, &y, &d_in, d_out, &w_ld,
-                  beta, seg_scale, st, &c);
-  if (rc || c.ksplit == 1) return rc;
-  ReduceArgs ra{};
-  ra.plan = tile_args(pv);
-  ra.partial = partial;
-  ra.out = reinterpret_cast<uint16_t*>(y);
-  ra.seg_scale = seg_scale;
-  ra.beta = beta;
-  ra.T = T; ra.d_out = d_out; ra.ksplit = c.ksplit;
-  return launch_reduce(dtype, pv.nt_max, st, ra);
+  return run_shrink(dtype, w_row_major != 0, pv, T, S, 1, &x, &w_ptrs, &partial, &y, &d_in, d_out, &w_ld,
+                    beta, seg_scale, st);
 }
 
 SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes) {
@@ -362,8 +416,9 @@ SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_
   size_t n = 0;
   for (int i = 0; i < n_proj; ++i) {
     if (h_in[i] <= 0) return SMLM_ERR_ARG;
-    const ShrinkCfg c = shrink_cfg(T, h_in[i], r);
-    n += align_up((size_t)c.ksplit * (T > 0 ? T : 1) * r * 4, 256);
+    const ShrinkCfg c = shrink_cfg(T, h_in[i], r, kFwdWaves);
+    const size_t rows = T > 0 ? T : 1;
+    n += align_up((size_t)c.ksplit * rows * r * 4, 256) + align_up(rows * r * 2, 256);
   }
   *bytes = n;
   return SMLM_OK;
@@ -374,11 +429,12 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
                                  const void* const* const* b_ptrs, const int* h_in,
                                  const int* h_out, const void* plan, void* workspace,
                                  size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
-                                 const float* seg_scale, void* stream) {
+                                 const float* seg_scale, int stages, void* stream) {
   int rc = check_common(T, S, dtype);
   if (rc) return rc;
   if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
     return SMLM_ERR_ARG;
+  if (stages < 1 || stages > (SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND)) return SMLM_ERR_ARG;
   if (r & 7) return SMLM_ERR_ALIGN;
   int max_h_out = 0;
   for (int i = 0; i < n_proj; ++i) {
@@ -403,37 +459,39 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
   PlanView pv;
   plan_carve(const_cast<void*>(plan), T, S, &pv);
 
-  // shrink: every projection's v as k-split fp32 partial sums (or 16-bit when not split)
+  // shrink: every projection's v, rounded to 16 bits (into v_out when the caller wants it)
   float* partial[kMaxProj];
-  void* out16[kMaxProj];
-  ShrinkCfg cfgs[kMaxProj];
+  void* v16[kMaxProj];
   {
     char* w = reinterpret_cast<char*>(workspace);
     for (int i = 0; i < n_proj; ++i) {
-      const ShrinkCfg c = shrink_cfg(T, h_in[i], r);
+      const ShrinkCfg c = shrink_cfg(T, h_in[i], r, kFwdWaves);
       partial[i] = reinterpret_cast<float*>(w);
-      out16[i] = w;
       w += align_up((size_t)c.ksplit * T * r * 4, 256);
+      v16[i] = (v_out && v_out[i]) ? v_out[i] : w;
+      w += align_up((size_t)T * r * 2, 256);
     }
   }
-  rc = run_shrink(dtype, false, pv, T, S, n_proj, x, a_ptrs, partial, out16, h_in, r, h_in, 0.0f,
-                  nullptr, st, cfgs);
-  if (rc) return rc;
+  if (stages & SMLM_STAGE_SHRINK) {
+    rc = run_shrink(dtype, false, pv, T, S, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in, 0.0f, nullptr,
+                    st);
+    if (rc) return rc;
+  }
+  if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;
 
   ExpandArgs ea{};
   ea.plan = tile_args(pv);
   ea.seg_scale = seg_scale;
   ea.beta = beta;
-  ea.T = T; ea.nproj = n_proj; ea.nt_max = pv.nt_max;
+  ea.T = T; ea.nt_max = pv.nt_max;
   for (int i = 0; i < n_proj; ++i) {
     ExpandProj& P = ea.p[i];
     P.y = reinterpret_cast<uint16_t*>(y[i]);
-    if (cfgs[i].ksplit > 1) P.partial = partial[i]; else P.v = reinterpret_cast<const uint16_t*>(out16[i]);
+    P.v = reinterpret_cast<const uint16_t*>(v16[i]);
     P.w_ptrs = b_ptrs[i];
-    P.v_out = v_out ? reinterpret_cast<uint16_t*>(v_out[i]) : nullptr;
-    P.d_in = r; P.d_out = h_out[i]; P.ldw = r; P.ksplit = cfgs[i].ksplit;
+    P.d_in = r; P.d_out = h_out[i]; P.ldw = r;
   }
-  return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, r, max_h_out, st, ea);
+  return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, n_proj, r, st, ea);
 }
 
 SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes) {
@@ -446,7 +504,8 @@ SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* cons
                            size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
                            float beta, const float* seg_scale, void* stream) {
   return smlm_lora_fwd_multi(1, &y, &x, v_out ? &v_out : nullptr, &a_ptrs, &b_ptrs, &h_in, &h_out, plan,
-                             workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale, stream);
+                             workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale,
+                             SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND, stream);
 }
 
 SMLM_API int smlm_lora_bwd_workspace_size(int n_rows, int P, int NA, int h_in, int h_out, int r,
@@ -492,35 +551,28 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   plan_carve(const_cast<void*>(plan), n_rows, P, &pv);
 
   // 1. transposed copies of the training adapters' weights: At [h_in, r], Bt [r, h_out]
-  TransposeArgs ta{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
-  if ((rc = launch(transpose_kernel, dim3(ceil_div(h_in, 32), ceil_div(r, 32), NA), dim3(256), st, ta)))
-    return rc;
-  TransposeArgs tb{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
-  if ((rc = launch(transpose_kernel, dim3(ceil_div(r, 32), ceil_div(h_out, 32), NA), dim3(256), st, tb)))
-    return rc;
+  TransposeArgs ta{};
+  ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
+  ta.set[1] = TransposeSet{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
+  ta.NA = NA;
+  {
+    const int gx = ceil_div(h_in > h_out ? h_in : h_out, 32), gy = ceil_div(r, 32);
+    if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
+  }
 
   // 2. v = round16(x A^T) unless the forward saved it
   const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
-  ShrinkCfg c;
   if (!vv) {
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
-                         0.0f, nullptr, st, &c)))
+                         0.0f, nullptr, st)))
       return rc;
-    if (c.ksplit > 1) {
-      ReduceArgs ra{};
-      ra.plan = tile_args(pv);
-      ra.partial = partial;
-      ra.out = reinterpret_cast<uint16_t*>(v16);
-      ra.T = n_rows; ra.d_out = r; ra.ksplit = c.ksplit;
-      if ((rc = launch_reduce(dtype, pv.nt_max, st, ra))) return rc;
-    }
     vv = reinterpret_cast<const uint16_t*>(v16);
   }
 
-  // 3. dV = dY B  (k-split partial sums, or 16-bit when not split)
+  // 3. dV = round16(dY B)
   const void* const* btp = bt_ptrs;
   if ((rc = run_shrink(dtype, false, pv, n_rows, P, 1, &dy, &btp, &partial, &dv16, &h_out, r, &h_out,
-                       0.0f, nullptr, st, &c)))
+                       0.0f, nullptr, st)))
     return rc;
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
@@ -531,15 +583,15 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   ea.pt_b = pt_b;
   ea.v2 = vv;
   ea.beta = 0.0f;
-  ea.T = n_rows; ea.nproj = 1; ea.nt_max = pv.nt_max;
+  ea.T = n_rows; ea.nt_max = pv.nt_max;
   {
     ExpandProj& E = ea.p[0];
     E.y = reinterpret_cast<uint16_t*>(dx);
-    if (c.ksplit > 1) E.partial = partial; else E.v = reinterpret_cast<const uint16_t*>(dv16);
+    E.v = reinterpret_cast<const uint16_t*>(dv16);
     E.w_ptrs = at_ptrs;
-    E.d_in = r; E.d_out = h_in; E.ldw = r; E.ksplit = c.ksplit;
+    E.d_in = r; E.d_out = h_in; E.ldw = r;
   }
-  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, r, h_in, st,
+  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, 1, r, st,
                           ea)))
     return rc;
 

@@ -9,7 +9,7 @@
 
 namespace smlm {
 
-struct TransposeArgs {
+struct TransposeSet {
   const void* const* src_ptrs;  // [NA] matrices [rows, cols] row-major
   uint16_t* dst_base;           // NA matrices [cols, rows], `stride` elements apart
   const void** dst_ptrs;        // [NA] receives the address of each transposed matrix
@@ -17,25 +17,34 @@ struct TransposeArgs {
   int rows, cols;
 };
 
-// 32x32 tiles through LDS; grid (ceil(cols/32), ceil(rows/32), NA), block 256.
+struct TransposeArgs {
+  TransposeSet set[2];  // A [r, h_in] -> At [h_in, r] and B [h_out, r] -> Bt [r, h_out]
+  int NA;
+};
+
+// 32x32 tiles through LDS; grid (tiles along the hidden dimension, tiles along the
+// rank, 2*NA), block 256: x walks the columns of A and the rows of B.
 __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   __shared__ uint16_t t[32][33];
-  const int ad = blockIdx.z;
-  const uint16_t* src = reinterpret_cast<const uint16_t*>(a.src_ptrs[ad]);
-  uint16_t* dst = a.dst_base + (long)ad * a.stride;
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) a.dst_ptrs[ad] = dst;
+  const int which = blockIdx.z / a.NA, ad = blockIdx.z - which * a.NA;
+  const TransposeSet S = a.set[which];
+  const int c0 = (which == 0 ? blockIdx.x : blockIdx.y) * 32;
+  const int r0 = (which == 0 ? blockIdx.y : blockIdx.x) * 32;
+  if (c0 >= S.cols || r0 >= S.rows) return;  // uniform over the workgroup
+  const uint16_t* src = reinterpret_cast<const uint16_t*>(S.src_ptrs[ad]);
+  uint16_t* dst = S.dst_base + (long)ad * S.stride;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) S.dst_ptrs[ad] = dst;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r0 + ty + 8 * i, c = c0 + tx;
-    t[ty + 8 * i][tx] = (r < a.rows && c < a.cols) ? src[(long)r * a.cols + c] : (uint16_t)0;
+    t[ty + 8 * i][tx] = (r < S.rows && c < S.cols) ? src[(long)r * S.cols + c] : (uint16_t)0;
   }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = c0 + ty + 8 * i, r = r0 + tx;
-    if (r < a.rows && c < a.cols) dst[(long)c * a.rows + r] = t[tx][ty + 8 * i];
+    if (r < S.rows && c < S.cols) dst[(long)c * S.rows + r] = t[tx][ty + 8 * i];
   }
 }
 

@@ -85,6 +85,31 @@ __device__ __forceinline__ f32x4 ldg_f4(const float* p) {
   return *(const SMLM_GLOBAL f32x4*)(p);
 }
 
+// 16 bytes from p when ok, zeros otherwise, without a branch: the load always
+// runs (from `safe`, any readable 16-byte aligned address, when !ok) so that
+// the compiler keeps a run of such loads back to back.
+__device__ __forceinline__ u32x4 ldg16_if(const uint16_t* p, bool ok, const uint16_t* safe) {
+  const u32x4 v = ldg16(ok ? p : safe);
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  return ok ? v : zero;
+}
+
+// Reads of plan tables and pointer tables at a wave-uniform index.  These are
+// written by an earlier kernel and never by the kernel that reads them, so they
+// may go through the scalar (constant) path: the loads then cost no vector
+// memory slot and do not hold back the vector loads issued after them.
+#define SMLM_CONST __attribute__((address_space(4)))
+__device__ __forceinline__ int32_t uload(const int32_t* p, int i) {
+  return ((const SMLM_CONST int32_t*)p)[i];
+}
+__device__ __forceinline__ float uload(const float* p, int i) {
+  return ((const SMLM_CONST float*)p)[i];
+}
+__device__ __forceinline__ const uint16_t* uload_ptr(const void* const* tab, int i) {
+  const uint64_t v = ((const SMLM_CONST uint64_t*)tab)[i];
+  return reinterpret_cast<const uint16_t*>(v);
+}
+
 // Eight 16-bit elements with a stride (the slow gather used for the weight
 // layout the reference never passes).
 __device__ __forceinline__ u32x4 ldg_strided8(const uint16_t* p, long stride) {

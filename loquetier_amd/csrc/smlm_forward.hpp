@@ -13,12 +13,14 @@
 // whatever other rows share its tile or its wave, so regrouping or
 // re-segmenting rows never changes a bit of any row.
 //
-// Launches are one-dimensional.  Workgroups are handed to the 8 XCDs round
-// robin by their linear id, and each XCD has its own L2; xcd_remap() turns the
-// linear id into a work index such that each XCD walks one contiguous range of
-// (column chunk | k slice, tile block) pairs: all tile blocks that read one
-// slice of an adapter's weights run on the same XCD close in time, so that
-// slice is fetched from HBM once instead of once per XCD.
+// Launches are one-dimensional and persistent: the number of work items (tiles
+// x column chunks | k slices x projections) is only known on the device, in the
+// plan header, so a fixed grid walks the items.  Workgroups are handed to the 8
+// XCDs round robin by their linear id, and each XCD has its own L2; work_range()
+// gives each XCD one contiguous range of (projection, column chunk | k slice,
+// tile block) items: all tile blocks that read one slice of an adapter's weights
+// run on the same XCD close in time, so that slice is fetched from HBM once
+// instead of once per XCD.
 #pragma once
 #include "smlm_common.hpp"
 
@@ -37,34 +39,65 @@ struct TileArgs {
   const int32_t* blk;        // (first tile << 3) | tile count, per tile block
 };
 
-__device__ __forceinline__ int xcd_remap(int linear, int total) {
-  const int xcd = linear % kNumXcd, idx = linear / kNumXcd;
-  const int base = total / kNumXcd, extra = total % kNumXcd;
-  return xcd * base + (xcd < extra ? xcd : extra) + idx;
+// Items [first, last) of this workgroup, visited with stride `step`.  The grid
+// size is a multiple of kNumXcd.
+struct WorkRange {
+  int first, last, step;
+};
+__device__ __forceinline__ WorkRange work_range(int n_work, bool interleave) {
+  if (interleave) return WorkRange{(int)blockIdx.x, n_work, (int)gridDim.x};
+  const int xcd = blockIdx.x % kNumXcd, local = blockIdx.x / kNumXcd;
+  const int base = n_work / kNumXcd, extra = n_work % kNumXcd;
+  const int start = xcd * base + (xcd < extra ? xcd : extra);
+  const int count = base + (xcd < extra ? 1 : 0);
+  return WorkRange{start + local, start + count, (int)gridDim.x / kNumXcd};
 }
 
-// which tiles this workgroup works on: a single tile (MT == 1) or one tile
-// block of the plan (tiles of one adapter)
+// Items are numbered (chunk row, tile unit) with the tile unit fastest; the
+// chunk rows of all projections are laid end to end (row_start[p] = first chunk
+// row of projection p), so there are no empty items to skew the XCD ranges.
+struct ItemSpace {
+  int row_start[kMaxProj + 1];
+  int nproj;
+  int interleave;  // tuning: plain round-robin items instead of one range per XCD
+};
+__device__ __forceinline__ void item_decode(const ItemSpace& sp, int V, int units, int* pj, int* yy,
+                                            int* tb) {
+  const int cr = V / units;
+  *tb = V - cr * units;
+  int p = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxProj; ++i) p += (i < sp.nproj && cr >= sp.row_start[i]) ? 1 : 0;
+  *pj = p;
+  *yy = cr - sp.row_start[p];
+}
+
+// number of units along the tile axis: single tiles (MT == 1) or the plan's tile
+// blocks (tiles of one adapter, up to kBlkTiles each)
 template <int MT>
-__device__ __forceinline__ bool pick_tiles(const TileArgs& p, int tb, int* t0, int* cnt) {
+__device__ __forceinline__ int tile_units(const TileArgs& p) {
+  return MT == 1 ? p.hdr[0] : p.hdr[4];
+}
+template <int MT>
+__device__ __forceinline__ void pick_tiles(const TileArgs& p, int tb, int* t0, int* cnt) {
   if (MT == 1) {
-    if (tb >= p.hdr[0]) return false;
     *t0 = tb;
     *cnt = 1;
   } else {
-    if (tb >= p.hdr[4]) return false;
-    const int packed = p.blk[tb];
+    const int packed = uload(p.blk, tb);
     *t0 = packed >> 3;
     *cnt = packed & 7;
   }
-  return true;
 }
 
+// eight consecutive-k elements of weight column n (zeros when !ok)
 template <bool ROWMAJOR>
-__device__ __forceinline__ u32x4 load_w8(const uint16_t* W, int n, int k, int ldw) {
-  // eight consecutive-k elements of weight column n
-  if (ROWMAJOR) return ldg_strided8(W + (long)k * ldw + n, ldw);
-  return ldg16(W + (long)n * ldw + k);
+__device__ __forceinline__ u32x4 load_w8(const uint16_t* W, int n, int k, int ldw, bool ok) {
+  if (ROWMAJOR) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    return ok ? ldg_strided8(W + (long)k * ldw + n, ldw) : zero;
+  }
+  return ldg16_if(W + (long)n * ldw + k, ok, W);
 }
 
 // out = beta*old + scale*acc for four consecutive columns of one row
@@ -96,140 +129,152 @@ struct ShrinkArgs {
   ShrinkProj p[kMaxProj];
   const float* seg_scale;     // applied when ksplit == 1
   float beta;
-  int T, nproj, gx, gy;       // gx tile blocks, gy = max over projections of ksplit*zblocks
+  int T;
+  ItemSpace items;            // chunk rows of projection p: ksplit*zblocks
 };
 
-// Work index -> (projection, k slice, 64-column block, tile block).  The four
+// Work item -> (projection, k slice, 64-column block, tile block).  The NW
 // waves of a workgroup take consecutive k ranges; their accumulators are summed
 // through LDS in wave order and written either as an fp32 partial (ksplit > 1)
-// or as the final 16-bit value.
-template <int DT, int NB, int U, int MT, bool ROWMAJOR>
-__global__ __launch_bounds__(kFwdThreads) void shrink_kernel(ShrinkArgs a) {
-  const int V = xcd_remap(blockIdx.x, gridDim.x);
-  const int per = a.gx * a.gy;
-  const int pj = V / per, rem = V - pj * per;
-  const int yy = rem / a.gx, tb = rem - yy * a.gx;
-  const ShrinkProj P = a.p[pj];
-  const int kz = yy % P.ksplit, zb = yy / P.ksplit;
-  if (zb >= P.zblocks) return;
-  int t0, cnt;
-  if (!pick_tiles<MT>(a.plan, tb, &t0, &cnt)) return;
-
-  const int n0 = zb * 64;
+// or as the final 16-bit value.  NW = 16 lets one workgroup cover all of k for
+// small batches, so no partial sums leave the CU.
+template <int DT, int NB, int U, int MT, int NW, bool ROWMAJOR>
+__global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
+  constexpr int TP = (MT * NB > 8) ? 8 / NB : MT;  // tiles per cross-wave reduction pass
+  __shared__ f32x4 red[NW][TP][NB][kWaveSize];
+  const int units = tile_units<MT>(a.plan);
+  const WorkRange wr = work_range(units * a.items.row_start[a.items.nproj], a.items.interleave != 0);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
-
-  int row[MT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i) row[i] = i < cnt ? a.plan.tile_row[(t0 + i) * kTileRows + c] : -1;
-  const uint16_t* W = reinterpret_cast<const uint16_t*>(P.w_ptrs[a.plan.tile_wid[t0]]);
-
-  const int kbeg = (kz * kFwdWaves + wave) * P.k_per_wave;
-  const int kend = min(kbeg + P.k_per_wave, P.d_in);
-
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  f32x4 acc[MT][NB];
+
+  for (int V = wr.first; V < wr.last; V += wr.step) {
+    int pj, yy, tb;
+    item_decode(a.items, V, units, &pj, &yy, &tb);
+    const ShrinkProj P = a.p[pj];
+    const int kz = yy % P.ksplit, zb = yy / P.ksplit;
+    int t0, cnt;
+    pick_tiles<MT>(a.plan, tb, &t0, &cnt);
+    const int n0 = zb * 64;
+
+    int row[MT];
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < MT; ++i) row[i] = i < cnt ? a.plan.tile_row[(t0 + i) * kTileRows + c] : -1;
+    const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, t0));
+
+    const int kbeg = (kz * NW + wave) * P.k_per_wave;
+    const int kend = min(kbeg + P.k_per_wave, P.d_in);
+
+    f32x4 acc[MT][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll 1
-  for (int k = kbeg; k < kend; k += 32 * U) {
-    u32x4 xf[MT][U], wf[NB][U];
+    for (int k = kbeg; k < kend; k += 32 * U) {
+      u32x4 xf[MT][U], wf[NB][U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = k + 32 * u + 8 * g;
-      const bool kin = kk < kend;
+      for (int u = 0; u < U; ++u) {
+        const int kk = k + 32 * u + 8 * g;
+        const bool kin = kk < kend;
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        const int n = n0 + 16 * nb + c;
-        wf[nb][u] = (kin && n < P.d_out) ? load_w8<ROWMAJOR>(W, n, kk, P.ldw) : zero;
-      }
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-        xf[i][u] = (kin && row[i] >= 0) ? ldg16(P.x + (long)row[i] * P.d_in + kk) : zero;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-        if (i < cnt) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) acc[i][nb] = Num<DT>::mfma(wf[nb][u], xf[i][u], acc[i][nb]);
-        }
-  }
-
-  // cross-wave sum, TP tiles per pass, wave j finishing tile j of the pass
-  constexpr int TP = (MT * NB > 8) ? 8 / NB : MT;
-  __shared__ f32x4 red[kFwdWaves][TP][NB][kWaveSize];
-#pragma unroll
-  for (int pass = 0; pass < MT / TP; ++pass) {
-    if (pass * TP >= cnt) break;  // uniform over the workgroup
-#pragma unroll
-    for (int j = 0; j < TP; ++j)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) red[wave][j][nb][lane] = acc[pass * TP + j][nb];
-    __syncthreads();
-    const int i = pass * TP + wave;
-    if (wave < TP && i < cnt) {
-      const int slot = (t0 + i) * kTileRows + c;
-      const int r = a.plan.tile_row[slot];
-      if (r >= 0) {
-        float scale = 1.0f;
-        if (P.ksplit == 1 && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
+        for (int i = 0; i < MT; ++i)
+          xf[i][u] = ldg16_if(P.x + (long)row[i] * P.d_in + kk, kin && row[i] >= 0, P.x);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          f32x4 sum = red[0][wave][nb][lane];
-#pragma unroll
-          for (int w = 1; w < kFwdWaves; ++w) sum += red[w][wave][nb][lane];
-          const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
-          if (n >= P.d_out) continue;
-          if (P.ksplit > 1)
-            *reinterpret_cast<f32x4*>(P.partial + ((long)kz * a.T + r) * P.d_out + n) = sum;
-          else
-            store4<DT>(P.out + (long)r * P.d_out + n, sum, scale, a.beta);
+          const int n = n0 + 16 * nb + c;
+          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out);
         }
       }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+          if (i < cnt) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) acc[i][nb] = Num<DT>::mfma(wf[nb][u], xf[i][u], acc[i][nb]);
+          }
     }
-    __syncthreads();
+
+    // cross-wave sum, TP tiles per pass, wave j finishing tile j of the pass
+#pragma unroll
+    for (int pass = 0; pass < MT / TP; ++pass) {
+      if (pass * TP >= cnt) break;  // uniform over the workgroup
+#pragma unroll
+      for (int j = 0; j < TP; ++j)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) red[wave][j][nb][lane] = acc[pass * TP + j][nb];
+      __syncthreads();
+      const int i = pass * TP + wave;
+      if (wave < TP && i < cnt) {
+        const int slot = (t0 + i) * kTileRows + c;
+        const int r = a.plan.tile_row[slot];
+        if (r >= 0) {
+          float scale = 1.0f;
+          if (P.ksplit == 1 && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            f32x4 sum = red[0][wave][nb][lane];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) sum += red[w][wave][nb][lane];
+            const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
+            if (n >= P.d_out) continue;
+            if (P.ksplit > 1)
+              *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + r) * P.d_out + n) = sum;
+            else
+              store4<DT>(P.out + (long)r * P.d_out + n, sum, scale, a.beta);
+          }
+        }
+      }
+      __syncthreads();
+    }
   }
 }
 
-struct ReduceArgs {
-  TileArgs plan;
+struct ReduceProj {
   const float* partial;  // [ksplit, T, d_out]
   uint16_t* out;         // [T, d_out]
-  const float* seg_scale;
-  float beta;
-  int T, d_out, ksplit;
+  int ksplit;            // 1: nothing to fold for this projection
 };
 
-// Folds the k-split partials of a standalone shrink call, in split order.
+struct ReduceArgs {
+  TileArgs plan;
+  ReduceProj p[kMaxProj];
+  const float* seg_scale;
+  float beta;
+  int T, d_out, nproj;
+};
+
+// Folds the k-split partial sums of a shrink launch, in split order, into the
+// 16-bit result (the reference's "v in the I/O dtype"): work item -> (projection,
+// tile), 16 threads per row.
 template <int DT>
 __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
-  const int tile = blockIdx.x;
-  if (tile >= a.plan.hdr[0]) return;
+  const int units = a.plan.hdr[0];
   const int c = threadIdx.x >> 4, q = threadIdx.x & 15;
-  const int row = a.plan.tile_row[tile * kTileRows + c];
-  if (row < 0) return;
-  const int rseg = a.plan.tile_rseg[tile * kTileRows + c];
-  const float scale = a.seg_scale ? a.seg_scale[rseg] : 1.0f;
-  for (int n = 4 * q; n < a.d_out; n += 64) {
-    f32x4 sum = ldg_f4(a.partial + (long)row * a.d_out + n);
-    for (int z = 1; z < a.ksplit; ++z) sum += ldg_f4(a.partial + ((long)z * a.T + row) * a.d_out + n);
-    store4<DT>(a.out + (long)row * a.d_out + n, sum, scale, a.beta);
+  for (int V = blockIdx.x; V < units * a.nproj; V += gridDim.x) {
+    const int pj = V / units, tile = V - pj * units;
+    const ReduceProj P = a.p[pj];
+    if (P.ksplit <= 1) continue;
+    const int row = a.plan.tile_row[tile * kTileRows + c];
+    if (row < 0) continue;
+    const float scale = a.seg_scale ? a.seg_scale[a.plan.tile_rseg[tile * kTileRows + c]] : 1.0f;
+    for (int n = 4 * q; n < a.d_out; n += 64) {
+      f32x4 sum = ldg_f4(P.partial + (long)row * a.d_out + n);
+      for (int z = 1; z < P.ksplit; ++z) sum += ldg_f4(P.partial + ((long)z * a.T + row) * a.d_out + n);
+      store4<DT>(P.out + (long)row * a.d_out + n, sum, scale, a.beta);
+    }
   }
 }
 
 // ------------------------------------------------------------------ expand --
 struct ExpandProj {
   uint16_t* y;                // [T, d_out]
-  const uint16_t* v;          // [T, d_in] 16-bit, or null when partials are given
-  const float* partial;       // [ksplit, T, d_in] fp32 partial sums of v
+  const uint16_t* v;          // [T, d_in]
   const void* const* w_ptrs;  // indexed by the plan's tile_wid
-  uint16_t* v_out;            // optional [T, d_in]: rounded v, by row
-  int d_in, d_out, ldw, ksplit;
+  uint16_t* v_out;            // optional [T, d_in]: copy of v, by row
+  int d_in, d_out, ldw;
 };
 
 struct ExpandArgs {
@@ -240,78 +285,86 @@ struct ExpandArgs {
   uint16_t* pt_b;            // optional: same treatment of v2 (a second [T, d_in] matrix)
   const uint16_t* v2;
   float beta;
-  int T, nproj, gx, gy, nt_max;  // gx tile blocks, gy = max column chunks
+  int T, nt_max;
+  ItemSpace items;           // chunk rows of projection p: its column chunks
 };
 
-// one 32-wide k step of the token operand: partial sums folded in split order
-// and rounded to 16 bits (the reference's "v in the I/O dtype"), or 16-bit v
+// by-products one wave per tile writes while it holds the token fragment: the
+// rounded v by row, and scale*v / scale*v2 by tile slot, transposed ([k][slot]),
+// which the weight-gradient kernel reads with the token index innermost
 template <int DT>
-__device__ __forceinline__ u32x4 load_v8(const ExpandProj& P, int T, int row, int kk) {
-  if (P.partial) {
-    const float* pp = P.partial + (long)row * P.d_in + kk;
-    f32x4 s0 = ldg_f4(pp), s1 = ldg_f4(pp + 4);
-    for (int z = 1; z < P.ksplit; ++z) {
-      const float* pz = pp + (long)z * T * P.d_in;
-      s0 += ldg_f4(pz);
-      s1 += ldg_f4(pz + 4);
+__device__ __forceinline__ void write_side(const ExpandArgs& a, const ExpandProj& P, int slot, int row,
+                                           int kk, u32x4 vf, float scale) {
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  if (P.v_out && row >= 0) stg16(P.v_out + (long)row * P.d_in + kk, vf);
+  if (a.pt_a) {
+    const long pitch = (long)a.nt_max * kTileRows;
+    u32x4 v2f = zero;
+    if (a.pt_b && row >= 0) v2f = ldg16(a.v2 + (long)row * P.d_in + kk);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a.pt_a[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(vf[e]));
+      a.pt_a[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(vf[e]));
+      if (a.pt_b) {
+        a.pt_b[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(v2f[e]));
+        a.pt_b[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(v2f[e]));
+      }
     }
-    u32x4 r;
-    r[0] = pack2<DT>(s0[0], s0[1]);
-    r[1] = pack2<DT>(s0[2], s0[3]);
-    r[2] = pack2<DT>(s1[0], s1[1]);
-    r[3] = pack2<DT>(s1[2], s1[3]);
-    return r;
   }
-  return ldg16(P.v + (long)row * P.d_in + kk);
 }
 
-// Work index -> (projection, column chunk, tile block); each wave of the
-// workgroup owns 32*NQ output columns.  K (= LoRA rank) is short: with KS > 0
-// the weight fragments of all KS 32-wide k steps stay in registers and serve
-// every tile of the block; KS == 0 is the general loop over k.
+// y = beta*y + scale*acc for the eight consecutive columns a lane holds per q
+template <int DT, int NQ>
+__device__ __forceinline__ void store_tile(uint16_t* yrow, int ncol, int d_out, const f32x4 (&acc)[NQ][2],
+                                           const u32x4 (&yold)[NQ], float scale, float beta) {
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    if (ncol + 32 * q >= d_out) continue;
+    const f32x4 lo4 = acc[q][0], hi4 = acc[q][1];
+    u32x4 o;
+    if (beta != 0.0f) {
+      const u32x4 old = yold[q];
+      o[0] = pack2<DT>(beta * Num<DT>::lo(old[0]) + scale * lo4[0], beta * Num<DT>::hi(old[0]) + scale * lo4[1]);
+      o[1] = pack2<DT>(beta * Num<DT>::lo(old[1]) + scale * lo4[2], beta * Num<DT>::hi(old[1]) + scale * lo4[3]);
+      o[2] = pack2<DT>(beta * Num<DT>::lo(old[2]) + scale * hi4[0], beta * Num<DT>::hi(old[2]) + scale * hi4[1]);
+      o[3] = pack2<DT>(beta * Num<DT>::lo(old[3]) + scale * hi4[2], beta * Num<DT>::hi(old[3]) + scale * hi4[3]);
+    } else {
+      o[0] = pack2<DT>(scale * lo4[0], scale * lo4[1]);
+      o[1] = pack2<DT>(scale * lo4[2], scale * lo4[3]);
+      o[2] = pack2<DT>(scale * hi4[0], scale * hi4[1]);
+      o[3] = pack2<DT>(scale * hi4[2], scale * hi4[3]);
+    }
+    stg16(yrow + 32 * q, o);
+  }
+}
+
+// Expand, one tile per work item (small batches, decode): work item -> (projection,
+// column chunk, tile); each wave of the workgroup owns 32*NQ output columns and
+// loads its weight fragments straight into registers.  K (= LoRA rank) is
+// short: KS > 0 unrolls KS 32-wide k steps, KS == 0 is the general loop over k.
 // MFMA row m of column block (q,p) is output column 32q + 8(m/4) + 4p + m%4, so
 // that a lane's eight accumulators for one q are eight consecutive columns.
-template <int DT, int NQ, int KS, int MT, bool ROWMAJOR>
-__global__ __launch_bounds__(kFwdThreads) void expand_kernel(ExpandArgs a) {
-  const int V = xcd_remap(blockIdx.x, gridDim.x);
-  const int per = a.gx * a.gy;
-  const int pj = V / per, rem = V - pj * per;
-  const int yy = rem / a.gx, tb = rem - yy * a.gx;
-  const ExpandProj P = a.p[pj];
+template <int DT, int NQ, int KS, bool ROWMAJOR>
+__global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) {
+  const int units = a.plan.hdr[0];
+  const WorkRange wr = work_range(units * a.items.row_start[a.items.nproj], a.items.interleave != 0);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
-  const int ncol0 = (yy * kFwdWaves + wave) * 32 * NQ;
-  if (ncol0 >= P.d_out) return;
-  int t0, cnt;
-  if (!pick_tiles<MT>(a.plan, tb, &t0, &cnt)) return;
-  const uint16_t* W = reinterpret_cast<const uint16_t*>(P.w_ptrs[a.plan.tile_wid[t0]]);
-
-  const u32x4 zero = {0u, 0u, 0u, 0u};
   const int mrow = 8 * (c >> 2) + (c & 3);  // column offset of MFMA row c inside a (q,p) block
-  const bool side = (yy == 0 && wave == 0);  // the one wave per tile that writes by-products
-  constexpr int KSR = KS > 0 ? KS : 1;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  constexpr int KSU = KS > 0 ? KS : 1;
 
-  u32x4 wf[KSR][NQ][2];
-  if (KS > 0) {
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int kk = 32 * ks + 8 * g;
-#pragma unroll
-      for (int q = 0; q < NQ; ++q)
-#pragma unroll
-        for (int p = 0; p < 2; ++p) {
-          const int n = ncol0 + 32 * q + 4 * p + mrow;
-          wf[ks][q][p] = (kk < P.d_in && n < P.d_out) ? load_w8<ROWMAJOR>(W, n, kk, P.ldw) : zero;
-        }
-    }
-  }
-
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    if (i >= cnt) break;
-    const int slot = (t0 + i) * kTileRows + c;
+  for (int V = wr.first; V < wr.last; V += wr.step) {
+    int pj, yy, tile;
+    item_decode(a.items, V, units, &pj, &yy, &tile);
+    const ExpandProj P = a.p[pj];
+    const int ncol0 = (yy * kFwdWaves + wave) * 32 * NQ;
+    if (ncol0 >= P.d_out) continue;
+    const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, tile));
+    const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
     const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
+    const bool side = (yy == 0 && wave == 0);  // the one wave per tile that writes by-products
 
     // y rows this lane will update: fetch the old values early
     u32x4 yold[NQ];
@@ -319,7 +372,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_kernel(ExpandArgs a) {
     if (a.beta != 0.0f) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q)
-        yold[q] = (row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out) ? ldg16(yrow + 32 * q) : zero;
+        yold[q] = ldg16_if(yrow + 32 * q, row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, P.y);
     }
 
     f32x4 acc[NQ][2];
@@ -327,70 +380,107 @@ __global__ __launch_bounds__(kFwdThreads) void expand_kernel(ExpandArgs a) {
     for (int q = 0; q < NQ; ++q) acc[q][0] = acc[q][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int nks = KS > 0 ? KS : (P.d_in + 31) / 32;
-#pragma unroll KSR
+#pragma unroll KSU
     for (int ks = 0; ks < nks; ++ks) {
       const int kk = 32 * ks + 8 * g;
       const bool kin = kk < P.d_in;
-      const u32x4 vf = (kin && row >= 0) ? load_v8<DT>(P, a.T, row, kk) : zero;
-      if (side && kin) {
-        if (P.v_out && row >= 0) stg16(P.v_out + (long)row * P.d_in + kk, vf);
-        if (a.pt_a) {
-          // scale*v (and scale*v2) by tile slot, transposed: [k][slot]
-          const long pitch = (long)a.nt_max * kTileRows;
-          u32x4 v2f = zero;
-          if (a.pt_b && row >= 0) v2f = ldg16(a.v2 + (long)row * P.d_in + kk);
+      u32x4 wf[NQ][2];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            a.pt_a[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(vf[e]));
-            a.pt_a[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(vf[e]));
-            if (a.pt_b) {
-              a.pt_b[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(v2f[e]));
-              a.pt_b[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(v2f[e]));
-            }
-          }
+      for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const int n = ncol0 + 32 * q + 4 * p + mrow;
+          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out);
         }
-      }
-      if (KS > 0) {
+      const u32x4 vf = ldg16_if(P.v + (long)row * P.d_in + kk, kin && row >= 0, P.v);
+      if (side && kin) write_side<DT>(a, P, slot, row, kk, vf, scale);
 #pragma unroll
-        for (int q = 0; q < NQ; ++q)
+      for (int q = 0; q < NQ; ++q)
 #pragma unroll
-          for (int p = 0; p < 2; ++p) acc[q][p] = Num<DT>::mfma(wf[ks < KSR ? ks : 0][q][p], vf, acc[q][p]);
-      } else {
-        u32x4 wg[NQ][2];
+        for (int p = 0; p < 2; ++p) acc[q][p] = Num<DT>::mfma(wf[q][p], vf, acc[q][p]);
+    }
+    if (row >= 0) store_tile<DT, NQ>(yrow, ncol0 + 8 * g, P.d_out, acc, yold, scale, a.beta);
+  }
+}
+
+// Expand, one tile BLOCK per work item (prefill / fine-tuning batches): work item
+// -> (projection, column chunk of 32*NQ columns, tile block).  The workgroup
+// stages the chunk's weight rows in LDS once; wave w then multiplies tile w of
+// the block with them, so an adapter's B chunk is read from L2 once per four
+// tiles instead of once per tile.
+template <int DT, int NQ, int KS>
+__global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a) {
+  constexpr int kPitch = 32 * KS + 8;  // LDS row pitch in 16-bit elements: rows 16 bytes apart mod 128
+  __shared__ __attribute__((aligned(16))) uint16_t wlds[32 * NQ * kPitch];
+  const int units = a.plan.hdr[4];
+  const WorkRange wr = work_range(units * a.items.row_start[a.items.nproj], a.items.interleave != 0);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const int mrow = 8 * (c >> 2) + (c & 3);
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  for (int V = wr.first; V < wr.last; V += wr.step) {
+    int pj, yy, tb;
+    item_decode(a.items, V, units, &pj, &yy, &tb);
+    const ExpandProj P = a.p[pj];
+    const int ncol0 = yy * 32 * NQ;
+    const int packed = uload(a.plan.blk, tb);
+    const int t0 = packed >> 3, cnt = packed & 7;
+    const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, t0));
+    const bool active = wave < cnt;
+    const int slot = (t0 + (active ? wave : 0)) * kTileRows + c;
+    const int row = active ? a.plan.tile_row[slot] : -1;
+
+    // weight chunk -> registers (written to LDS below): 32*NQ rows of 4*KS 16-byte pieces
+    constexpr int kPieces = 32 * NQ * 4 * KS;
+    constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
+    u32x4 stage[kPer];
 #pragma unroll
-        for (int q = 0; q < NQ; ++q)
+    for (int j = 0; j < kPer; ++j) {
+      const int idx = threadIdx.x + j * kFwdThreads;
+      const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
+      stage[j] = ldg16_if(W + (long)(ncol0 + nl) * P.ldw + k8,
+                          idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in, W);
+    }
+    const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
+    u32x4 yold[NQ];
+    uint16_t* yrow = P.y + (long)(row < 0 ? 0 : row) * P.d_out + ncol0 + 8 * g;
+    if (a.beta != 0.0f) {
 #pragma unroll
-          for (int p = 0; p < 2; ++p) {
-            const int n = ncol0 + 32 * q + 4 * p + mrow;
-            wg[q][p] = (kin && n < P.d_out) ? load_w8<ROWMAJOR>(W, n, kk, P.ldw) : zero;
-          }
+      for (int q = 0; q < NQ; ++q)
+        yold[q] = ldg16_if(yrow + 32 * q, row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, P.y);
+    }
+    u32x4 vf[KS];
 #pragma unroll
-        for (int q = 0; q < NQ; ++q)
-#pragma unroll
-          for (int p = 0; p < 2; ++p) acc[q][p] = Num<DT>::mfma(wg[q][p], vf, acc[q][p]);
-      }
+    for (int ks = 0; ks < KS; ++ks) {
+      const int kk = 32 * ks + 8 * g;
+      vf[ks] = ldg16_if(P.v + (long)row * P.d_in + kk, kk < P.d_in && row >= 0, P.v);
+      if (yy == 0 && active && kk < P.d_in) write_side<DT>(a, P, slot, row, kk, vf[ks], scale);
     }
 
-    if (row < 0) continue;
+    __syncthreads();  // every wave is done reading the previous item's weights
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      if (ncol0 + 32 * q + 8 * g >= P.d_out) continue;
-      const f32x4 lo4 = acc[q][0], hi4 = acc[q][1];
-      u32x4 o;
-      if (a.beta != 0.0f) {
-        const u32x4 old = yold[q];
-        o[0] = pack2<DT>(a.beta * Num<DT>::lo(old[0]) + scale * lo4[0], a.beta * Num<DT>::hi(old[0]) + scale * lo4[1]);
-        o[1] = pack2<DT>(a.beta * Num<DT>::lo(old[1]) + scale * lo4[2], a.beta * Num<DT>::hi(old[1]) + scale * lo4[3]);
-        o[2] = pack2<DT>(a.beta * Num<DT>::lo(old[2]) + scale * hi4[0], a.beta * Num<DT>::hi(old[2]) + scale * hi4[1]);
-        o[3] = pack2<DT>(a.beta * Num<DT>::lo(old[3]) + scale * hi4[2], a.beta * Num<DT>::hi(old[3]) + scale * hi4[3]);
-      } else {
-        o[0] = pack2<DT>(scale * lo4[0], scale * lo4[1]);
-        o[1] = pack2<DT>(scale * lo4[2], scale * lo4[3]);
-        o[2] = pack2<DT>(scale * hi4[0], scale * hi4[1]);
-        o[3] = pack2<DT>(scale * hi4[2], scale * hi4[3]);
-      }
-      stg16(yrow + 32 * q, o);
+    for (int j = 0; j < kPer; ++j) {
+      const int idx = threadIdx.x + j * kFwdThreads;
+      const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
+      if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[nl * kPitch + k8]) = stage[j];
     }
+    __syncthreads();
+    if (!active) continue;  // whole waves only (MFMA runs with every lane); barriers are behind us
+
+    f32x4 acc[NQ][2];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) acc[q][0] = acc[q][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const u32x4 wf = *reinterpret_cast<const u32x4*>(&wlds[(32 * q + 4 * p + mrow) * kPitch + 32 * ks + 8 * g]);
+          acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
+        }
+    if (row >= 0) store_tile<DT, NQ>(yrow, ncol0 + 8 * g, P.d_out, acc, yold, scale, a.beta);
   }
 }
 

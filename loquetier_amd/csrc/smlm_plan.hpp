@@ -27,9 +27,9 @@ struct PlanSortArgs {
   int key_kind, S, N;  // N = power of two >= S
 };
 
-// Inclusive scan of one 64-bit value per thread over a 1024-thread block.
-// `wave_tot` is LDS scratch of 17 entries.  Returns the inclusive prefix; the
-// block total is left in wave_tot[16].
+// Inclusive scan of one 64-bit value per thread over the block (a multiple of 64
+// threads, at most 1024).  `wave_tot` is LDS scratch of 17 entries.  Returns the
+// inclusive prefix; the block total is left in wave_tot[16].
 __device__ __forceinline__ uint64_t block_scan_incl(uint64_t v, uint64_t* wave_tot) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -42,7 +42,7 @@ __device__ __forceinline__ uint64_t block_scan_incl(uint64_t v, uint64_t* wave_t
   __syncthreads();
   if (threadIdx.x == 0) {
     uint64_t run = 0;
-    for (int w = 0; w < kPlanThreads / 64; ++w) {
+    for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
       uint64_t t = wave_tot[w];
       wave_tot[w] = run;
       run += t;
@@ -70,7 +70,7 @@ __device__ __forceinline__ int usable_kind(const void* key, int key_kind, int S,
   __syncthreads();
   if (key_kind == SMLM_KEY_PTR) {
     const uint64_t* pk = reinterpret_cast<const uint64_t*>(key);
-    for (int i = threadIdx.x; i < S; i += kPlanThreads)
+    for (int i = threadIdx.x; i < S; i += blockDim.x)
       if ((pk[i] >> 48) != 0 || (pk[i] & 15) != 0) *bad_key = 1;
   }
   __syncthreads();
@@ -87,7 +87,7 @@ template <typename KeyArray>
 __device__ __forceinline__ void bitonic_sort(KeyArray K, int N) {
   for (int size = 2; size <= N; size <<= 1) {
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int i = threadIdx.x; i < (N >> 1); i += kPlanThreads) {
+      for (int i = threadIdx.x; i < (N >> 1); i += blockDim.x) {
         const int lo = 2 * i - (i & (stride - 1));
         const int hi = lo + stride;
         const bool asc = (lo & size) == 0;
@@ -115,7 +115,7 @@ __device__ __forceinline__ int last_le(Arr a, int n, int q) {
 
 // ---------------------------------------------------------------- one launch
 __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs args) {
-  __shared__ uint64_t K[kPlanSmallSegs];
+  __shared__ uint64_t K[kPlanSmallSegs], K0[kPlanSmallSegs];
   __shared__ int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];
   __shared__ int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
   __shared__ int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
@@ -123,12 +123,25 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   __shared__ int bad_key;
   const PlanView pv = args.pv;
   const int32_t* __restrict__ s = args.s;
-  const int S = args.S, N = args.N, tid = threadIdx.x;
+  const int S = args.S, tid = threadIdx.x;  // blockDim.x >= S
   const int kind = usable_kind(args.key, args.key_kind, S, &bad_key);
 
-  K[tid] = tid < S ? make_key(args.key, kind, tid) : ~0ull;
+  // Sort by counting: keys are distinct (segment index inside), so the sorted
+  // position of a key is the number of smaller keys.  One barrier instead of the
+  // log^2 barriers of a sorting network; S <= 1024 keeps the loop short.
+  const uint64_t mine = tid < S ? make_key(args.key, kind, tid) : ~0ull;
+  if (kind != SMLM_KEY_NONE) {
+    if (tid < S) K0[tid] = mine;
+    __syncthreads();
+    if (tid < S) {
+      int rank = 0;
+      for (int j = 0; j < S; ++j) rank += K0[j] < mine ? 1 : 0;
+      K[rank] = mine;
+    }
+  } else if (tid < S) {
+    K[tid] = mine;
+  }
   __syncthreads();
-  if (kind != SMLM_KEY_NONE) bitonic_sort(K, N);
 
   // gathered-row position of every sorted segment, group heads
   constexpr uint64_t kRowMask = (1ull << 40) - 1;
@@ -202,7 +215,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   }
   __syncthreads();
 
-  for (int b = tid; b < n_blocks; b += kPlanThreads) {
+  for (int b = tid; b < n_blocks; b += blockDim.x) {
     const int G = last_le(gblk, NG, b);
     const int tile0 = gtile[G] + (b - gblk[G]) * kBlkTiles;
     const int left = gtile[G + 1] - tile0;
@@ -210,7 +223,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   }
 
   // fill: one thread per tile slot
-  for (int slot = tid; slot < n_tiles * kTileRows; slot += kPlanThreads) {
+  for (int slot = tid; slot < n_tiles * kTileRows; slot += blockDim.x) {
     const int tile = slot / kTileRows, c = slot % kTileRows;
     const int G = last_le(gtile, NG, tile);
     const int q = grow[G] + (tile - gtile[G]) * kTileRows + c;

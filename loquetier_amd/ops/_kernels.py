@@ -210,9 +210,11 @@ def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_
 
 def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
-                            v_out=None) -> None:
+                            v_out=None, stages: int = 3) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
-    in two launches.  Lists of equal length; entries of xs may be the same tensor."""
+    in two launches.  Lists of equal length; entries of xs may be the same tensor.
+    stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
+    arguments on the same stream), 3 = both."""
     n = len(ys)
     if not (1 <= n <= 8) or len(xs) != n or len(a_ptrs) != n or len(b_ptrs) != n or \
             (v_out is not None and len(v_out) != n):
@@ -247,7 +249,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]), h_in, h_out,
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
-            _ptr(seg_scale), _stream(dev))
+            _ptr(seg_scale), int(stages), _stream(dev))
     _lib.check(rc, "smlm_lora_forward")
 
 
