@@ -111,14 +111,17 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
  * The same grouped GEMM with a plan built beforehand by smlm_plan_build for
  * (seg_indptr, T, S): nothing but the GEMM kernels is launched, so a caller
  * that issues many GEMMs over one batch (every layer and projection of a
- * model step) pays for the plan once.  No counterpart in the reference, which
- * rebuilds its problem table inside every call (smlm_forward_cutlass.cuh:76-79).
+ * model step) pays for the plan once.  n_weights is the number of entries of
+ * w_ptrs (adapters for an id-keyed plan, S otherwise; 0 = unknown): the number
+ * of distinct keys cannot exceed it, which bounds the launch size.  No
+ * counterpart in the reference, which rebuilds its problem table inside every
+ * call (smlm_forward_cutlass.cuh:76-79).
  */
 SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t* bytes);
-SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs, const void* plan,
-                               void* workspace, size_t workspace_bytes, int T, int S, int d_in,
-                               int d_out, int w_ld, int w_row_major, int dtype, float beta,
-                               const float* seg_scale, void* stream);
+SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs, int n_weights,
+                               const void* plan, void* workspace, size_t workspace_bytes, int T,
+                               int S, int d_in, int d_out, int w_ld, int w_row_major, int dtype,
+                               float beta, const float* seg_scale, void* stream);
 
 /*
  * Fused LoRA forward  y = beta*y + scale_i * round16(x A^T) B^T.
@@ -126,14 +129,14 @@ SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs
  * (src/loquetier_src/kernel_utils.py:115-119) plus, with beta = 1 and
  * seg_scale, the scale multiply and residual add of MixedLoraLinear.forward
  * (src/loquetier_src/models/mixed_lora.py:214-217).
- *   a_ptrs / b_ptrs: device arrays of device addresses, indexed as the plan's
- *     key kind says (see smlm_plan_build).
+ *   a_ptrs / b_ptrs: device arrays of n_weights device addresses, indexed as
+ *     the plan's key kind says (see smlm_plan_build); n_weights = 0 if unknown.
  *   plan: built by smlm_plan_build for the batch's (seg_indptr, T, S).
  *   v_out: NULL, or [T, r] receiving the rounded intermediate for backward.
  */
 SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes);
 SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* const* a_ptrs,
-                           const void* const* b_ptrs, const void* plan, void* workspace,
+                           const void* const* b_ptrs, int n_weights, const void* plan, void* workspace,
                            size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
                            float beta, const float* seg_scale, void* stream);
 
@@ -154,7 +157,7 @@ SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_
                                                 size_t* bytes);
 SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* x,
                                  void* const* v_out, const void* const* const* a_ptrs,
-                                 const void* const* const* b_ptrs, const int* h_in,
+                                 const void* const* const* b_ptrs, int n_weights, const int* h_in,
                                  const int* h_out, const void* plan, void* workspace,
                                  size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
                                  const float* seg_scale, int stages, void* stream);

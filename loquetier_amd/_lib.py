@@ -32,11 +32,12 @@ SIGNATURES = {
     "smlm_gemm_workspace_size": (_i, [_i, _i, _i, _i, _psz]),
     "smlm_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_gemm_planned_workspace_size": (_i, [_i, _i, _i, _psz]),
-    "smlm_gemm_planned": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
+    "smlm_gemm_planned": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_lora_fwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _psz]),
-    "smlm_lora_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
+    "smlm_lora_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _f, _vp,
+                           _vp]),
     "smlm_lora_fwd_multi_workspace_size": (_i, [_i, _i, _pi, _i, _psz]),
-    "smlm_lora_fwd_multi": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _pi, _pi, _vp, _vp, _sz, _i, _i, _i,
+    "smlm_lora_fwd_multi": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _i, _pi, _pi, _vp, _vp, _sz, _i, _i, _i,
                                  _i, _f, _vp, _i, _vp]),
     "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
     "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,

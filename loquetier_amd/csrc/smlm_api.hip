@@ -47,11 +47,20 @@ inline int tune(const char* name, int dflt) {
 
 inline int tiles_per_wave(int T) { return tune("SMLM_TUNE_MT", T >= 1024 ? kBlkTiles : 1); }
 
-// upper bound of the number of work units along the tile axis
-inline int tile_units_max(int T, int S, int mt) {
-  const int nt_max = plan_nt_max(T, S);
-  return mt == 1 ? nt_max : nt_max / kBlkTiles + S + 2;
+// Upper bound of the number of work units along the tile axis.  `groups` bounds
+// the number of distinct plan keys (adapters): every group ends in at most one
+// partly filled tile and one partly filled tile block.
+inline int tile_units_max(int T, int S, int groups, int mt) {
+  const int g = (groups > 0 && groups < S) ? groups : S;
+  const int nt = T / kTileRows + g + 1;  // never above the plan's own bound plan_nt_max(T, S)
+  const int nb = nt / kBlkTiles + g + 2;
+  return (mt == 1 || nb > nt) ? nt : nb;  // there are never more tile blocks than tiles
 }
+
+// Launches of at most this many items run one item per workgroup (direct mode); measured
+// faster than the persistent walk at every size tried (up to ~130k workgroups), so the walk
+// is only the fallback for batches far beyond those.
+constexpr long kDirectItems = 1L << 22;
 
 // persistent 1-D grid: a multiple of the XCD count, no larger than the work bound
 constexpr int kMaxGrid = 2048;
@@ -106,60 +115,84 @@ TileArgs tile_args(const PlanView& pv) {
   return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
 }
 
-template <int DT, int MT, int NW, bool RM>
+// grid of a launch: three-dimensional (tile unit, chunk row, projection) in direct mode,
+// else the persistent one-dimensional grid
+inline dim3 item_grid(const ItemSpace& sp, long items) {
+  if (!sp.units_max) return work_grid(items);
+  int rows = 1;
+  for (int i = 0; i < sp.nproj; ++i)
+    if (sp.row_start[i + 1] - sp.row_start[i] > rows) rows = sp.row_start[i + 1] - sp.row_start[i];
+  return dim3((unsigned)sp.units_max, (unsigned)rows, (unsigned)sp.nproj);
+}
+
+template <int DT, int MT, int NW, bool RM, bool DIRECT>
 int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   const dim3 block(NW * kWaveSize);
   constexpr int UF = NW == 16 ? 2 : 1;  // must match shrink_cfg
-  if (NB == 1) return launch(shrink_kernel<DT, 1, 4 * UF, MT, NW, RM>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_kernel<DT, 2, 4 * UF, MT, NW, RM>, grid, block, st, a);
-  return launch(shrink_kernel<DT, 4, 2 * UF, MT, NW, RM>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4 * UF, MT, NW, RM, DIRECT>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4 * UF, MT, NW, RM, DIRECT>, grid, block, st, a);
+  return launch(shrink_kernel<DT, 4, 2 * UF, MT, NW, RM, DIRECT>, grid, block, st, a);
 }
 
-template <int DT>
+template <int DT, bool DIRECT>
 int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStream_t st,
                      const ShrinkArgs& a) {
-  if (row_major) return launch_shrink_nb<DT, 1, kFwdWaves, true>(NB, grid, st, a);  // the slow layout
+  if (row_major)  // the slow layout
+    return launch_shrink_nb<DT, 1, kFwdWaves, true, DIRECT>(NB, grid, st, a);
   if (MT == 1)
-    return NW == 16 ? launch_shrink_nb<DT, 1, 16, false>(NB, grid, st, a)
-                    : launch_shrink_nb<DT, 1, kFwdWaves, false>(NB, grid, st, a);
-  return launch_shrink_nb<DT, kBlkTiles, kFwdWaves, false>(NB, grid, st, a);
+    return NW == 16 ? launch_shrink_nb<DT, 1, 16, false, DIRECT>(NB, grid, st, a)
+                    : launch_shrink_nb<DT, 1, kFwdWaves, false, DIRECT>(NB, grid, st, a);
+  return launch_shrink_nb<DT, kBlkTiles, kFwdWaves, false, DIRECT>(NB, grid, st, a);
 }
 
 // all projections of one launch share NB / U / MT / NW (same rank, same T)
-int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, hipStream_t st, ShrinkArgs& a) {
+int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int groups, hipStream_t st,
+                  ShrinkArgs& a) {
   const int MT = row_major ? 1 : c.MT;
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 1);
-  const dim3 grid = work_grid((long)tile_units_max(a.T, S, MT) * a.items.row_start[a.items.nproj]);
-  if (dtype == SMLM_DTYPE_F16)
-    return launch_shrink_dt<SMLM_DTYPE_F16>(row_major, c.NB, MT, c.NW, grid, st, a);
-  return launch_shrink_dt<SMLM_DTYPE_BF16>(row_major, c.NB, MT, c.NW, grid, st, a);
+  const int units = tile_units_max(a.T, S, groups, MT);
+  const long items = (long)units * a.items.row_start[a.items.nproj];
+  a.items.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;
+  const dim3 grid = item_grid(a.items, items);
+  const bool f16 = dtype == SMLM_DTYPE_F16;
+  if (a.items.units_max)
+    return f16 ? launch_shrink_dt<SMLM_DTYPE_F16, true>(row_major, c.NB, MT, c.NW, grid, st, a)
+               : launch_shrink_dt<SMLM_DTYPE_BF16, true>(row_major, c.NB, MT, c.NW, grid, st, a);
+  return f16 ? launch_shrink_dt<SMLM_DTYPE_F16, false>(row_major, c.NB, MT, c.NW, grid, st, a)
+             : launch_shrink_dt<SMLM_DTYPE_BF16, false>(row_major, c.NB, MT, c.NW, grid, st, a);
 }
 
-int launch_reduce(int dtype, int nt_max, hipStream_t st, const ReduceArgs& a) {
-  const dim3 grid = work_grid((long)nt_max * a.nproj);
+int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
+  const int units = tile_units_max(a.T, S, groups, 1);
+  const long items = (long)units * a.nproj;
+  a.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;
+  const dim3 grid = a.units_max ? dim3((unsigned)items) : work_grid(items);
   if (dtype == SMLM_DTYPE_F16) return launch(reduce_kernel<SMLM_DTYPE_F16>, grid, dim3(256), st, a);
   return launch(reduce_kernel<SMLM_DTYPE_BF16>, grid, dim3(256), st, a);
 }
 
-template <int DT, int NQ>
+template <int DT, int NQ, bool DIRECT>
 int launch_expand_wave(int KS, dim3 grid, hipStream_t st, const ExpandArgs& a) {
-  if (KS == 1) return launch(expand_wave_kernel<DT, NQ, 1, false>, grid, dim3(kFwdThreads), st, a);
-  if (KS == 2) return launch(expand_wave_kernel<DT, NQ, 2, false>, grid, dim3(kFwdThreads), st, a);
-  return launch(expand_wave_kernel<DT, NQ, 0, false>, grid, dim3(kFwdThreads), st, a);
+  const dim3 block(kFwdThreads);
+  if (KS == 1) return launch(expand_wave_kernel<DT, NQ, 1, false, DIRECT>, grid, block, st, a);
+  if (KS == 2) return launch(expand_wave_kernel<DT, NQ, 2, false, DIRECT>, grid, block, st, a);
+  return launch(expand_wave_kernel<DT, NQ, 0, false, DIRECT>, grid, block, st, a);
 }
 
-template <int DT>
+template <int DT, bool DIRECT>
 int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipStream_t st,
                      const ExpandArgs& a) {
-  if (row_major) return launch(expand_wave_kernel<DT, 2, 0, true>, grid, dim3(kFwdThreads), st, a);
+  if (row_major)
+    return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT>, grid, dim3(kFwdThreads), st, a);
   if (block)
-    return KS == 1 ? launch(expand_block_kernel<DT, 4, 1>, grid, dim3(kFwdThreads), st, a)
-                   : launch(expand_block_kernel<DT, 4, 2>, grid, dim3(kFwdThreads), st, a);
-  return nq == 4 ? launch_expand_wave<DT, 4>(KS, grid, st, a) : launch_expand_wave<DT, 2>(KS, grid, st, a);
+    return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
+                   : launch(expand_block_kernel<DT, 4, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
+  return nq == 4 ? launch_expand_wave<DT, 4, DIRECT>(KS, grid, st, a)
+                 : launch_expand_wave<DT, 2, DIRECT>(KS, grid, st, a);
 }
 
 // all projections of one launch share the rank (d_in); d_out may differ
-int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int nproj, int max_d_in,
+int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, int nproj, int max_d_in,
                   hipStream_t st, ExpandArgs& a) {
   const int KS = max_d_in <= 32 ? 1 : (max_d_in <= 64 ? 2 : 0);
   const bool block = !row_major && MT > 1 && KS > 0;  // tile blocks with the weights staged in LDS
@@ -172,11 +205,16 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int nproj, i
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 0);
   a.items.row_start[0] = 0;
   for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);
-  const dim3 grid =
-      work_grid((long)tile_units_max(a.T, S, block ? kBlkTiles : 1) * a.items.row_start[nproj]);
-  if (dtype == SMLM_DTYPE_F16)
-    return launch_expand_dt<SMLM_DTYPE_F16>(row_major, block, nq, KS, grid, st, a);
-  return launch_expand_dt<SMLM_DTYPE_BF16>(row_major, block, nq, KS, grid, st, a);
+  const int units = tile_units_max(a.T, S, groups, block ? kBlkTiles : 1);
+  const long items = (long)units * a.items.row_start[nproj];
+  a.items.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;
+  const dim3 grid = item_grid(a.items, items);
+  const bool f16 = dtype == SMLM_DTYPE_F16;
+  if (a.items.units_max)
+    return f16 ? launch_expand_dt<SMLM_DTYPE_F16, true>(row_major, block, nq, KS, grid, st, a)
+               : launch_expand_dt<SMLM_DTYPE_BF16, true>(row_major, block, nq, KS, grid, st, a);
+  return f16 ? launch_expand_dt<SMLM_DTYPE_F16, false>(row_major, block, nq, KS, grid, st, a)
+             : launch_expand_dt<SMLM_DTYPE_BF16, false>(row_major, block, nq, KS, grid, st, a);
 }
 
 int check_common(int T, int S, int dtype) {
@@ -191,7 +229,7 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
   const int N = next_pow2(S);
   const PlanSortArgs sa{pv, seg_indptr, seg_key, key_kind, S, N};
   if (S <= kPlanSmallSegs && pv.nt_max <= kPlanSmallTiles)
-    return launch(plan_small_kernel, dim3(1), dim3(round_up(S < 256 ? 256 : S, 64)), st, sa);
+    return launch(plan_small_kernel, dim3(1), dim3(kPlanThreads), st, sa);
   int rc = (N <= kPlanLdsKeys)
                ? launch(plan_sort_kernel<true>, dim3(1), dim3(kPlanThreads), st, sa)
                : launch(plan_sort_kernel<false>, dim3(1), dim3(kPlanThreads), st, sa);
@@ -204,7 +242,7 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 // shrink of one or more projections that share row routing and output width:
 // out[i] = beta*out[i] + scale * x[i] W_i^T in 16 bits, via k-split fp32 partial
 // sums folded by a second launch when the split is wider than one workgroup
-int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int nproj,
+int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
                const float* seg_scale, hipStream_t st) {
@@ -233,13 +271,17 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
     ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit};
     need_reduce = need_reduce || c.ksplit > 1;
   }
-  int rc = launch_shrink(dtype, row_major, c0, S, st, a);
+  // Folding the k-split partials inside the shrink launch (last-arriving workgroup, ticket
+  // counters) was measured and dropped: the device-scope release/acquire it needs writes back
+  // and invalidates a whole L2 per workgroup on this multi-XCD part and cost 5-10x the launch
+  // it saves.
+  int rc = launch_shrink(dtype, row_major, c0, S, groups, st, a);
   if (rc || !need_reduce) return rc;
   ra.plan = a.plan;
   ra.seg_scale = seg_scale;
   ra.beta = beta;
   ra.T = T; ra.d_out = d_out; ra.nproj = nproj;
-  return launch_reduce(dtype, pv.nt_max, st, ra);
+  return launch_reduce(dtype, S, groups, st, ra);
 }
 
 struct BwdLayout {
@@ -332,10 +374,10 @@ SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t
   return SMLM_OK;
 }
 
-SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs, const void* plan,
-                               void* workspace, size_t workspace_bytes, int T, int S, int d_in,
-                               int d_out, int w_ld, int w_row_major, int dtype, float beta,
-                               const float* seg_scale, void* stream) {
+SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs, int n_weights,
+                               const void* plan, void* workspace, size_t workspace_bytes, int T,
+                               int S, int d_in, int d_out, int w_ld, int w_row_major, int dtype,
+                               float beta, const float* seg_scale, void* stream) {
   int rc = check_common(T, S, dtype);
   if (rc) return rc;
   if (d_in <= 0 || d_out <= 0 || w_ld <= 0) return SMLM_ERR_ARG;
@@ -365,12 +407,12 @@ SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs
     P.v = reinterpret_cast<const uint16_t*>(x);
     P.w_ptrs = w_ptrs;
     P.d_in = d_in; P.d_out = d_out; P.ldw = w_ld;
-    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T), S, 1, d_in,
-                         st, a);
+    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T), S, n_weights,
+                         1, d_in, st, a);
   }
   float* partial = reinterpret_cast<float*>(workspace);
-  return run_shrink(dtype, w_row_major != 0, pv, T, S, 1, &x, &w_ptrs, &partial, &y, &d_in, d_out, &w_ld,
-                    beta, seg_scale, st);
+  return run_shrink(dtype, w_row_major != 0, pv, T, S, n_weights, 1, &x, &w_ptrs, &partial, &y, &d_in,
+                    d_out, &w_ld, beta, seg_scale, st);
 }
 
 SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes) {
@@ -405,7 +447,7 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
   const size_t plan_bytes = plan_carve(workspace, T, S, &pv);
   rc = plan_build_impl(pv, seg_indptr, w_ptrs, SMLM_KEY_PTR, S, st);
   if (rc) return rc;
-  return smlm_gemm_planned(y, x, w_ptrs, workspace, reinterpret_cast<char*>(workspace) + plan_bytes,
+  return smlm_gemm_planned(y, x, w_ptrs, S, workspace, reinterpret_cast<char*>(workspace) + plan_bytes,
                            workspace_bytes - plan_bytes, T, S, d_in, d_out, w_ld, w_row_major, dtype,
                            beta, seg_scale, stream);
 }
@@ -426,7 +468,7 @@ SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_
 
 SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* x,
                                  void* const* v_out, const void* const* const* a_ptrs,
-                                 const void* const* const* b_ptrs, const int* h_in,
+                                 const void* const* const* b_ptrs, int n_weights, const int* h_in,
                                  const int* h_out, const void* plan, void* workspace,
                                  size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
                                  const float* seg_scale, int stages, void* stream) {
@@ -473,8 +515,8 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
     }
   }
   if (stages & SMLM_STAGE_SHRINK) {
-    rc = run_shrink(dtype, false, pv, T, S, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in, 0.0f, nullptr,
-                    st);
+    rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
+                    0.0f, nullptr, st);
     if (rc) return rc;
   }
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;
@@ -491,7 +533,8 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
     P.w_ptrs = b_ptrs[i];
     P.d_in = r; P.d_out = h_out[i]; P.ldw = r;
   }
-  return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, n_proj, r, st, ea);
+  return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, n_weights, n_proj, r,
+                       st, ea);
 }
 
 SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes) {
@@ -500,10 +543,11 @@ SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int
 }
 
 SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* const* a_ptrs,
-                           const void* const* b_ptrs, const void* plan, void* workspace,
+                           const void* const* b_ptrs, int n_weights, const void* plan, void* workspace,
                            size_t workspace_bytes, int T, int S, int h_in, int h_out, int r, int dtype,
                            float beta, const float* seg_scale, void* stream) {
-  return smlm_lora_fwd_multi(1, &y, &x, v_out ? &v_out : nullptr, &a_ptrs, &b_ptrs, &h_in, &h_out, plan,
+  return smlm_lora_fwd_multi(1, &y, &x, v_out ? &v_out : nullptr, &a_ptrs, &b_ptrs, n_weights, &h_in,
+                             &h_out, plan,
                              workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale,
                              SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND, stream);
 }
@@ -563,7 +607,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   // 2. v = round16(x A^T) unless the forward saved it
   const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
   if (!vv) {
-    if ((rc = run_shrink(dtype, false, pv, n_rows, P, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
+    if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
                          0.0f, nullptr, st)))
       return rc;
     vv = reinterpret_cast<const uint16_t*>(v16);
@@ -571,7 +615,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
 
   // 3. dV = round16(dY B)
   const void* const* btp = bt_ptrs;
-  if ((rc = run_shrink(dtype, false, pv, n_rows, P, 1, &dy, &btp, &partial, &dv16, &h_out, r, &h_out,
+  if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &h_out,
                        0.0f, nullptr, st)))
     return rc;
 
@@ -591,7 +635,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
     E.w_ptrs = at_ptrs;
     E.d_in = r; E.d_out = h_in; E.ldw = r;
   }
-  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, 1, r, st,
+  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, NA, 1, r, st,
                           ea)))
     return rc;
 

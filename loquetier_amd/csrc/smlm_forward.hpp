@@ -56,10 +56,15 @@ __device__ __forceinline__ WorkRange work_range(int n_work, bool interleave) {
 // Items are numbered (chunk row, tile unit) with the tile unit fastest; the
 // chunk rows of all projections are laid end to end (row_start[p] = first chunk
 // row of projection p), so there are no empty items to skew the XCD ranges.
+// units_max > 0 selects the direct mode used for small launches: one item per
+// workgroup, numbered over the host's upper bound of the tile units, so the
+// kernel need not wait for the plan header; units past the real count are
+// marked empty in the plan (tile_wid < 0, blk == 0).
 struct ItemSpace {
   int row_start[kMaxProj + 1];
   int nproj;
-  int interleave;  // tuning: plain round-robin items instead of one range per XCD
+  int interleave;  // plain round-robin items instead of one range per XCD
+  int units_max;
 };
 __device__ __forceinline__ void item_decode(const ItemSpace& sp, int V, int units, int* pj, int* yy,
                                             int* tb) {
@@ -71,22 +76,46 @@ __device__ __forceinline__ void item_decode(const ItemSpace& sp, int V, int unit
   *pj = p;
   *yy = cr - sp.row_start[p];
 }
+// DIRECT launches are three-dimensional: x = tile unit, y = chunk row of the
+// projection, z = projection, so that the projection's arguments can be read
+// at once with the rest of the kernel arguments.
+template <bool DIRECT>
+__device__ __forceinline__ WorkRange item_range(const ItemSpace& sp, int units) {
+  if (DIRECT) return WorkRange{0, 1, 1};
+  return work_range(units * sp.row_start[sp.nproj], sp.interleave != 0);
+}
+template <bool DIRECT>
+__device__ __forceinline__ bool item_get(const ItemSpace& sp, int V, int units, int* pj, int* yy,
+                                         int* tb) {
+  if (DIRECT) {
+    *pj = blockIdx.z;
+    *yy = blockIdx.y;
+    *tb = blockIdx.x;
+    return *yy < sp.row_start[*pj + 1] - sp.row_start[*pj];
+  }
+  item_decode(sp, V, units, pj, yy, tb);
+  return true;
+}
 
 // number of units along the tile axis: single tiles (MT == 1) or the plan's tile
 // blocks (tiles of one adapter, up to kBlkTiles each)
 template <int MT>
-__device__ __forceinline__ int tile_units(const TileArgs& p) {
+__device__ __forceinline__ int tile_units(const TileArgs& p, int units_max) {
+  if (units_max > 0) return units_max;
   return MT == 1 ? p.hdr[0] : p.hdr[4];
 }
+// tiles of unit tb and their weight index; cnt == 0 for a unit past the end
 template <int MT>
-__device__ __forceinline__ void pick_tiles(const TileArgs& p, int tb, int* t0, int* cnt) {
+__device__ __forceinline__ void pick_tiles(const TileArgs& p, int tb, int* t0, int* cnt, int* wid) {
   if (MT == 1) {
     *t0 = tb;
-    *cnt = 1;
+    *wid = uload(p.tile_wid, tb);
+    *cnt = *wid < 0 ? 0 : 1;
   } else {
     const int packed = uload(p.blk, tb);
     *t0 = packed >> 3;
     *cnt = packed & 7;
+    *wid = *cnt ? uload(p.tile_wid, *t0) : -1;
   }
 }
 
@@ -136,31 +165,42 @@ struct ShrinkArgs {
 // Work item -> (projection, k slice, 64-column block, tile block).  The NW
 // waves of a workgroup take consecutive k ranges; their accumulators are summed
 // through LDS in wave order and written either as an fp32 partial (ksplit > 1)
-// or as the final 16-bit value.  NW = 16 lets one workgroup cover all of k for
-// small batches, so no partial sums leave the CU.
-template <int DT, int NB, int U, int MT, int NW, bool ROWMAJOR>
+// or as the final 16-bit value.  NW = 16 lets one workgroup cover all of k, so
+// no partial sums leave the CU.
+template <int DT, int NB, int U, int MT, int NW, bool ROWMAJOR, bool DIRECT>
 __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
   constexpr int TP = (MT * NB > 8) ? 8 / NB : MT;  // tiles per cross-wave reduction pass
   __shared__ f32x4 red[NW][TP][NB][kWaveSize];
-  const int units = tile_units<MT>(a.plan);
-  const WorkRange wr = work_range(units * a.items.row_start[a.items.nproj], a.items.interleave != 0);
+  const int units = DIRECT ? 0 : tile_units<MT>(a.plan, 0);
+  const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
-  const u32x4 zero = {0u, 0u, 0u, 0u};
 
+#ifdef SMLM_TUNING
+  long long tick[6];
+  tick[0] = wall_clock64();
+#define SMLM_TICK(i) tick[i] = wall_clock64()
+#else
+#define SMLM_TICK(i) do {} while (0)
+#endif
   for (int V = wr.first; V < wr.last; V += wr.step) {
     int pj, yy, tb;
-    item_decode(a.items, V, units, &pj, &yy, &tb);
+    if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tb)) break;
     const ShrinkProj P = a.p[pj];
     const int kz = yy % P.ksplit, zb = yy / P.ksplit;
-    int t0, cnt;
-    pick_tiles<MT>(a.plan, tb, &t0, &cnt);
+    int t0, cnt, wid;
+    pick_tiles<MT>(a.plan, tb, &t0, &cnt, &wid);
+    if (cnt == 0) continue;  // uniform over the workgroup
     const int n0 = zb * 64;
 
     int row[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) row[i] = i < cnt ? a.plan.tile_row[(t0 + i) * kTileRows + c] : -1;
-    const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, t0));
+    const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+#ifdef SMLM_TUNING
+    SMLM_TICK(1);
+    if (row[0] == -12345 || W == nullptr) continue;  // keeps the tick after the metadata loads
+#endif
 
     const int kbeg = (kz * NW + wave) * P.k_per_wave;
     const int kend = min(kbeg + P.k_per_wave, P.d_in);
@@ -197,6 +237,10 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
           }
     }
 
+#ifdef SMLM_TUNING
+    SMLM_TICK(2);
+    if (acc[0][0][0] == -12345.678f) continue;  // keeps the tick after the MFMA loop
+#endif
     // cross-wave sum, TP tiles per pass, wave j finishing tile j of the pass
 #pragma unroll
     for (int pass = 0; pass < MT / TP; ++pass) {
@@ -209,7 +253,9 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
       const int i = pass * TP + wave;
       if (wave < TP && i < cnt) {
         const int slot = (t0 + i) * kTileRows + c;
-        const int r = a.plan.tile_row[slot];
+        int r = row[0];  // row of tile i, picked from registers
+#pragma unroll
+        for (int j = 1; j < MT; ++j) r = (i == j) ? row[j] : r;
         if (r >= 0) {
           float scale = 1.0f;
           if (P.ksplit == 1 && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
@@ -229,7 +275,16 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
       }
       __syncthreads();
     }
+
+#ifdef SMLM_TUNING
+    SMLM_TICK(3);
+    if (threadIdx.x == 0 && blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0) {
+      int32_t* dbg = const_cast<int32_t*>(a.plan.hdr);
+      for (int i = 1; i < 4; ++i) dbg[8 + i - 1] = (int)(tick[i] - tick[i - 1]);
+    }
+#endif
   }
+#undef SMLM_TICK
 }
 
 struct ReduceProj {
@@ -244,6 +299,7 @@ struct ReduceArgs {
   const float* seg_scale;
   float beta;
   int T, d_out, nproj;
+  int units_max;  // > 0: direct mode, one (projection, tile) per workgroup over this tile bound
 };
 
 // Folds the k-split partial sums of a shrink launch, in split order, into the
@@ -251,12 +307,14 @@ struct ReduceArgs {
 // tile), 16 threads per row.
 template <int DT>
 __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
-  const int units = a.plan.hdr[0];
+  const int units = tile_units<1>(a.plan, a.units_max);
   const int c = threadIdx.x >> 4, q = threadIdx.x & 15;
-  for (int V = blockIdx.x; V < units * a.nproj; V += gridDim.x) {
+  const int last = a.units_max > 0 ? (int)blockIdx.x + 1 : units * a.nproj;
+  for (int V = blockIdx.x; V < last; V += gridDim.x) {
     const int pj = V / units, tile = V - pj * units;
     const ReduceProj P = a.p[pj];
     if (P.ksplit <= 1) continue;
+    if (uload(a.plan.tile_wid, tile) < 0) continue;  // past the last tile (direct mode)
     const int row = a.plan.tile_row[tile * kTileRows + c];
     if (row < 0) continue;
     const float scale = a.seg_scale ? a.seg_scale[a.plan.tile_rseg[tile * kTileRows + c]] : 1.0f;
@@ -344,23 +402,24 @@ __device__ __forceinline__ void store_tile(uint16_t* yrow, int ncol, int d_out, 
 // short: KS > 0 unrolls KS 32-wide k steps, KS == 0 is the general loop over k.
 // MFMA row m of column block (q,p) is output column 32q + 8(m/4) + 4p + m%4, so
 // that a lane's eight accumulators for one q are eight consecutive columns.
-template <int DT, int NQ, int KS, bool ROWMAJOR>
+template <int DT, int NQ, int KS, bool ROWMAJOR, bool DIRECT>
 __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) {
-  const int units = a.plan.hdr[0];
-  const WorkRange wr = work_range(units * a.items.row_start[a.items.nproj], a.items.interleave != 0);
+  const int units = DIRECT ? 0 : tile_units<1>(a.plan, 0);
+  const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
   const int mrow = 8 * (c >> 2) + (c & 3);  // column offset of MFMA row c inside a (q,p) block
-  const u32x4 zero = {0u, 0u, 0u, 0u};
   constexpr int KSU = KS > 0 ? KS : 1;
 
   for (int V = wr.first; V < wr.last; V += wr.step) {
     int pj, yy, tile;
-    item_decode(a.items, V, units, &pj, &yy, &tile);
+    if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tile)) break;
     const ExpandProj P = a.p[pj];
     const int ncol0 = (yy * kFwdWaves + wave) * 32 * NQ;
     if (ncol0 >= P.d_out) continue;
-    const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, tile));
+    const int wid = uload(a.plan.tile_wid, tile);
+    if (wid < 0) continue;  // past the last tile (direct mode)
+    const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
     const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
@@ -408,24 +467,24 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 // stages the chunk's weight rows in LDS once; wave w then multiplies tile w of
 // the block with them, so an adapter's B chunk is read from L2 once per four
 // tiles instead of once per tile.
-template <int DT, int NQ, int KS>
+template <int DT, int NQ, int KS, bool DIRECT>
 __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a) {
   constexpr int kPitch = 32 * KS + 8;  // LDS row pitch in 16-bit elements: rows 16 bytes apart mod 128
   __shared__ __attribute__((aligned(16))) uint16_t wlds[32 * NQ * kPitch];
-  const int units = a.plan.hdr[4];
-  const WorkRange wr = work_range(units * a.items.row_start[a.items.nproj], a.items.interleave != 0);
+  const int units = DIRECT ? 0 : tile_units<kBlkTiles>(a.plan, 0);
+  const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
   const int mrow = 8 * (c >> 2) + (c & 3);
-  const u32x4 zero = {0u, 0u, 0u, 0u};
 
   for (int V = wr.first; V < wr.last; V += wr.step) {
     int pj, yy, tb;
-    item_decode(a.items, V, units, &pj, &yy, &tb);
+    if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tb)) break;
     const ExpandProj P = a.p[pj];
     const int ncol0 = yy * 32 * NQ;
     const int packed = uload(a.plan.blk, tb);
     const int t0 = packed >> 3, cnt = packed & 7;
+    if (cnt == 0) continue;  // past the last block (direct mode); uniform over the workgroup
     const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, t0));
     const bool active = wave < cnt;
     const int slot = (t0 + (active ? wave : 0)) * kTileRows + c;

@@ -40,14 +40,17 @@ __device__ __forceinline__ uint64_t block_scan_incl(uint64_t v, uint64_t* wave_t
   __syncthreads();  // previous users of wave_tot are done
   if (lane == 63) wave_tot[wave] = v;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint64_t run = 0;
-    for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
-      uint64_t t = wave_tot[w];
-      wave_tot[w] = run;
-      run += t;
+  if (wave == 0) {  // exclusive scan of the (at most 16) wave totals, in registers
+    const int nw = (int)(blockDim.x >> 6);
+    const uint64_t t = lane < nw ? wave_tot[lane] : 0;
+    uint64_t run = t;
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) {
+      uint64_t o = __shfl_up((unsigned long long)run, d, 64);
+      if (lane >= d) run += o;
     }
-    wave_tot[16] = run;
+    if (lane < nw) wave_tot[lane] = run - t;
+    if (lane == nw - 1) wave_tot[16] = run;
   }
   __syncthreads();
   return v + wave_tot[wave];
@@ -114,35 +117,90 @@ __device__ __forceinline__ int last_le(Arr a, int n, int q) {
 }
 
 // ---------------------------------------------------------------- one launch
+// All global reads (keys, segment boundaries) are issued together up front: a
+// first-touch global load costs more than everything else in this kernel, so
+// nothing that was loaded is asked for again; the sorted arrays live in LDS.
 __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs args) {
   __shared__ uint64_t K[kPlanSmallSegs], K0[kPlanSmallSegs];
-  __shared__ int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];
+  __shared__ int32_t start0[kPlanSmallSegs], len0[kPlanSmallSegs];  // by segment
+  __shared__ int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];  // by sorted position
   __shared__ int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
   __shared__ int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
   __shared__ uint64_t wave_tot[17];
   __shared__ int bad_key;
   const PlanView pv = args.pv;
-  const int32_t* __restrict__ s = args.s;
   const int S = args.S, tid = threadIdx.x;  // blockDim.x >= S
-  const int kind = usable_kind(args.key, args.key_kind, S, &bad_key);
+#ifdef SMLM_TUNING
+  long long tick[8];
+  int ntick = 0;
+#define SMLM_TICK() do { __syncthreads(); tick[ntick++] = wall_clock64(); } while (0)
+#else
+#define SMLM_TICK() do {} while (0)
+#endif
+  SMLM_TICK();
+
+  uint64_t raw = 0;
+  int s0 = 0, s1 = 0;
+  if (tid < S) {
+    if (args.key_kind == SMLM_KEY_I32) raw = (uint32_t) reinterpret_cast<const int32_t*>(args.key)[tid];
+    if (args.key_kind == SMLM_KEY_PTR) raw = reinterpret_cast<const uint64_t*>(args.key)[tid];
+    s0 = args.s[tid];
+    s1 = args.s[tid + 1];
+  }
+  if (tid == 0) bad_key = 0;
+  __syncthreads();
+  // A 16-byte aligned address below 2^48 packs into 44 bits; anything else
+  // cannot be a sort key, so such a batch is planned segment by segment.
+  if (args.key_kind == SMLM_KEY_PTR && tid < S && ((raw >> 48) != 0 || (raw & 15) != 0)) bad_key = 1;
+  if (tid < S) {
+    start0[tid] = s0;
+    len0[tid] = s1 > s0 ? s1 - s0 : 0;
+  }
+  __syncthreads();
+  SMLM_TICK();
+  const int kind = bad_key ? SMLM_KEY_NONE : args.key_kind;
+  uint64_t mine = ~0ull;
+  if (tid < S) {
+    const uint64_t gkey = kind == SMLM_KEY_I32 ? raw : (kind == SMLM_KEY_PTR ? raw >> 4 : (uint64_t)tid);
+    mine = (gkey << kSegBits) | (uint32_t)tid;
+  }
 
   // Sort by counting: keys are distinct (segment index inside), so the sorted
-  // position of a key is the number of smaller keys.  One barrier instead of the
-  // log^2 barriers of a sorting network; S <= 1024 keeps the loop short.
-  const uint64_t mine = tid < S ? make_key(args.key, kind, tid) : ~0ull;
+  // position of a key is the number of smaller keys.  The block's threads split
+  // the S x S comparisons: thread (part, i) counts the keys of its part below
+  // key i, eight LDS reads in flight at a time, and adds its count to rank[i].
   if (kind != SMLM_KEY_NONE) {
-    if (tid < S) K0[tid] = mine;
-    __syncthreads();
     if (tid < S) {
-      int rank = 0;
-      for (int j = 0; j < S; ++j) rank += K0[j] < mine ? 1 : 0;
-      K[rank] = mine;
+      K0[tid] = mine;
+      sseg[tid] = 0;  // rank accumulator for now
     }
+    __syncthreads();
+    const int Sp = S <= 64 ? 64 : (S <= 128 ? 128 : (S <= 256 ? 256 : (S <= 512 ? 512 : 1024)));
+    const int parts = (int)blockDim.x / Sp;  // blockDim.x is a multiple of Sp
+    const int i = tid % Sp, part = tid / Sp;
+    if (i < S && part < parts) {
+      const uint64_t key = K0[i];
+      const int per = (S + parts - 1) / parts;
+      const int j0 = part * per, j1 = (j0 + per < S) ? j0 + per : S;
+      int rank = 0, j = j0;
+      for (; j + 8 <= j1; j += 8) {
+        uint64_t k8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) k8[e] = K0[j + e];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rank += k8[e] < key ? 1 : 0;
+      }
+      for (; j < j1; ++j) rank += K0[j] < key ? 1 : 0;
+      if (rank) atomicAdd(&sseg[i], rank);  // integer adds: the total does not depend on their order
+    }
+    __syncthreads();
+    if (tid < S) K[sseg[tid]] = mine;
   } else if (tid < S) {
     K[tid] = mine;
   }
   __syncthreads();
 
+  SMLM_TICK();
   // gathered-row position of every sorted segment, group heads
   constexpr uint64_t kRowMask = (1ull << 40) - 1;
   int seg = 0, len = 0;
@@ -152,8 +210,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     const uint64_t k = K[tid];
     seg = (int)(k & (kMaxSegments - 1));
     gk = k >> kSegBits;
-    len = s[seg + 1] - s[seg];
-    if (len < 0) len = 0;
+    len = len0[seg];
     head = true;
     if (tid > 0) head = (K[tid - 1] >> kSegBits) != gk;
   }
@@ -181,25 +238,22 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   }
   __syncthreads();
 
-  // tiles per group -> first tile of each group
+  // tiles and tile blocks per group -> first tile / first block of each group (one scan)
   uint64_t nt = 0;
   if (tid < NG) nt = (uint64_t)((grow[tid + 1] - grow[tid] + kTileRows - 1) / kTileRows);
-  const uint64_t tincl = block_scan_incl(nt, wave_tot);
-  const int n_tiles = (int)wave_tot[16];
+  const uint64_t nb = (nt + kBlkTiles - 1) / kBlkTiles;
+  const uint64_t both = nt | (nb << 32);
+  const uint64_t bincl = block_scan_incl(both, wave_tot);
+  const int n_tiles = (int)(wave_tot[16] & 0xffffffffu), n_blocks = (int)(wave_tot[16] >> 32);
   if (tid < NG) {
-    gtile[tid] = (int)(tincl - nt);
-    pv.grp_tile[tid] = (int)(tincl - nt);
+    const uint64_t ex = bincl - both;
+    gtile[tid] = (int)(ex & 0xffffffffu);
+    gblk[tid] = (int)(ex >> 32);
+    pv.grp_tile[tid] = gtile[tid];
+    pv.grp_blk[tid] = gblk[tid];
     pv.grp_row[tid] = grow[tid];
     pv.grp_seg[tid] = gseg[tid];
     pv.grp_id[tid] = gid[tid];
-  }
-  // tile blocks per group -> first block of each group
-  const uint64_t nb = (nt + kBlkTiles - 1) / kBlkTiles;
-  const uint64_t bincl = block_scan_incl(nb, wave_tot);
-  const int n_blocks = (int)wave_tot[16];
-  if (tid < NG) {
-    gblk[tid] = (int)(bincl - nb);
-    pv.grp_blk[tid] = (int)(bincl - nb);
   }
   if (tid == 0) {
     gtile[NG] = n_tiles;
@@ -215,14 +269,22 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   }
   __syncthreads();
 
-  for (int b = tid; b < n_blocks; b += blockDim.x) {
-    const int G = last_le(gblk, NG, b);
-    const int tile0 = gtile[G] + (b - gblk[G]) * kBlkTiles;
-    const int left = gtile[G + 1] - tile0;
-    pv.blk[b] = (tile0 << 3) | (left < kBlkTiles ? left : kBlkTiles);
+  SMLM_TICK();
+  // tile blocks; entries past the last one say "no tiles" (kernels launched over an
+  // upper bound of the block count stop there without reading the header)
+  for (int b = tid; b < pv.nt_max; b += blockDim.x) {
+    int packed = 0;
+    if (b < n_blocks) {
+      const int G = last_le(gblk, NG, b);
+      const int tile0 = gtile[G] + (b - gblk[G]) * kBlkTiles;
+      const int left = gtile[G + 1] - tile0;
+      packed = (tile0 << 3) | (left < kBlkTiles ? left : kBlkTiles);
+    }
+    pv.blk[b] = packed;
   }
 
-  // fill: one thread per tile slot
+  // fill: one thread per tile slot; tiles past the last one get weight index -1
+  for (int tile = n_tiles + tid; tile < pv.nt_max; tile += blockDim.x) pv.tile_wid[tile] = -1;
   for (int slot = tid; slot < n_tiles * kTileRows; slot += blockDim.x) {
     const int tile = slot / kTileRows, c = slot % kTileRows;
     const int G = last_le(gtile, NG, tile);
@@ -231,12 +293,18 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     if (q < grow[G + 1]) {
       const int a = last_le(rowpos, S, q);
       rseg = sseg[a];
-      row = s[rseg] + (q - rowpos[a]);
+      row = start0[rseg] + (q - rowpos[a]);
     }
     pv.tile_row[slot] = row;
     pv.tile_rseg[slot] = rseg;
     if (c == 0) pv.tile_wid[tile] = (kind == SMLM_KEY_I32) ? gid[G] : gseg[G];
   }
+  SMLM_TICK();
+#ifdef SMLM_TUNING
+  if (tid == 0)
+    for (int i = 1; i < ntick; ++i) pv.hdr[8 + i - 1] = (int)(tick[i] - tick[i - 1]);
+#endif
+#undef SMLM_TICK
 }
 
 // --------------------------------------------------------------- two launches
@@ -365,14 +433,21 @@ __global__ __launch_bounds__(256) void plan_fill_kernel(PlanFillArgs args) {
   const int tile = (int)(slot / kTileRows), c = (int)(slot % kTileRows);
   if (tile >= pv.nt_max) return;
   const int NG = pv.hdr[1];
-  if (slot < pv.hdr[4]) {  // the first n_blocks threads also write the tile-block table
+  if (slot < pv.nt_max) {  // the first nt_max threads also write the tile-block table
     const int b = (int)slot;
-    const int Gb = last_le(pv.grp_blk, NG, b);
-    const int tile0 = pv.grp_tile[Gb] + (b - pv.grp_blk[Gb]) * kBlkTiles;
-    const int left = pv.grp_tile[Gb + 1] - tile0;
-    pv.blk[b] = (tile0 << 3) | (left < kBlkTiles ? left : kBlkTiles);
+    int packed = 0;  // past the last block: "no tiles"
+    if (b < pv.hdr[4]) {
+      const int Gb = last_le(pv.grp_blk, NG, b);
+      const int tile0 = pv.grp_tile[Gb] + (b - pv.grp_blk[Gb]) * kBlkTiles;
+      const int left = pv.grp_tile[Gb + 1] - tile0;
+      packed = (tile0 << 3) | (left < kBlkTiles ? left : kBlkTiles);
+    }
+    pv.blk[b] = packed;
   }
-  if (tile >= pv.hdr[0]) return;
+  if (tile >= pv.hdr[0]) {  // past the last tile: weight index -1
+    if (c == 0) pv.tile_wid[tile] = -1;
+    return;
+  }
   // last group whose first tile is <= tile (empty groups share a first tile
   // with their successor, so "last" lands on the one that owns the tile)
   const int G = last_le(pv.grp_tile, NG, tile);

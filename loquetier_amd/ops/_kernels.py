@@ -191,7 +191,7 @@ def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, pl
     with torch.cuda.device(dev):
         need = _lib.size_query("smlm_gemm_planned_workspace_size", T, d_in, d_out)
         ws = _workspace(dev, need)
-        rc = _lib.load().smlm_gemm_planned(y.data_ptr(), x.data_ptr(), w_ptrs.data_ptr(),
+        rc = _lib.load().smlm_gemm_planned(y.data_ptr(), x.data_ptr(), w_ptrs.data_ptr(), w_ptrs.size(0),
                                            plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), T, plan.S,
                                            d_in, d_out, w_ld, int(bool(is_row_major)), code,
                                            float(beta), _ptr(seg_scale), _stream(dev))
@@ -247,7 +247,8 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
         ws = _workspace(dev, need.value)
         rc = _lib.load().smlm_lora_fwd_multi(
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
-            VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]), h_in, h_out,
+            VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
+            min(t.size(0) for t in list(a_ptrs) + list(b_ptrs)), h_in, h_out,
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
             _ptr(seg_scale), int(stages), _stream(dev))
     _lib.check(rc, "smlm_lora_forward")

@@ -78,7 +78,7 @@ def test_argument_validation_codes(lib):
     assert L.smlm_plan_build(p, big, p, None, 2, 16, 2, None) == -1   # key kind needs keys
     assert L.smlm_plan_build(p, big, p, p, 9, 16, 2, None) == -1      # unknown key kind
     assert L.smlm_plan_build(p, 64, p, None, 0, 16, 2, None) == -4
-    assert L.smlm_lora_fwd(p, p, None, p, p, p, p, big, 16, 2, 64, 64, 12, 0, 0.0, None, None) == -3
+    assert L.smlm_lora_fwd(p, p, None, p, p, 2, p, p, big, 16, 2, 64, 64, 12, 0, 0.0, None, None) == -3
     assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, big, 16, 1, 1, 64, 64, 128, 1,
                            None, None) == -6        # rank above the backward kernels' limit
     assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, 16, 16, 1, 1, 64, 64, 8, 1,
