@@ -103,6 +103,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
     ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch the steps one by one instead of replaying a graph (for counter runs)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a 128 MiB device copy three times before the timed region: a kernel "
+                         "of known traffic to scale FETCH_SIZE / WRITE_SIZE readings with")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; every box has one MI355X and no collective, "
@@ -183,8 +188,9 @@ def main():
                                   [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
                                   v_out=[d["v"] for d in pr] if P else None, stages=stages)
 
-    def step(st):
-        st["plan"] = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
+    def step(st, build_plan=True):
+        if build_plan:
+            st["plan"] = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
         fwd(st)
         if P:
             bplan = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
@@ -199,7 +205,27 @@ def main():
             step(st)
     torch.cuda.synchronize()
 
+    if args.calibration_copy:
+        src = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    class Eager:
+        """Stands in for a captured graph: replay() launches the work directly."""
+
+        def __init__(self, fn):
+            self.fn = fn
+
+        def replay(self):
+            with torch.cuda.stream(cap_stream):
+                self.fn()
+
     def capture(fn):
+        if args.eager:
+            return Eager(fn)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, stream=cap_stream):
             fn()
@@ -209,11 +235,12 @@ def main():
         """graph_runs: list of (graph, times).  Returns elapsed ms between HIP events
         recorded on the stream the graphs are launched on."""
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
+        run_stream = cap_stream if args.eager else torch.cuda.current_stream()
+        a.record(run_stream)
         for g, n in graph_runs:
             for _ in range(n):
                 g.replay()
-        b.record()
+        b.record(run_stream)
         torch.cuda.synchronize()
         return a.elapsed_time(b)
 
@@ -252,6 +279,12 @@ def main():
         g = capture(lambda: [fwd(st, stages) for _ in range(reps) for st in sets])
         timed([(g, 2)])
         return timed([(g, 10)]) * 1e3 / (10 * reps * R)  # us per launch
+
+    # the same step with the batch's plan built once and reused, as the layers of one model
+    # step reuse it (reported beside the headline value, never as it)
+    g_reuse = capture(lambda: [step(st, build_plan=False) for st in sets])
+    timed([(g_reuse, 2)])
+    reuse_ms = timed([(g_reuse, max(1, args.steps // R))]) / (max(1, args.steps // R) * R)
 
     expand_us = stage_us(2)
     shrink_us = stage_us(1)
@@ -305,10 +338,11 @@ def main():
         "config": {"workload": w["name"], "tokens_per_step": T, "segments": S, "adapters": NA, "rank": r,
                    "projections": [f"{n}:{a}->{b}" for n, a, b in w["proj"]],
                    "buffer_sets_rotated": R, "step_includes": "plan build + fused forward per projection"
-                   + (" + backward" if P else ""), "graph_replay": True},
+                   + (" + backward" if P else ""), "graph_replay": not args.eager},
         "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
         "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "ms_per_step_plan_reused": round(reuse_ms, 5),
         "roofline": roofline,
         "kernels": {"shrink_us": round(shrink_us, 3), "shrink_bytes": shrink_bytes,
                     "shrink_gbps": round(shrink_bytes / (shrink_us * 1e-6) / 1e9, 1),

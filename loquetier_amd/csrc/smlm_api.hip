@@ -61,6 +61,7 @@ inline int tile_units_max(int T, int S, int groups, int mt) {
 // faster than the persistent walk at every size tried (up to ~130k workgroups), so the walk
 // is only the fallback for batches far beyond those.
 constexpr long kDirectItems = 1L << 22;
+constexpr int kMaxGridY = 65535;  // tile units are the y axis of a direct launch
 
 // persistent 1-D grid: a multiple of the XCD count, no larger than the work bound
 constexpr int kMaxGrid = 2048;
@@ -115,14 +116,14 @@ TileArgs tile_args(const PlanView& pv) {
   return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
 }
 
-// grid of a launch: three-dimensional (tile unit, chunk row, projection) in direct mode,
+// grid of a launch: three-dimensional (chunk row, tile unit, projection) in direct mode,
 // else the persistent one-dimensional grid
 inline dim3 item_grid(const ItemSpace& sp, long items) {
   if (!sp.units_max) return work_grid(items);
   int rows = 1;
   for (int i = 0; i < sp.nproj; ++i)
     if (sp.row_start[i + 1] - sp.row_start[i] > rows) rows = sp.row_start[i + 1] - sp.row_start[i];
-  return dim3((unsigned)sp.units_max, (unsigned)rows, (unsigned)sp.nproj);
+  return dim3((unsigned)rows, (unsigned)sp.units_max, (unsigned)sp.nproj);
 }
 
 template <int DT, int MT, int NW, bool RM, bool DIRECT>
@@ -152,7 +153,7 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 1);
   const int units = tile_units_max(a.T, S, groups, MT);
   const long items = (long)units * a.items.row_start[a.items.nproj];
-  a.items.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;
+  a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
   const dim3 grid = item_grid(a.items, items);
   const bool f16 = dtype == SMLM_DTYPE_F16;
   if (a.items.units_max)
@@ -207,7 +208,7 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);
   const int units = tile_units_max(a.T, S, groups, block ? kBlkTiles : 1);
   const long items = (long)units * a.items.row_start[nproj];
-  a.items.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;
+  a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
   const dim3 grid = item_grid(a.items, items);
   const bool f16 = dtype == SMLM_DTYPE_F16;
   if (a.items.units_max)
@@ -282,6 +283,18 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   ra.beta = beta;
   ra.T = T; ra.d_out = d_out; ra.nproj = nproj;
   return launch_reduce(dtype, S, groups, st, ra);
+}
+
+template <int DT>
+int launch_wgrad(int nbj, bool split, dim3 grid, hipStream_t st, const WgradArgs& wa) {
+  if (split) {
+    if (nbj == 1) return launch(wgrad_kernel<DT, 1, 4>, grid, dim3(256), st, wa);
+    if (nbj == 2) return launch(wgrad_kernel<DT, 2, 4>, grid, dim3(256), st, wa);
+    return launch(wgrad_kernel<DT, 4, 4>, grid, dim3(256), st, wa);
+  }
+  if (nbj == 1) return launch(wgrad_kernel<DT, 1, 1>, grid, dim3(64), st, wa);
+  if (nbj == 2) return launch(wgrad_kernel<DT, 2, 1>, grid, dim3(64), st, wa);
+  return launch(wgrad_kernel<DT, 4, 1>, grid, dim3(64), st, wa);
 }
 
 struct BwdLayout {
@@ -656,14 +669,10 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   wa.chunks_a = ceil_div(h_in, kWgCols);
   dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA);
   const int nbj = ceil_div(r, 16);
-  if (dtype == SMLM_DTYPE_F16) {
-    if (nbj == 1) return launch(wgrad_kernel<SMLM_DTYPE_F16, 1>, grid, dim3(256), st, wa);
-    if (nbj == 2) return launch(wgrad_kernel<SMLM_DTYPE_F16, 2>, grid, dim3(256), st, wa);
-    return launch(wgrad_kernel<SMLM_DTYPE_F16, 4>, grid, dim3(256), st, wa);
-  }
-  if (nbj == 1) return launch(wgrad_kernel<SMLM_DTYPE_BF16, 1>, grid, dim3(256), st, wa);
-  if (nbj == 2) return launch(wgrad_kernel<SMLM_DTYPE_BF16, 2>, grid, dim3(256), st, wa);
-  return launch(wgrad_kernel<SMLM_DTYPE_BF16, 4>, grid, dim3(256), st, wa);
+  // four waves splitting the rows of an adapter pay off when adapters have many rows each
+  const bool split = n_rows / NA >= 256;
+  return dtype == SMLM_DTYPE_F16 ? launch_wgrad<SMLM_DTYPE_F16>(nbj, split, grid, st, wa)
+                                 : launch_wgrad<SMLM_DTYPE_BF16>(nbj, split, grid, st, wa);
 }
 
 }  // extern "C"

@@ -63,19 +63,45 @@ struct WgradArgs {
   int h_in, h_out, r, chunks_a;  // chunks_a = ceil(h_in/64): blockIdx.x below it works on dA
 };
 
-constexpr int kWgCols = 64;    // columns of x / dY per workgroup
-constexpr int kWgPitch = 72;   // LDS row pitch in 16-bit elements (144 B: 16-byte aligned rows)
+constexpr int kWgCols = 64;     // columns of x / dY per workgroup
+constexpr int kWgPitch = 80;    // LDS row pitch in 16-bit elements: 40 banks, so any eight
+                                // consecutive rows start 8 banks apart and tile the 64 banks
+constexpr int kWgSlots = 64;    // gathered rows (four tiles) per wave and loop step
 
-// grid: (ceil(h_in/64) + ceil(h_out/64), NA), block 256.  A workgroup owns 64
-// columns of one adapter's dA or dB and walks all of that adapter's tiles, 32
-// gathered rows (two tiles) per MFMA k step, the four waves taking k steps
-// round-robin; the waves' accumulators are then summed through LDS in wave
-// order.  The token dimension is the contraction, so the [token][column] block
-// of x / dY is staged in LDS and read back with the token index innermost.
-template <int DT, int NBJ>
-__global__ __launch_bounds__(256) void wgrad_kernel(WgradArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t stage[4][32 * kWgPitch];
-  __shared__ f32x4 red[4][4][kWaveSize];
+// Transposing LDS read of gfx950: within each 16 lanes, lane i names a "row" of
+// four 16-bit elements M[i][0..3]; lane 4a+b receives M[a][b], M[4+a][b],
+// M[8+a][b], M[12+a][b].
+typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 lds_tr_f16x4;
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_addr) {
+  typedef __attribute__((address_space(3))) lds_tr_f16x4 lds_vec;
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_vec*)lds_addr));
+}
+
+// LDS row of gathered-row slot s of a step: bits 2 and 3 of s change places, so
+// that the eight rows one half-wave reads together (slots 8g+4h+{0..3}, g = 0,1)
+// are consecutive and the read touches every bank once.
+__device__ __forceinline__ int wg_lds_row(int s) {
+  return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1);
+}
+
+// grid: (ceil(h_in/64) + ceil(h_out/64), NA), block 64*NW.  A workgroup owns 64
+// columns of one adapter's dA or dB and walks all of that adapter's tiles, 64
+// gathered rows (four tiles, two MFMA k steps) per wave and loop step.  With
+// NW = 4 (adapters with many rows each) the waves take steps round-robin and
+// their accumulators are summed through LDS in wave order; with NW = 1 (many
+// adapters with few rows each) a lone wave does it all and more workgroups fit
+// on a CU.  The token dimension is the contraction, so a wave stages its
+// [token][column] block of x / dY in its own part of LDS and reads it back
+// token-innermost with the transposing LDS read; no workgroup barrier is needed
+// inside the loop, and the rows of the next step are already on their way from
+// memory while the current step is multiplied.
+template <int DT, int NBJ, int NW>
+__global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
+  constexpr int kWgWaves = NW;
+  constexpr int kStageElems = kWgSlots * kWgPitch;
+  constexpr int kStageBytes = kWgWaves * kStageElems * 2;
+  constexpr int kRedBytes = NW > 1 ? kWgWaves * 4 * kWaveSize * 16 : 0;
+  __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
 
   const int ad = blockIdx.y;
   const bool is_a = (int)blockIdx.x < a.chunks_a;
@@ -90,20 +116,22 @@ __global__ __launch_bounds__(256) void wgrad_kernel(WgradArgs a) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
 
-  // group of this adapter: groups are sorted by id
-  const int NG = a.hdr[1];
-  int lo = 0, hi = NG;
-  while (lo < hi) {
-    const int mid = (lo + hi) >> 1;
-    if (a.grp_id[mid] < ad) lo = mid + 1; else hi = mid;
-  }
+  // group of this adapter (ids are distinct): every lane looks at one group
+  const int NG = uload(a.hdr, 1);
   int t_beg = 0, t_end = 0;
-  if (lo < NG && a.grp_id[lo] == ad) {
-    t_beg = a.grp_tile[lo];
-    t_end = a.grp_tile[lo + 1];
+  for (int base = 0; base < NG; base += kWaveSize) {
+    const int G = base + lane;
+    const bool hit = G < NG && a.grp_id[G] == ad;
+    const unsigned long long m = __ballot(hit);
+    if (m) {
+      const int Gh = base + __builtin_ctzll(m);
+      t_beg = uload(a.grp_tile, Gh);
+      t_end = uload(a.grp_tile, Gh + 1);
+      break;
+    }
   }
-  const int n_steps = (t_end - t_beg + 1) >> 1;
-  const int n_iter = (n_steps + 3) >> 2;  // same trip count for all four waves
+  constexpr int kStepTiles = kWgSlots / kTileRows;
+  const int n_steps = (t_end - t_beg + kStepTiles - 1) / kStepTiles;
 
   const u32x4 zero = {0u, 0u, 0u, 0u};
   f32x4 acc[NBJ][4];
@@ -112,67 +140,110 @@ __global__ __launch_bounds__(256) void wgrad_kernel(WgradArgs a) {
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) acc[jb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  uint16_t* st = stage[wave];
-  const int lrow = lane >> 3, lcol = (lane & 7) * 8;  // staging: 8 lanes cover 64 columns of a row
+  uint16_t* st = reinterpret_cast<uint16_t*>(smem) + wave * kStageElems;
+  // staging: load u of a lane brings 8 columns (lane & 7) of the slot whose LDS row is
+  // 8u + rlow; the two rows a 16-lane group writes together are 4 apart (32 banks)
+  const int q8 = lane >> 3, lcol = (lane & 7) * 8;
+  const int rlow = (q8 >> 1) + 4 * (q8 & 1);
+  const bool col_ok = n0 + lcol < h;
+  // transposed reads: lane i of a 16-lane group names row (8g + 4h + i/4) of the k step,
+  // columns 16nb + 4(i%4) .. +3
+  const int tr_row = wg_lds_row(8 * g + (c >> 2));  // + 4h -> LDS row + 8h; + 32 per k step
+  const int tr_col = 4 * (c & 3);
 
-  for (int it = 0; it < n_iter; ++it) {
-    const int step = it * 4 + wave;
-    const int tile0 = t_beg + 2 * step;
-    const bool live = step < n_steps;
-    // stage 32 gathered rows x 64 columns
+  auto load_rows = [&](int step, int32_t (&row)[8]) {
+    const int tile0 = t_beg + kStepTiles * step;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int sl = 8 * u + lrow;  // slot 0..31 of this k step
-      const int tile = tile0 + (sl >> 4);
-      u32x4 val = zero;
-      if (live && tile < t_end && n0 + lcol < h) {
-        const int row = a.tile_row[tile * kTileRows + (sl & 15)];
-        if (row >= 0) val = ldg16(Q + (long)row * h + n0 + lcol);
-      }
-      *reinterpret_cast<u32x4*>(st + sl * kWgPitch + lcol) = val;
+    for (int u = 0; u < 8; ++u) {
+      const int s = wg_lds_row(8 * u + rlow);  // the swap is its own inverse
+      const int tile = tile0 + (s >> 4);
+      row[u] = (step < n_steps && tile < t_end) ? a.tile_row[tile * kTileRows + (s & 15)] : -1;
     }
-    // token-side operand: PT[j][slot .. slot+7] for the 8 slots of lane group g
-    u32x4 pf[NBJ];
+  };
+  auto load_data = [&](const int32_t (&row)[8], u32x4 (&val)[8]) {
 #pragma unroll
-    for (int jb = 0; jb < NBJ; ++jb) {
-      const int j = 16 * jb + c;
-      const int tile = tile0 + (g >> 1);
-      pf[jb] = (live && tile < t_end && j < a.r)
-                   ? ldg16(PT + (long)j * a.pitch + (long)tile0 * kTileRows + 8 * g)
-                   : zero;
+    for (int u = 0; u < 8; ++u) {
+      const bool ok = row[u] >= 0 && col_ok;
+      val[u] = ldg16_if(Q + (long)(ok ? row[u] : 0) * h + n0 + lcol, ok, Q);
     }
-    __syncthreads();
+  };
+  auto load_p = [&](int step, u32x4 (&pf)[NBJ][2]) {
+    const int tile0 = t_beg + kStepTiles * step;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-      // column-side operand: Q[slot 8g..8g+7][n0 + 16nb + c], token index innermost
-      u32x4 qf;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t v0 = st[(8 * g + 2 * e) * kWgPitch + 16 * nb + c];
-        const uint32_t v1 = st[(8 * g + 2 * e + 1) * kWgPitch + 16 * nb + c];
-        qf[e] = v0 | (v1 << 16);
-      }
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
       for (int jb = 0; jb < NBJ; ++jb) {
-        // dA: rows = columns of x, cols = rank -> lane holds 4 consecutive x columns of rank c
-        // dB: rows = rank, cols = columns of dY -> lane holds 4 consecutive ranks of column c
-        acc[jb][nb] = is_a ? Num<DT>::mfma(qf, pf[jb], acc[jb][nb]) : Num<DT>::mfma(pf[jb], qf, acc[jb][nb]);
+        const int j = 16 * jb + c;
+        const int tile = tile0 + 2 * ks + (g >> 1);
+        const bool ok = step < n_steps && tile < t_end && j < a.r;
+        pf[jb][ks] = ldg16_if(PT + (long)(ok ? j : 0) * a.pitch + (long)(ok ? tile0 : 0) * kTileRows +
+                                  32 * ks + 8 * g, ok, PT);
       }
-    }
-    __syncthreads();
+  };
+
+  int32_t row_next[8];
+  u32x4 val[8], pf[NBJ][2];
+  load_rows(wave, row_next);
+  load_data(row_next, val);
+  load_p(wave, pf);
+  load_rows(wave + kWgWaves, row_next);
+
+  for (int step = wave; step < n_steps; step += kWgWaves) {
+    // the next step's rows and token-side operand start their way from memory now
+    u32x4 val_next[8], pf_next[NBJ][2];
+    load_data(row_next, val_next);
+    load_p(step + kWgWaves, pf_next);
+    load_rows(step + 2 * kWgWaves, row_next);
+
+#pragma unroll
+    for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4*>(st + (8 * u + rlow) * kWgPitch + lcol) = val[u];
+    // the wave's own LDS accesses are served in order; only the compiler must not move
+    // the reads above the writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+        // column-side operand: Q[slots 32ks + 8g .. +7][n0 + 16nb + c], token index innermost
+        const uint16_t* base = st + (32 * ks + tr_row) * kWgPitch + 16 * nb + tr_col;
+        const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 8 * kWgPitch);
+        const u32x4 qf = {q0[0], q0[1], q1[0], q1[1]};
+#pragma unroll
+        for (int jb = 0; jb < NBJ; ++jb) {
+          // dA: rows = columns of x, cols = rank -> lane holds 4 consecutive x columns of rank c
+          // dB: rows = rank, cols = columns of dY -> lane holds 4 consecutive ranks of column c
+          acc[jb][nb] = is_a ? Num<DT>::mfma(qf, pf[jb][ks], acc[jb][nb])
+                             : Num<DT>::mfma(pf[jb][ks], qf, acc[jb][nb]);
+        }
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < 8; ++u) val[u] = val_next[u];
+#pragma unroll
+    for (int jb = 0; jb < NBJ; ++jb) pf[jb][0] = pf_next[jb][0], pf[jb][1] = pf_next[jb][1];
   }
 
   // cross-wave sum in wave order, one rank block at a time, then store
+  f32x4(*red)[4][kWaveSize] = reinterpret_cast<f32x4(*)[4][kWaveSize]>(smem);
+  if (NW > 1) __syncthreads();  // every wave is done with its staging area, which red overlays
   for (int jb = 0; jb < NBJ; ++jb) {
+    if (NW > 1) {
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) red[wave][nb][lane] = acc[jb][nb];
-    __syncthreads();
+      for (int nb = 0; nb < 4; ++nb) red[wave][nb][lane] = acc[jb][nb];
+      __syncthreads();
+    }
     if (wave == 0) {
 #pragma unroll
       for (int nb = 0; nb < 4; ++nb) {
-        f32x4 s = red[0][nb][lane];
+        f32x4 s = acc[jb][nb];
+        if (NW > 1) {
+          s = red[0][nb][lane];
 #pragma unroll
-        for (int w = 1; w < 4; ++w) s += red[w][nb][lane];
+          for (int w = 1; w < kWgWaves; ++w) s += red[w][nb][lane];
+        }
         u32x2 o;
         o[0] = pack2<DT>(s[0], s[1]);
         o[1] = pack2<DT>(s[2], s[3]);
@@ -187,7 +258,7 @@ __global__ __launch_bounds__(256) void wgrad_kernel(WgradArgs a) {
         }
       }
     }
-    __syncthreads();
+    if (NW > 1) __syncthreads();
   }
 }
 

@@ -76,9 +76,14 @@ __device__ __forceinline__ void item_decode(const ItemSpace& sp, int V, int unit
   *pj = p;
   *yy = cr - sp.row_start[p];
 }
-// DIRECT launches are three-dimensional: x = tile unit, y = chunk row of the
-// projection, z = projection, so that the projection's arguments can be read
-// at once with the rest of the kernel arguments.
+// DIRECT launches are three-dimensional: x = chunk row of the projection, y =
+// tile unit, z = projection, so that the projection's arguments can be read at
+// once with the rest of the kernel arguments.  Chunk rows are the fast axis:
+// the workgroups in flight at one time then cover whole output rows of a few
+// tile units, which the memory system serves better than a few columns of all
+// rows.  (Re-indexing the plane so that the workgroups sharing a weight chunk
+// share an XCD's L2 was measured: it removes the repeated weight fetches and is
+// no faster, or much slower when it spreads the rows in flight.)
 template <bool DIRECT>
 __device__ __forceinline__ WorkRange item_range(const ItemSpace& sp, int units) {
   if (DIRECT) return WorkRange{0, 1, 1};
@@ -89,9 +94,9 @@ __device__ __forceinline__ bool item_get(const ItemSpace& sp, int V, int units, 
                                          int* tb) {
   if (DIRECT) {
     *pj = blockIdx.z;
-    *yy = blockIdx.y;
-    *tb = blockIdx.x;
-    return *yy < sp.row_start[*pj + 1] - sp.row_start[*pj];
+    *yy = blockIdx.x;
+    *tb = blockIdx.y;
+    return *tb < sp.units_max && *yy < sp.row_start[*pj + 1] - sp.row_start[*pj];
   }
   item_decode(sp, V, units, pj, yy, tb);
   return true;
