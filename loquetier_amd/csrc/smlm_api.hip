@@ -116,10 +116,11 @@ TileArgs tile_args(const PlanView& pv) {
   return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
 }
 
-// grid of a launch: three-dimensional (chunk row, tile unit, projection) in direct mode,
-// else the persistent one-dimensional grid
+// grid of a launch: (chunk row, tile unit, projection), or (chunk row over all projections,
+// tile unit) when flat, in direct mode; else the persistent one-dimensional grid
 inline dim3 item_grid(const ItemSpace& sp, long items) {
   if (!sp.units_max) return work_grid(items);
+  if (sp.flat) return dim3((unsigned)sp.row_start[sp.nproj], (unsigned)sp.units_max, 1u);
   int rows = 1;
   for (int i = 0; i < sp.nproj; ++i)
     if (sp.row_start[i + 1] - sp.row_start[i] > rows) rows = sp.row_start[i + 1] - sp.row_start[i];
@@ -185,6 +186,9 @@ int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipS
                      const ExpandArgs& a) {
   if (row_major)
     return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT>, grid, dim3(kFwdThreads), st, a);
+  if (block && nq == 8)
+    return KS == 1 ? launch(expand_block_kernel<DT, 8, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
+                   : launch(expand_block_kernel<DT, 8, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
   if (block)
     return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
                    : launch(expand_block_kernel<DT, 4, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
@@ -200,14 +204,21 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   if (row_major) nq = 2;
   if (block) nq = 4;
   nq = tune("SMLM_TUNE_NQ", nq);
-  if (block) nq = 4;
+  if (block && nq != 8) nq = 4;
   const int chunk = block ? 32 * nq : kFwdWaves * 32 * nq;  // columns per workgroup
   a.items.nproj = nproj;
+#ifdef SMLM_TUNING
+  a.dbg = tune("SMLM_TUNE_DBG", 0);
+#endif
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 0);
   a.items.row_start[0] = 0;
   for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);
   const int units = tile_units_max(a.T, S, groups, block ? kBlkTiles : 1);
   const long items = (long)units * a.items.row_start[nproj];
+  bool same_rows = true;
+  for (int i = 1; i < nproj; ++i)
+    same_rows = same_rows && (a.items.row_start[i + 1] - a.items.row_start[i] == a.items.row_start[1]);
+  a.items.flat = tune("SMLM_TUNE_FLAT", same_rows ? 0 : 1);
   a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
   const dim3 grid = item_grid(a.items, items);
   const bool f16 = dtype == SMLM_DTYPE_F16;

@@ -65,6 +65,7 @@ struct ItemSpace {
   int nproj;
   int interleave;  // plain round-robin items instead of one range per XCD
   int units_max;
+  int flat;        // direct mode: projections end to end along x instead of on z
 };
 __device__ __forceinline__ void item_decode(const ItemSpace& sp, int V, int units, int* pj, int* yy,
                                             int* tb) {
@@ -76,14 +77,16 @@ __device__ __forceinline__ void item_decode(const ItemSpace& sp, int V, int unit
   *pj = p;
   *yy = cr - sp.row_start[p];
 }
-// DIRECT launches are three-dimensional: x = chunk row of the projection, y =
-// tile unit, z = projection, so that the projection's arguments can be read at
-// once with the rest of the kernel arguments.  Chunk rows are the fast axis:
-// the workgroups in flight at one time then cover whole output rows of a few
-// tile units, which the memory system serves better than a few columns of all
-// rows.  (Re-indexing the plane so that the workgroups sharing a weight chunk
-// share an XCD's L2 was measured: it removes the repeated weight fetches and is
-// no faster, or much slower when it spreads the rows in flight.)
+// DIRECT launches put the chunk rows on x and the tile units on y.  Chunk rows
+// are the fast axis: the workgroups in flight at one time then cover whole
+// output rows of a few tile units, which the memory system serves better than a
+// few columns of all rows.  The projections are either the z axis (x then spans
+// the longest projection and shorter ones leave empty workgroups, but the
+// projection's arguments are known at once) or, with `flat`, laid end to end
+// along x (row_start; no empty workgroups -- better when the projections differ
+// much in width).  (Re-indexing the plane so that the workgroups sharing a
+// weight chunk share an XCD's L2 was measured: it removes the repeated weight
+// fetches and is no faster, or much slower when it spreads the rows in flight.)
 template <bool DIRECT>
 __device__ __forceinline__ WorkRange item_range(const ItemSpace& sp, int units) {
   if (DIRECT) return WorkRange{0, 1, 1};
@@ -92,11 +95,21 @@ __device__ __forceinline__ WorkRange item_range(const ItemSpace& sp, int units) 
 template <bool DIRECT>
 __device__ __forceinline__ bool item_get(const ItemSpace& sp, int V, int units, int* pj, int* yy,
                                          int* tb) {
-  if (DIRECT) {
+  if (DIRECT && !sp.flat) {
     *pj = blockIdx.z;
     *yy = blockIdx.x;
     *tb = blockIdx.y;
-    return *tb < sp.units_max && *yy < sp.row_start[*pj + 1] - sp.row_start[*pj];
+    return *yy < sp.row_start[*pj + 1] - sp.row_start[*pj];
+  }
+  if (DIRECT) {
+    const int cr = blockIdx.x;
+    int p = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxProj; ++i) p += (i < sp.nproj && cr >= sp.row_start[i]) ? 1 : 0;
+    *pj = p;
+    *yy = cr - sp.row_start[p];
+    *tb = blockIdx.y;
+    return true;
   }
   item_decode(sp, V, units, pj, yy, tb);
   return true;
@@ -350,6 +363,9 @@ struct ExpandArgs {
   float beta;
   int T, nt_max;
   ItemSpace items;           // chunk rows of projection p: its column chunks
+#ifdef SMLM_TUNING
+  int dbg;                   // experiments: 1 = no weights / multiply, 2 = no read of y
+#endif
 };
 
 // by-products one wave per tile writes while it holds the token fragment: the
@@ -504,15 +520,26 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
       const int idx = threadIdx.x + j * kFwdThreads;
       const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
       stage[j] = ldg16_if(W + (long)(ncol0 + nl) * P.ldw + k8,
-                          idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in, W);
+                          idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in
+#ifdef SMLM_TUNING
+                              && !(a.dbg & 1)
+#endif
+                          , W);
     }
     const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
     u32x4 yold[NQ];
     uint16_t* yrow = P.y + (long)(row < 0 ? 0 : row) * P.d_out + ncol0 + 8 * g;
-    if (a.beta != 0.0f) {
+    bool read_y = a.beta != 0.0f;
+#ifdef SMLM_TUNING
+    if (a.dbg & 2) read_y = false;
+#endif
+    if (read_y) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q)
         yold[q] = ldg16_if(yrow + 32 * q, row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, P.y);
+    } else {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) yold[q] = u32x4{0u, 0u, 0u, 0u};
     }
     u32x4 vf[KS];
 #pragma unroll
