@@ -76,11 +76,16 @@ struct ShrinkCfg {
   int NB, U, MT, NW, ksplit, k_per_wave, zblocks;
 };
 
+#ifndef SMLM_DECODE_SPLIT
+#define SMLM_DECODE_SPLIT 2
+#endif
+constexpr int kDecodeSplit = SMLM_DECODE_SPLIT;  // k halves of the sixteen-wave shrink
+constexpr int kMaxExpandFold = 4;  // most partials the expand kernel folds itself
+
 // waves per shrink workgroup, one choice for all projections of a launch: small
-// batches whose every projection has a long enough k use sixteen waves that
-// cover all of k, so nothing is left to fold afterwards
+// batches whose every projection has a long enough k use sixteen waves
 int shrink_waves(int T, int nproj, const int* d_in, int d_out) {
-  const int kq = 32 * (d_out > 32 ? 4 : 8);  // k per wave and load batch of the sixteen-wave kernels
+  const int kq = 32 * (d_out > 32 ? 2 : 4);  // k per wave and load batch of the sixteen-wave kernels
   bool all_long = tiles_per_wave(T) == 1;
   for (int i = 0; i < nproj; ++i) all_long = all_long && d_in[i] >= 16 * kq;
   return tune("SMLM_TUNE_NW", all_long ? 16 : kFwdWaves);
@@ -91,12 +96,23 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   c.zblocks = ceil_div(d_out, 64);
   const int cols = d_out >= 64 ? 64 : d_out;
   c.NB = cols <= 16 ? 1 : (cols <= 32 ? 2 : 4);
-  c.U = (c.NB == 4 ? 2 : 4) * (nw == 16 ? 2 : 1);  // one batch of loads covers a sixteenth of k
   c.MT = tiles_per_wave(T);
+  // 32-wide k steps per load batch; tile blocks hold four tiles of operands per batch and two
+  // batches at a time, so their batches are shorter
+  c.U = (c.NB == 4 ? 2 : 4) / (c.MT > 1 ? 2 : 1);
   const int kq = 32 * c.U;
   c.NW = nw;
   const int units = ceil_div(T > 0 ? T : 1, kTileRows * c.MT);
-  const int want = c.NW == 16 ? 1 : ceil_div(1024, units);
+  // k split over workgroups: enough of them to fill the chip, but every split writes and
+  // re-reads an fp32 partial of the output (8*r bytes a row against 2*d_in of input), so
+  // beyond 256 workgroups the split stops where the partials reach an eighth of the input.
+  // Sixteen-wave workgroups (decode batches: few tiles) split k in two, which doubles the
+  // number of CUs at work; the expand kernel adds the two halves.
+  int want = c.NW == 16 ? kDecodeSplit : ceil_div(1024, units);
+  const int cheap = d_in / (32 * d_out), fill = ceil_div(256, units);
+  const int cap = cheap > fill ? cheap : fill;
+  if (want > cap) want = cap;
+  want = tune("SMLM_TUNE_KSPLIT", want);
   int max_split = d_in / (c.NW * kq);
   if (max_split < 1) max_split = 1;
   if (max_split > 16) max_split = 16;
@@ -104,6 +120,12 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   c.k_per_wave = round_up(ceil_div(d_in, c.NW * ks), kq);
   c.ksplit = ceil_div(d_in, c.NW * c.k_per_wave);
   return c;
+}
+
+// most k-split partials a shrink of this shape can leave behind, whichever wave count it runs with
+int fwd_ksplit_bound(int T, int d_in, int d_out) {
+  const int a = shrink_cfg(T, d_in, d_out, kFwdWaves).ksplit, b = shrink_cfg(T, d_in, d_out, 16).ksplit;
+  return a > b ? a : b;
 }
 
 int expand_nq(int T, int d_out) {
@@ -130,10 +152,10 @@ inline dim3 item_grid(const ItemSpace& sp, long items) {
 template <int DT, int MT, int NW, bool RM, bool DIRECT>
 int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   const dim3 block(NW * kWaveSize);
-  constexpr int UF = NW == 16 ? 2 : 1;  // must match shrink_cfg
-  if (NB == 1) return launch(shrink_kernel<DT, 1, 4 * UF, MT, NW, RM, DIRECT>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_kernel<DT, 2, 4 * UF, MT, NW, RM, DIRECT>, grid, block, st, a);
-  return launch(shrink_kernel<DT, 4, 2 * UF, MT, NW, RM, DIRECT>, grid, block, st, a);
+  constexpr int UD = MT > 1 ? 2 : 1;  // must match shrink_cfg
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4 / UD, MT, NW, RM, DIRECT>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4 / UD, MT, NW, RM, DIRECT>, grid, block, st, a);
+  return launch(shrink_kernel<DT, 4, 2 / UD, MT, NW, RM, DIRECT>, grid, block, st, a);
 }
 
 template <int DT, bool DIRECT>
@@ -152,6 +174,9 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
                   ShrinkArgs& a) {
   const int MT = row_major ? 1 : c.MT;
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 1);
+#ifdef SMLM_TUNING
+  a.dbg = tune("SMLM_TUNE_SDBG", 0);
+#endif
   const int units = tile_units_max(a.T, S, groups, MT);
   const long items = (long)units * a.items.row_start[a.items.nproj];
   a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
@@ -254,10 +279,11 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 // shrink of one or more projections that share row routing and output width:
 // out[i] = beta*out[i] + scale * x[i] W_i^T in 16 bits, via k-split fp32 partial
 // sums folded by a second launch when the split is wider than one workgroup
+// (fold = false leaves the partials of split projections for the consumer to fold)
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
-               const float* seg_scale, hipStream_t st) {
+               const float* seg_scale, hipStream_t st, bool fold = true) {
   ShrinkArgs a{};
   a.plan = tile_args(pv);
   a.seg_scale = seg_scale;
@@ -288,7 +314,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   // and invalidates a whole L2 per workgroup on this multi-XCD part and cost 5-10x the launch
   // it saves.
   int rc = launch_shrink(dtype, row_major, c0, S, groups, st, a);
-  if (rc || !need_reduce) return rc;
+  if (rc || !need_reduce || !fold) return rc;
   ra.plan = a.plan;
   ra.seg_scale = seg_scale;
   ra.beta = beta;
@@ -324,7 +350,8 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
   };
   L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves);
   L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves);
-  const int ks = L.cfg_dv.ksplit > L.cfg_v.ksplit ? L.cfg_dv.ksplit : L.cfg_v.ksplit;
+  const int ks_dv = fwd_ksplit_bound(n_rows, h_out, r), ks_v = fwd_ksplit_bound(n_rows, h_in, r);
+  const int ks = ks_dv > ks_v ? ks_dv : ks_v;
   L.pitch = (long)plan_nt_max(n_rows, P) * kTileRows;
   L.at = take((size_t)NA * h_in * r * 2);
   L.bt = take((size_t)NA * h_out * r * 2);
@@ -390,9 +417,8 @@ SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t
   if (T > (1 << 30)) return SMLM_ERR_LIMIT;
   size_t n = 256;
   if (d_in >= d_out) {
-    // sized for the four-wave split, which never needs less than the sixteen-wave one
-    const ShrinkCfg c = shrink_cfg(T, d_in, d_out, kFwdWaves);
-    if (c.ksplit > 1) n = align_up((size_t)c.ksplit * T * d_out * 4, 256);
+    const int ks = fwd_ksplit_bound(T, d_in, d_out);
+    if (ks > 1) n = align_up((size_t)ks * T * d_out * 4, 256);
   }
   *bytes = n;
   return SMLM_OK;
@@ -482,9 +508,8 @@ SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_
   size_t n = 0;
   for (int i = 0; i < n_proj; ++i) {
     if (h_in[i] <= 0) return SMLM_ERR_ARG;
-    const ShrinkCfg c = shrink_cfg(T, h_in[i], r, kFwdWaves);
     const size_t rows = T > 0 ? T : 1;
-    n += align_up((size_t)c.ksplit * rows * r * 4, 256) + align_up(rows * r * 2, 256);
+    n += align_up((size_t)fwd_ksplit_bound(T, h_in[i], r) * rows * r * 4, 256) + align_up(rows * r * 2, 256);
   }
   *bytes = n;
   return SMLM_OK;
@@ -525,22 +550,28 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
   PlanView pv;
   plan_carve(const_cast<void*>(plan), T, S, &pv);
 
-  // shrink: every projection's v, rounded to 16 bits (into v_out when the caller wants it)
+  // shrink: every projection's v, rounded to 16 bits (into v_out when the caller wants it).
+  // Decode batches (sixteen-wave shrink, one-tile expand) skip the fold launch: the expand
+  // kernel adds the few partials while it loads v.
   float* partial[kMaxProj];
   void* v16[kMaxProj];
+  int vsplit[kMaxProj];
+  const int nw = shrink_waves(T, n_proj, h_in, r);
+  bool expand_folds = nw == 16 && tiles_per_wave(T) == 1;
   {
     char* w = reinterpret_cast<char*>(workspace);
     for (int i = 0; i < n_proj; ++i) {
-      const ShrinkCfg c = shrink_cfg(T, h_in[i], r, kFwdWaves);
+      vsplit[i] = shrink_cfg(T, h_in[i], r, nw).ksplit;
+      expand_folds = expand_folds && vsplit[i] <= kMaxExpandFold;
       partial[i] = reinterpret_cast<float*>(w);
-      w += align_up((size_t)c.ksplit * T * r * 4, 256);
+      w += align_up((size_t)fwd_ksplit_bound(T, h_in[i], r) * T * r * 4, 256);
       v16[i] = (v_out && v_out[i]) ? v_out[i] : w;
       w += align_up((size_t)T * r * 2, 256);
     }
   }
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                    0.0f, nullptr, st);
+                    0.0f, nullptr, st, !expand_folds);
     if (rc) return rc;
   }
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;
@@ -556,6 +587,12 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
     P.v = reinterpret_cast<const uint16_t*>(v16[i]);
     P.w_ptrs = b_ptrs[i];
     P.d_in = r; P.d_out = h_out[i]; P.ldw = r;
+    if (expand_folds && vsplit[i] > 1) {
+      P.vpart = partial[i];
+      P.vsplit = vsplit[i];
+      // the rounded v exists only inside the expand kernel: it writes the caller's copy
+      if (v_out && v_out[i]) P.v_out = reinterpret_cast<uint16_t*>(v_out[i]);
+    }
   }
   return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, n_weights, n_proj, r,
                        st, ea);

@@ -95,16 +95,14 @@ __device__ __forceinline__ int wg_lds_row(int s) {
 // token-innermost with the transposing LDS read; no workgroup barrier is needed
 // inside the loop, and the rows of the next step are already on their way from
 // memory while the current step is multiplied.
-template <int DT, int NBJ, int NW>
-__global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
+template <int DT, int NBJ, int NW, bool IS_A>
+__device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   constexpr int kWgWaves = NW;
   constexpr int kStageElems = kWgSlots * kWgPitch;
   constexpr int kStageBytes = kWgWaves * kStageElems * 2;
-  constexpr int kRedBytes = NW > 1 ? kWgWaves * 4 * kWaveSize * 16 : 0;
-  __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
 
   const int ad = blockIdx.y;
-  const bool is_a = (int)blockIdx.x < a.chunks_a;
+  constexpr bool is_a = IS_A;
   const int n0 = (is_a ? blockIdx.x : blockIdx.x - a.chunks_a) * kWgCols;
   const int h = is_a ? a.h_in : a.h_out;
   const uint16_t* Q = is_a ? a.q_a : a.q_b;
@@ -133,7 +131,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
   constexpr int kStepTiles = kWgSlots / kTileRows;
   const int n_steps = (t_end - t_beg + kStepTiles - 1) / kStepTiles;
 
-  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.hdr + kHdrZeros);
   f32x4 acc[NBJ][4];
 #pragma unroll
   for (int jb = 0; jb < NBJ; ++jb)
@@ -164,7 +162,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const bool ok = row[u] >= 0 && col_ok;
-      val[u] = ldg16_if(Q + (long)(ok ? row[u] : 0) * h + n0 + lcol, ok, Q);
+      val[u] = ldg16_or(Q + (long)row[u] * h + n0 + lcol, ok, zeros);
     }
   };
   auto load_p = [&](int step, u32x4 (&pf)[NBJ][2]) {
@@ -176,8 +174,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
         const int j = 16 * jb + c;
         const int tile = tile0 + 2 * ks + (g >> 1);
         const bool ok = step < n_steps && tile < t_end && j < a.r;
-        pf[jb][ks] = ldg16_if(PT + (long)(ok ? j : 0) * a.pitch + (long)(ok ? tile0 : 0) * kTileRows +
-                                  32 * ks + 8 * g, ok, PT);
+        pf[jb][ks] = ldg16_or(PT + (long)j * a.pitch + (long)tile0 * kTileRows + 32 * ks + 8 * g, ok, zeros);
       }
   };
 
@@ -202,22 +199,28 @@ __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // column-side operands: Q[slots 32ks + 8g .. +7][n0 + 16nb + c], token index innermost;
+    // all sixteen reads are issued before the first multiply waits for them
+    u32x4 qf[2][4];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
       for (int nb = 0; nb < 4; ++nb) {
-        // column-side operand: Q[slots 32ks + 8g .. +7][n0 + 16nb + c], token index innermost
         const uint16_t* base = st + (32 * ks + tr_row) * kWgPitch + 16 * nb + tr_col;
         const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 8 * kWgPitch);
-        const u32x4 qf = {q0[0], q0[1], q1[0], q1[1]};
+        qf[ks][nb] = u32x4{q0[0], q0[1], q1[0], q1[1]};
+      }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
         for (int jb = 0; jb < NBJ; ++jb) {
           // dA: rows = columns of x, cols = rank -> lane holds 4 consecutive x columns of rank c
           // dB: rows = rank, cols = columns of dY -> lane holds 4 consecutive ranks of column c
-          acc[jb][nb] = is_a ? Num<DT>::mfma(qf, pf[jb][ks], acc[jb][nb])
-                             : Num<DT>::mfma(pf[jb][ks], qf, acc[jb][nb]);
+          acc[jb][nb] = is_a ? Num<DT>::mfma(qf[ks][nb], pf[jb][ks], acc[jb][nb])
+                             : Num<DT>::mfma(pf[jb][ks], qf[ks][nb], acc[jb][nb]);
         }
-      }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -260,6 +263,17 @@ __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
     }
     if (NW > 1) __syncthreads();
   }
+}
+
+template <int DT, int NBJ, int NW>
+__global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
+  constexpr int kStageBytes = NW * kWgSlots * kWgPitch * 2;
+  constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
+  __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+  if ((int)blockIdx.x < a.chunks_a)  // uniform over the workgroup
+    wgrad_body<DT, NBJ, NW, true>(a, smem);
+  else
+    wgrad_body<DT, NBJ, NW, false>(a, smem);
 }
 
 }  // namespace smlm

@@ -94,6 +94,14 @@ __device__ __forceinline__ u32x4 ldg16_if(const uint16_t* p, bool ok, const uint
   return ok ? v : zero;
 }
 
+// 16 bytes from p when ok, else from `zeros` (16 zero bytes in device memory: a
+// plan header carries them).  Unlike ldg16_if nothing is done to the value after
+// the load, so the wave need not wait for it before it goes on issuing loads.
+__device__ __forceinline__ u32x4 ldg16_or(const uint16_t* p, bool ok, const uint16_t* zeros) {
+  return ldg16(ok ? p : zeros);
+}
+constexpr int kHdrZeros = 12;  // header words 12..15 are always zero
+
 // Reads of plan tables and pointer tables at a wave-uniform index.  These are
 // written by an earlier kernel and never by the kernel that reads them, so they
 // may go through the scalar (constant) path: the loads then cost no vector
@@ -126,7 +134,8 @@ __device__ __forceinline__ u32x4 ldg_strided8(const uint16_t* p, long stride) {
 
 // Views into a plan buffer (all int32).  Sizes are functions of (T, S) only.
 struct PlanView {
-  int32_t* hdr;         // [16]: 0 n_tiles, 1 n_groups, 2 rows covered, 3 key kind used, 4 n_blocks
+  int32_t* hdr;         // [16]: 0 n_tiles, 1 n_groups, 2 rows covered, 3 key kind used, 4 n_blocks,
+                        //       12..15 zero (16 zero bytes for predicated-off loads to read)
   int32_t* sorted_seg;  // [S]   segment at sorted position p
   int32_t* rowpos;      // [S+1] first gathered-row index of sorted position p
   int32_t* grp_tile;    // [S+1] first tile of group G (exclusive scan), [NG] = n_tiles

@@ -139,12 +139,13 @@ __device__ __forceinline__ void pick_tiles(const TileArgs& p, int tb, int* t0, i
 
 // eight consecutive-k elements of weight column n (zeros when !ok)
 template <bool ROWMAJOR>
-__device__ __forceinline__ u32x4 load_w8(const uint16_t* W, int n, int k, int ldw, bool ok) {
+__device__ __forceinline__ u32x4 load_w8(const uint16_t* W, int n, int k, int ldw, bool ok,
+                                         const uint16_t* zeros) {
   if (ROWMAJOR) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
     return ok ? ldg_strided8(W + (long)k * ldw + n, ldw) : zero;
   }
-  return ldg16_if(W + (long)n * ldw + k, ok, W);
+  return ldg16_or(W + (long)n * ldw + k, ok, zeros);
 }
 
 // out = beta*old + scale*acc for four consecutive columns of one row
@@ -178,6 +179,9 @@ struct ShrinkArgs {
   float beta;
   int T;
   ItemSpace items;            // chunk rows of projection p: ksplit*zblocks
+#ifdef SMLM_TUNING
+  int dbg;                    // experiments: 1 = no weight loads, 2 = no x loads, 4 = no partial/output store
+#endif
 };
 
 // Work item -> (projection, k slice, 64-column block, tile block).  The NW
@@ -222,6 +226,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 
     const int kbeg = (kz * NW + wave) * P.k_per_wave;
     const int kend = min(kbeg + P.k_per_wave, P.d_in);
+    const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
 
     f32x4 acc[MT][NB];
 #pragma unroll
@@ -229,22 +234,32 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) acc[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-#pragma unroll 1
-    for (int k = kbeg; k < kend; k += 32 * U) {
-      u32x4 xf[MT][U], wf[NB][U];
+    // k loop, two load batches in turn: the loads of one batch are on their way while the
+    // other batch is multiplied
+    auto load_batch = [&](int k, u32x4 (&xf)[MT][U], u32x4 (&wf)[NB][U]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int kk = k + 32 * u + 8 * g;
         const bool kin = kk < kend;
 #pragma unroll
         for (int i = 0; i < MT; ++i)
-          xf[i][u] = ldg16_if(P.x + (long)row[i] * P.d_in + kk, kin && row[i] >= 0, P.x);
+          xf[i][u] = ldg16_or(P.x + (long)row[i] * P.d_in + kk, kin && row[i] >= 0
+#ifdef SMLM_TUNING
+                                                                         && !(a.dbg & 2)
+#endif
+                              , zeros);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const int n = n0 + 16 * nb + c;
-          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out);
+          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out
+#ifdef SMLM_TUNING
+                                                             && !(a.dbg & 1)
+#endif
+                                        , zeros);
         }
       }
+    };
+    auto multiply = [&](const u32x4 (&xf)[MT][U], const u32x4 (&wf)[NB][U]) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -253,6 +268,26 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) acc[i][nb] = Num<DT>::mfma(wf[nb][u], xf[i][u], acc[i][nb]);
           }
+    };
+    if (NW < 16) {
+      u32x4 xa[MT][U], wa[NB][U], xb[MT][U], wb[NB][U];
+      load_batch(kbeg, xa, wa);
+#pragma unroll 1
+      for (int k = kbeg; k < kend; k += 64 * U) {
+        const bool more = k + 32 * U < kend;  // uniform over the wave
+        if (more) load_batch(k + 32 * U, xb, wb);
+        multiply(xa, wa);
+        if (!more) break;
+        if (k + 64 * U < kend) load_batch(k + 64 * U, xa, wa);
+        multiply(xb, wb);
+      }
+    } else {  // sixteen waves share the VGPR file: one batch at a time (k is usually one batch)
+#pragma unroll 1
+      for (int k = kbeg; k < kend; k += 32 * U) {
+        u32x4 xf[MT][U], wf[NB][U];
+        load_batch(k, xf, wf);
+        multiply(xf, wf);
+      }
     }
 
 #ifdef SMLM_TUNING
@@ -279,11 +314,21 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
           if (P.ksplit == 1 && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
-            f32x4 sum = red[0][wave][nb][lane];
+            // all NW reads are issued before the first add waits for one (left to itself the
+            // compiler keeps two in flight, and the sixteen-wave kernel spends as long here
+            // as in its k loop)
+            f32x4 part[NW];
 #pragma unroll
-            for (int w = 1; w < NW; ++w) sum += red[w][wave][nb][lane];
+            for (int w = 0; w < NW; ++w) part[w] = red[w][wave][nb][lane];
+            __builtin_amdgcn_sched_barrier(0);
+            f32x4 sum = part[0];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) sum += part[w];
             const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
             if (n >= P.d_out) continue;
+#ifdef SMLM_TUNING
+            if ((a.dbg & 4) && sum[0] != 12345.f) continue;
+#endif
             if (P.ksplit > 1)
               *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + r) * P.d_out + n) = sum;
             else
@@ -350,6 +395,8 @@ struct ExpandProj {
   const uint16_t* v;          // [T, d_in]
   const void* const* w_ptrs;  // indexed by the plan's tile_wid
   uint16_t* v_out;            // optional [T, d_in]: copy of v, by row
+  const float* vpart;         // vsplit > 1: v arrives as fp32 k-split partials [vsplit, T, d_in]
+  int vsplit;                 //   (wave kernel only), summed here in split order and rounded
   int d_in, d_out, ldw;
 };
 
@@ -470,9 +517,26 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           const int n = ncol0 + 32 * q + 4 * p + mrow;
-          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out);
+          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out,
+                                       reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros));
         }
-      const u32x4 vf = ldg16_if(P.v + (long)row * P.d_in + kk, kin && row >= 0, P.v);
+      u32x4 vf;
+      if (P.vsplit > 1) {  // uniform: fold the shrink's partial sums as its fold launch would
+        const bool ok = kin && row >= 0;
+        const float* pz = P.vpart + (long)(ok ? row : 0) * P.d_in + (ok ? kk : 0);
+        f32x4 s0 = ldg_f4(pz), s1 = ldg_f4(pz + 4);
+        for (int z = 1; z < P.vsplit; ++z) {
+          pz += (long)a.T * P.d_in;
+          s0 += ldg_f4(pz);
+          s1 += ldg_f4(pz + 4);
+        }
+        const u32x4 packed = {pack2<DT>(s0[0], s0[1]), pack2<DT>(s0[2], s0[3]), pack2<DT>(s1[0], s1[1]),
+                              pack2<DT>(s1[2], s1[3])};
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        vf = ok ? packed : zero;
+      } else {
+        vf = ldg16_if(P.v + (long)row * P.d_in + kk, kin && row >= 0, P.v);
+      }
       if (side && kin) write_side<DT>(a, P, slot, row, kk, vf, scale);
 #pragma unroll
       for (int q = 0; q < NQ; ++q)

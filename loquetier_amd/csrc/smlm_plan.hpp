@@ -266,6 +266,8 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     pv.hdr[2] = rows_total;
     pv.hdr[3] = kind;
     pv.hdr[4] = n_blocks;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pv.hdr[kHdrZeros + i] = 0;
   }
   __syncthreads();
 
@@ -377,6 +379,8 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
     pv.hdr[1] = NG;
     pv.hdr[2] = rows_total;
     pv.hdr[3] = kind;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pv.hdr[kHdrZeros + i] = 0;
   }
   __syncthreads();
 
