@@ -80,7 +80,7 @@ struct ShrinkCfg {
 #define SMLM_DECODE_SPLIT 2
 #endif
 constexpr int kDecodeSplit = SMLM_DECODE_SPLIT;  // k halves of the sixteen-wave shrink
-constexpr int kMaxExpandFold = 4;  // most partials the expand kernel folds itself
+constexpr int kMaxExpandFold = kMaxVsplit;  // most partials the expand kernel folds itself
 
 // waves per shrink workgroup, one choice for all projections of a launch: small
 // batches whose every projection has a long enough k use sixteen waves
@@ -199,26 +199,32 @@ int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
 }
 
 template <int DT, int NQ, bool DIRECT>
-int launch_expand_wave(int KS, dim3 grid, hipStream_t st, const ExpandArgs& a) {
+int launch_expand_wave(int KS, bool vfold, dim3 grid, hipStream_t st, const ExpandArgs& a) {
   const dim3 block(kFwdThreads);
-  if (KS == 1) return launch(expand_wave_kernel<DT, NQ, 1, false, DIRECT>, grid, block, st, a);
-  if (KS == 2) return launch(expand_wave_kernel<DT, NQ, 2, false, DIRECT>, grid, block, st, a);
-  return launch(expand_wave_kernel<DT, NQ, 0, false, DIRECT>, grid, block, st, a);
+  if (vfold) {
+    if (KS == 1) return launch(expand_wave_kernel<DT, NQ, 1, false, DIRECT, true>, grid, block, st, a);
+    if (KS == 2) return launch(expand_wave_kernel<DT, NQ, 2, false, DIRECT, true>, grid, block, st, a);
+    return launch(expand_wave_kernel<DT, NQ, 0, false, DIRECT, true>, grid, block, st, a);
+  }
+  if (KS == 1) return launch(expand_wave_kernel<DT, NQ, 1, false, DIRECT, false>, grid, block, st, a);
+  if (KS == 2) return launch(expand_wave_kernel<DT, NQ, 2, false, DIRECT, false>, grid, block, st, a);
+  return launch(expand_wave_kernel<DT, NQ, 0, false, DIRECT, false>, grid, block, st, a);
 }
 
 template <int DT, bool DIRECT>
 int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipStream_t st,
                      const ExpandArgs& a) {
   if (row_major)
-    return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT>, grid, dim3(kFwdThreads), st, a);
+    return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
   if (block && nq == 8)
     return KS == 1 ? launch(expand_block_kernel<DT, 8, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
                    : launch(expand_block_kernel<DT, 8, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
   if (block)
     return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
                    : launch(expand_block_kernel<DT, 4, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
-  return nq == 4 ? launch_expand_wave<DT, 4, DIRECT>(KS, grid, st, a)
-                 : launch_expand_wave<DT, 2, DIRECT>(KS, grid, st, a);
+  const bool vfold = a.p[0].vsplit > 0;  // set for all projections of a launch or for none
+  return nq == 4 ? launch_expand_wave<DT, 4, DIRECT>(KS, vfold, grid, st, a)
+                 : launch_expand_wave<DT, 2, DIRECT>(KS, vfold, grid, st, a);
 }
 
 // all projections of one launch share the rank (d_in); d_out may differ
@@ -279,7 +285,7 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 // shrink of one or more projections that share row routing and output width:
 // out[i] = beta*out[i] + scale * x[i] W_i^T in 16 bits, via k-split fp32 partial
 // sums folded by a second launch when the split is wider than one workgroup
-// (fold = false leaves the partials of split projections for the consumer to fold)
+// (fold = false leaves every projection's fp32 partials, one or more, for the consumer to fold)
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
@@ -305,6 +311,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
     P.out = reinterpret_cast<uint16_t*>(out[i]);
     P.d_in = d_in[i]; P.d_out = d_out; P.ldw = ldw[i];
     P.k_per_wave = c.k_per_wave; P.ksplit = c.ksplit; P.zblocks = c.zblocks;
+    P.to_partial = fold ? 0 : 1;
     a.items.row_start[i + 1] = a.items.row_start[i] + c.ksplit * c.zblocks;
     ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit};
     need_reduce = need_reduce || c.ksplit > 1;
@@ -587,7 +594,7 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
     P.v = reinterpret_cast<const uint16_t*>(v16[i]);
     P.w_ptrs = b_ptrs[i];
     P.d_in = r; P.d_out = h_out[i]; P.ldw = r;
-    if (expand_folds && vsplit[i] > 1) {
+    if (expand_folds) {
       P.vpart = partial[i];
       P.vsplit = vsplit[i];
       // the rounded v exists only inside the expand kernel: it writes the caller's copy

@@ -170,6 +170,7 @@ struct ShrinkProj {
   float* partial;             // [ksplit, T, d_out] fp32 when ksplit > 1
   uint16_t* out;              // [T, d_out] when ksplit == 1
   int d_in, d_out, ldw, k_per_wave, ksplit, zblocks;
+  int to_partial;             // write the fp32 partial even when ksplit == 1 (the consumer rounds)
 };
 
 struct ShrinkArgs {
@@ -311,7 +312,8 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         for (int j = 1; j < MT; ++j) r = (i == j) ? row[j] : r;
         if (r >= 0) {
           float scale = 1.0f;
-          if (P.ksplit == 1 && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
+          const bool as_partial = P.ksplit > 1 || P.to_partial;
+          if (!as_partial && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
             // all NW reads are issued before the first add waits for one (left to itself the
@@ -329,7 +331,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #ifdef SMLM_TUNING
             if ((a.dbg & 4) && sum[0] != 12345.f) continue;
 #endif
-            if (P.ksplit > 1)
+            if (as_partial)
               *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + r) * P.d_out + n) = sum;
             else
               store4<DT>(P.out + (long)r * P.d_out + n, sum, scale, a.beta);
@@ -395,10 +397,12 @@ struct ExpandProj {
   const uint16_t* v;          // [T, d_in]
   const void* const* w_ptrs;  // indexed by the plan's tile_wid
   uint16_t* v_out;            // optional [T, d_in]: copy of v, by row
-  const float* vpart;         // vsplit > 1: v arrives as fp32 k-split partials [vsplit, T, d_in]
-  int vsplit;                 //   (wave kernel only), summed here in split order and rounded
+  const float* vpart;         // VFOLD wave kernels: v arrives as vsplit (1..4) fp32 k-split partials
+  int vsplit;                 //   [vsplit, T, d_in], summed here in split order and rounded
   int d_in, d_out, ldw;
 };
+
+constexpr int kMaxVsplit = 4;  // most k-split partials of v the wave kernel folds itself
 
 struct ExpandArgs {
   TileArgs plan;
@@ -470,7 +474,7 @@ __device__ __forceinline__ void store_tile(uint16_t* yrow, int ncol, int d_out, 
 // short: KS > 0 unrolls KS 32-wide k steps, KS == 0 is the general loop over k.
 // MFMA row m of column block (q,p) is output column 32q + 8(m/4) + 4p + m%4, so
 // that a lane's eight accumulators for one q are eight consecutive columns.
-template <int DT, int NQ, int KS, bool ROWMAJOR, bool DIRECT>
+template <int DT, int NQ, int KS, bool ROWMAJOR, bool DIRECT, bool VFOLD>
 __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) {
   const int units = DIRECT ? 0 : tile_units<1>(a.plan, 0);
   const WorkRange wr = item_range<DIRECT>(a.items, units);
@@ -490,17 +494,22 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
-    const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
+    const int rseg = a.seg_scale ? a.plan.tile_rseg[slot] : -1;  // -1 on empty slots too
     const bool side = (yy == 0 && wave == 0);  // the one wave per tile that writes by-products
+    const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
 
-    // y rows this lane will update: fetch the old values early
+    // Every load of the item is issued before anything waits for one: the old values of the
+    // y rows this lane will update, the weight fragments and v (predicated-off loads read
+    // zeros instead of being patched afterwards, which would make the wave wait in between).
     u32x4 yold[NQ];
     uint16_t* yrow = P.y + (long)(row < 0 ? 0 : row) * P.d_out + ncol0 + 8 * g;
     if (a.beta != 0.0f) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q)
-        yold[q] = ldg16_if(yrow + 32 * q, row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, P.y);
+        yold[q] = ldg16_or(yrow + 32 * q, row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, zeros);
     }
+
+    const float scale = rseg >= 0 ? a.seg_scale[rseg] : 1.0f;  // rseg came with row: no extra wait
 
     f32x4 acc[NQ][2];
 #pragma unroll
@@ -517,25 +526,27 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           const int n = ncol0 + 32 * q + 4 * p + mrow;
-          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out,
-                                       reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros));
+          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out, zeros);
         }
       u32x4 vf;
-      if (P.vsplit > 1) {  // uniform: fold the shrink's partial sums as its fold launch would
-        const bool ok = kin && row >= 0;
-        const float* pz = P.vpart + (long)(ok ? row : 0) * P.d_in + (ok ? kk : 0);
-        f32x4 s0 = ldg_f4(pz), s1 = ldg_f4(pz + 4);
-        for (int z = 1; z < P.vsplit; ++z) {
-          pz += (long)a.T * P.d_in;
-          s0 += ldg_f4(pz);
-          s1 += ldg_f4(pz + 4);
+      const bool vok = kin && row >= 0;
+      if (VFOLD) {  // fold (and round) the shrink's fp32 partial sums as its fold launch would
+        const float* zf = reinterpret_cast<const float*>(zeros);
+        f32x4 part[kMaxVsplit][2];
+#pragma unroll
+        for (int z = 0; z < kMaxVsplit; ++z) {
+          const bool ok = vok && z < P.vsplit;
+          const float* pz = ok ? P.vpart + ((long)z * a.T + row) * P.d_in + kk : zf;
+          part[z][0] = ldg_f4(pz);
+          part[z][1] = ldg_f4(ok ? pz + 4 : zf);
         }
-        const u32x4 packed = {pack2<DT>(s0[0], s0[1]), pack2<DT>(s0[2], s0[3]), pack2<DT>(s1[0], s1[1]),
-                              pack2<DT>(s1[2], s1[3])};
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        vf = ok ? packed : zero;
+        f32x4 s0 = part[0][0], s1 = part[0][1];
+#pragma unroll
+        for (int z = 1; z < kMaxVsplit; ++z) s0 += part[z][0], s1 += part[z][1];  // + 0.0 past vsplit
+        vf = u32x4{pack2<DT>(s0[0], s0[1]), pack2<DT>(s0[2], s0[3]), pack2<DT>(s1[0], s1[1]),
+                   pack2<DT>(s1[2], s1[3])};
       } else {
-        vf = ldg16_if(P.v + (long)row * P.d_in + kk, kin && row >= 0, P.v);
+        vf = ldg16_or(P.v + (long)row * P.d_in + kk, vok, zeros);
       }
       if (side && kin) write_side<DT>(a, P, slot, row, kk, vf, scale);
 #pragma unroll
@@ -574,7 +585,11 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
     const bool active = wave < cnt;
     const int slot = (t0 + (active ? wave : 0)) * kTileRows + c;
     const int row = active ? a.plan.tile_row[slot] : -1;
+    const int rseg = (a.seg_scale && active) ? a.plan.tile_rseg[slot] : -1;  // -1 on empty slots too
+    const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
 
+    // Every load of the item is issued before anything waits for one (predicated-off loads
+    // read zeros instead of being patched afterwards).
     // weight chunk -> registers (written to LDS below): 32*NQ rows of 4*KS 16-byte pieces
     constexpr int kPieces = 32 * NQ * 4 * KS;
     constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
@@ -583,34 +598,35 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
     for (int j = 0; j < kPer; ++j) {
       const int idx = threadIdx.x + j * kFwdThreads;
       const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
-      stage[j] = ldg16_if(W + (long)(ncol0 + nl) * P.ldw + k8,
+      stage[j] = ldg16_or(W + (long)(ncol0 + nl) * P.ldw + k8,
                           idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in
 #ifdef SMLM_TUNING
                               && !(a.dbg & 1)
 #endif
-                          , W);
+                          , zeros);
     }
-    const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
     u32x4 yold[NQ];
     uint16_t* yrow = P.y + (long)(row < 0 ? 0 : row) * P.d_out + ncol0 + 8 * g;
     bool read_y = a.beta != 0.0f;
 #ifdef SMLM_TUNING
     if (a.dbg & 2) read_y = false;
 #endif
-    if (read_y) {
 #pragma unroll
-      for (int q = 0; q < NQ; ++q)
-        yold[q] = ldg16_if(yrow + 32 * q, row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, P.y);
-    } else {
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) yold[q] = u32x4{0u, 0u, 0u, 0u};
-    }
+    for (int q = 0; q < NQ; ++q)
+      yold[q] = ldg16_or(yrow + 32 * q, read_y && row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, zeros);
     u32x4 vf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int kk = 32 * ks + 8 * g;
-      vf[ks] = ldg16_if(P.v + (long)row * P.d_in + kk, kk < P.d_in && row >= 0, P.v);
-      if (yy == 0 && active && kk < P.d_in) write_side<DT>(a, P, slot, row, kk, vf[ks], scale);
+      vf[ks] = ldg16_or(P.v + (long)row * P.d_in + kk, kk < P.d_in && row >= 0, zeros);
+    }
+    const float scale = (rseg >= 0 && row >= 0) ? a.seg_scale[rseg] : 1.0f;
+    if (yy == 0 && active) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int kk = 32 * ks + 8 * g;
+        if (kk < P.d_in) write_side<DT>(a, P, slot, row, kk, vf[ks], scale);
+      }
     }
 
     __syncthreads();  // every wave is done reading the previous item's weights
