@@ -129,9 +129,10 @@ int fwd_ksplit_bound(int T, int d_in, int d_out) {
 }
 
 int expand_nq(int T, int d_out) {
-  if (tiles_per_wave(T) > 1) return 4;  // block kernel: a 128-column chunk per workgroup
-  const int units = ceil_div(T > 0 ? T : 1, kTileRows);
-  return ((long)units * ceil_div(d_out, 512) >= 512) ? 4 : 2;
+  (void)T;
+  // 32-column blocks per wave: four (a workgroup then covers 512 columns) unless the
+  // projection is narrower than that
+  return d_out >= 512 ? 4 : 2;
 }
 
 TileArgs tile_args(const PlanView& pv) {

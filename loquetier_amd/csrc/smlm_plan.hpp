@@ -19,6 +19,7 @@ constexpr int kPlanThreads = 1024;
 constexpr int kPlanLdsKeys = 4096;   // two-launch route: sorts up to this many keys stay in LDS
 constexpr int kPlanSmallSegs = 1024; // one-launch route: at most this many segments ...
 constexpr int kPlanSmallTiles = 4096; // ... and at most this many possible tiles
+constexpr int kNarrowIdBits = 21;     // ids below 2^21 and 10 bits of segment index make a 32-bit key
 
 struct PlanSortArgs {
   PlanView pv;
@@ -27,33 +28,46 @@ struct PlanSortArgs {
   int key_kind, S, N;  // N = power of two >= S
 };
 
-// Inclusive scan of one 64-bit value per thread over the block (a multiple of 64
-// threads, at most 1024).  `wave_tot` is LDS scratch of 17 entries.  Returns the
+// Inclusive scan of a 32-bit value over the wave with DPP adds: four shifts
+// inside each row of 16 lanes (a lane whose source falls outside its row adds
+// zero), then lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into rows
+// 2 and 3.
+__device__ __forceinline__ uint32_t wave_scan_incl_u32(uint32_t x) {
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, false);  // row_shr:1
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, false);  // row_shr:2
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, false);  // row_shr:4
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, false);  // row_shr:8
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xc, 0xf, false);  // row_bcast:31
+  return x;
+}
+// the two 32-bit halves of v are scanned independently (no carry between them)
+__device__ __forceinline__ uint64_t wave_scan_incl_2x32(uint64_t v) {
+  const uint32_t lo = wave_scan_incl_u32((uint32_t)v), hi = wave_scan_incl_u32((uint32_t)(v >> 32));
+  return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
+// Inclusive scan over the block (a multiple of 64 threads, at most 1024) of two
+// independent 32-bit counters packed into one 64-bit value per thread; neither
+// total may reach 2^32.  `wave_tot` is LDS scratch of 17 entries.  Returns the
 // inclusive prefix; the block total is left in wave_tot[16].
 __device__ __forceinline__ uint64_t block_scan_incl(uint64_t v, uint64_t* wave_tot) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    uint64_t o = __shfl_up((unsigned long long)v, d, 64);
-    if (lane >= d) v += o;
-  }
+  v = wave_scan_incl_2x32(v);
   __syncthreads();  // previous users of wave_tot are done
   if (lane == 63) wave_tot[wave] = v;
   __syncthreads();
   if (wave == 0) {  // exclusive scan of the (at most 16) wave totals, in registers
     const int nw = (int)(blockDim.x >> 6);
     const uint64_t t = lane < nw ? wave_tot[lane] : 0;
-    uint64_t run = t;
-#pragma unroll
-    for (int d = 1; d < 16; d <<= 1) {
-      uint64_t o = __shfl_up((unsigned long long)run, d, 64);
-      if (lane >= d) run += o;
-    }
-    if (lane < nw) wave_tot[lane] = run - t;
+    const uint64_t run = wave_scan_incl_2x32(t);
+    if (lane < nw) wave_tot[lane] = (uint64_t)((uint32_t)run - (uint32_t)t) |
+                                    ((uint64_t)((uint32_t)(run >> 32) - (uint32_t)(t >> 32)) << 32);
     if (lane == nw - 1) wave_tot[16] = run;
   }
   __syncthreads();
-  return v + wave_tot[wave];
+  const uint64_t base = wave_tot[wave];
+  return (uint64_t)((uint32_t)v + (uint32_t)base) | ((uint64_t)((uint32_t)(v >> 32) + (uint32_t)(base >> 32)) << 32);
 }
 
 // Sort key of segment i: group key in the high bits, segment index in the low
@@ -116,6 +130,21 @@ __device__ __forceinline__ int last_le(Arr a, int n, int q) {
   return lo;
 }
 
+// number of keys[j], j in [j0, j1), below `key`; eight LDS reads in flight at a time
+template <typename T>
+__device__ __forceinline__ int count_below(const T* keys, T key, int j0, int j1) {
+  int n = 0, j = j0;
+  for (; j + 8 <= j1; j += 8) {
+    T k8[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) k8[e] = keys[j + e];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) n += k8[e] < key ? 1 : 0;
+  }
+  for (; j < j1; ++j) n += keys[j] < key ? 1 : 0;
+  return n;
+}
+
 // ---------------------------------------------------------------- one launch
 // All global reads (keys, segment boundaries) are issued together up front: a
 // first-touch global load costs more than everything else in this kernel, so
@@ -127,7 +156,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   __shared__ int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
   __shared__ int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
   __shared__ uint64_t wave_tot[17];
-  __shared__ int bad_key;
+  __shared__ int bad_key, wide_key;
   const PlanView pv = args.pv;
   const int S = args.S, tid = threadIdx.x;  // blockDim.x >= S
 #ifdef SMLM_TUNING
@@ -147,11 +176,13 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     s0 = args.s[tid];
     s1 = args.s[tid + 1];
   }
-  if (tid == 0) bad_key = 0;
+  if (tid == 0) bad_key = 0, wide_key = 0;
   __syncthreads();
   // A 16-byte aligned address below 2^48 packs into 44 bits; anything else
   // cannot be a sort key, so such a batch is planned segment by segment.
   if (args.key_kind == SMLM_KEY_PTR && tid < S && ((raw >> 48) != 0 || (raw & 15) != 0)) bad_key = 1;
+  // adapter ids below 2^21 sort as 32-bit keys (id, segment), half the LDS traffic and compares
+  if (tid < S && (args.key_kind != SMLM_KEY_I32 || raw >= (1u << kNarrowIdBits))) wide_key = 1;
   if (tid < S) {
     start0[tid] = s0;
     len0[tid] = s1 > s0 ? s1 - s0 : 0;
@@ -168,10 +199,12 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   // Sort by counting: keys are distinct (segment index inside), so the sorted
   // position of a key is the number of smaller keys.  The block's threads split
   // the S x S comparisons: thread (part, i) counts the keys of its part below
-  // key i, eight LDS reads in flight at a time, and adds its count to rank[i].
+  // key i and adds its count to rank[i].
   if (kind != SMLM_KEY_NONE) {
+    const bool narrow = !wide_key;
+    uint32_t* K32 = reinterpret_cast<uint32_t*>(K0);
     if (tid < S) {
-      K0[tid] = mine;
+      if (narrow) K32[tid] = ((uint32_t)raw << 10) | (uint32_t)tid; else K0[tid] = mine;
       sseg[tid] = 0;  // rank accumulator for now
     }
     __syncthreads();
@@ -179,18 +212,10 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     const int parts = (int)blockDim.x / Sp;  // blockDim.x is a multiple of Sp
     const int i = tid % Sp, part = tid / Sp;
     if (i < S && part < parts) {
-      const uint64_t key = K0[i];
-      const int per = (S + parts - 1) / parts;
+      const int per = (((S + parts - 1) / parts) + 7) & ~7;
       const int j0 = part * per, j1 = (j0 + per < S) ? j0 + per : S;
-      int rank = 0, j = j0;
-      for (; j + 8 <= j1; j += 8) {
-        uint64_t k8[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) k8[e] = K0[j + e];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) rank += k8[e] < key ? 1 : 0;
-      }
-      for (; j < j1; ++j) rank += K0[j] < key ? 1 : 0;
+      int rank = 0;
+      if (j0 < j1) rank = narrow ? count_below<uint32_t>(K32, K32[i], j0, j1) : count_below<uint64_t>(K0, K0[i], j0, j1);
       if (rank) atomicAdd(&sseg[i], rank);  // integer adds: the total does not depend on their order
     }
     __syncthreads();
@@ -202,7 +227,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
 
   SMLM_TICK();
   // gathered-row position of every sorted segment, group heads
-  constexpr uint64_t kRowMask = (1ull << 40) - 1;
+  constexpr uint64_t kRowMask = 0xffffffffull;  // rows in the low half, group heads in the high half
   int seg = 0, len = 0;
   uint64_t gk = 0;
   bool head = false;
@@ -214,10 +239,10 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     head = true;
     if (tid > 0) head = (K[tid - 1] >> kSegBits) != gk;
   }
-  const uint64_t v = (uint64_t)len | ((uint64_t)(head ? 1 : 0) << 40);
+  const uint64_t v = (uint64_t)len | ((uint64_t)(head ? 1 : 0) << 32);
   const uint64_t incl = block_scan_incl(v, wave_tot);
   const uint64_t total = wave_tot[16];
-  const int rows_total = (int)(total & kRowMask), NG = (int)(total >> 40);
+  const int rows_total = (int)(total & kRowMask), NG = (int)(total >> 32);
   if (tid < S) {
     const int rows_before = (int)((incl - v) & kRowMask);
     sseg[tid] = seg;
@@ -225,7 +250,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     pv.sorted_seg[tid] = seg;
     pv.rowpos[tid] = rows_before;
     if (head) {
-      const int G = (int)(incl >> 40) - 1;
+      const int G = (int)(incl >> 32) - 1;
       grow[G] = rows_before;
       gseg[G] = seg;
       gid[G] = (int32_t)(uint32_t)gk;
@@ -337,7 +362,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
   // Pass A: gathered-row position of every sorted segment, group heads.
   if (tid == 0) carry = 0;
   __syncthreads();
-  constexpr uint64_t kRowMask = (1ull << 40) - 1;
+  constexpr uint64_t kRowMask = 0xffffffffull;  // rows in the low half, group heads in the high half
   for (int base = 0; base < S; base += kPlanThreads) {
     const int p = base + tid;
     const bool valid = p < S;
@@ -353,7 +378,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
       head = true;
       if (p > 0) head = (K[p - 1] >> kSegBits) != gk;
     }
-    const uint64_t v = (uint64_t)len | ((uint64_t)(head ? 1 : 0) << 40);
+    const uint64_t v = (uint64_t)len | ((uint64_t)(head ? 1 : 0) << 32);
     const uint64_t incl = block_scan_incl(v, wave_tot) + carry;
     const uint64_t excl = incl - v;
     if (valid) {
@@ -361,7 +386,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
       pv.sorted_seg[p] = seg;
       pv.rowpos[p] = rows_before;
       if (head) {
-        const int G = (int)(incl >> 40) - 1;
+        const int G = (int)(incl >> 32) - 1;
         pv.grp_row[G] = rows_before;
         pv.grp_seg[G] = seg;
         pv.grp_id[G] = (int32_t)(uint32_t)gk;
@@ -372,7 +397,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
     __syncthreads();
   }
   const int rows_total = (int)(carry & kRowMask);
-  const int NG = (int)(carry >> 40);
+  const int NG = (int)(carry >> 32);
   if (tid == 0) {
     pv.rowpos[S] = rows_total;
     pv.grp_row[NG] = rows_total;
