@@ -669,7 +669,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   ta.set[1] = TransposeSet{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
   ta.NA = NA;
   {
-    const int gx = ceil_div(h_in > h_out ? h_in : h_out, 32), gy = ceil_div(r, 32);
+    const int gx = ceil_div(h_in > h_out ? h_in : h_out, 64), gy = ceil_div(r, 64);
     if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
   }
 

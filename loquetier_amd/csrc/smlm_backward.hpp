@@ -22,29 +22,58 @@ struct TransposeArgs {
   int NA;
 };
 
-// 32x32 tiles through LDS; grid (tiles along the hidden dimension, tiles along the
-// rank, 2*NA), block 256: x walks the columns of A and the rows of B.
+constexpr int kTrPitch = 80;  // LDS row pitch in 16-bit elements (40 banks: see kWgPitch)
+
+// Transposing LDS read of gfx950: within each 16 lanes, lane i names a "row" of
+// four 16-bit elements M[i][0..3]; lane 4a+b receives M[a][b], M[4+a][b],
+// M[8+a][b], M[12+a][b].
+typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 lds_tr_f16x4;
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_addr) {
+  typedef __attribute__((address_space(3))) lds_tr_f16x4 lds_vec;
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_vec*)lds_addr));
+}
+
+// 64x64 tiles through LDS, 16-byte global accesses on both sides: rows of the
+// source tile are written to LDS as they are and read back down the columns
+// with the transposing LDS read.  grid (tiles along the hidden dimension, tiles
+// along the rank, 2*NA), block 256: x walks the columns of A and the rows of B.
+// Rows and columns are multiples of 8.
 __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
-  __shared__ uint16_t t[32][33];
+  __shared__ __attribute__((aligned(16))) uint16_t t[64 * kTrPitch];
   const int which = blockIdx.z / a.NA, ad = blockIdx.z - which * a.NA;
   const TransposeSet S = a.set[which];
-  const int c0 = (which == 0 ? blockIdx.x : blockIdx.y) * 32;
-  const int r0 = (which == 0 ? blockIdx.y : blockIdx.x) * 32;
+  const int c0 = (which == 0 ? blockIdx.x : blockIdx.y) * 64;
+  const int r0 = (which == 0 ? blockIdx.y : blockIdx.x) * 64;
   if (c0 >= S.cols || r0 >= S.rows) return;  // uniform over the workgroup
   const uint16_t* src = reinterpret_cast<const uint16_t*>(S.src_ptrs[ad]);
   uint16_t* dst = S.dst_base + (long)ad * S.stride;
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) S.dst_ptrs[ad] = dst;
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  // in: lane -> (row = tid / 8 (+32), 8 columns at (tid % 8) * 8)
+  const int ir = threadIdx.x >> 3, ic = (threadIdx.x & 7) * 8;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = r0 + ty + 8 * i, c = c0 + tx;
-    t[ty + 8 * i][tx] = (r < S.rows && c < S.cols) ? src[(long)r * S.cols + c] : (uint16_t)0;
+  for (int h = 0; h < 2; ++h) {
+    const int r = r0 + ir + 32 * h, c = c0 + ic;
+    const u32x4 v = (r < S.rows && c < S.cols) ? ldg16(src + (long)r * S.cols + c) : zero;
+    *reinterpret_cast<u32x4*>(&t[(ir + 32 * h) * kTrPitch + ic]) = v;
   }
   __syncthreads();
+  // out: thread -> output row (source column) oc = tid / 8 (+32), 8 source rows at 8 * (tid % 8).
+  // Within 16 lanes (two output rows... ) the transposing read wants lane i to name source row
+  // (i / 4) and four columns at 4 * (i % 4); lane 4a+b then holds column 4*... of rows a, a+4, ...
+  // so a wave covers 16 source columns x 16 source rows per read: organise the 256 threads as
+  // (column block cb = tid / 64 -> 16 columns, wave-lane l): g = l / 16 picks 16 of the 64 rows.
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = lane >> 4, i = lane & 15;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = c0 + ty + 8 * i, r = r0 + tx;
-    if (r < S.rows && c < S.cols) dst[(long)c * S.rows + r] = t[tx][ty + 8 * i];
+  for (int h = 0; h < 2; ++h) {
+    // rows 16g + 8h + {0..7} of the tile: two reads of four rows each; lane i = 4a+b names row
+    // (base + i/4), columns 16*wave + 4*(i%4) .. +3 and receives column 16*wave + i, rows base + {0..3}
+    const int rb = 16 * g + 8 * h;
+    const uint16_t* p0 = &t[(rb + (i >> 2)) * kTrPitch + 16 * wave + 4 * (i & 3)];
+    const u32x2 q0 = lds_read_tr16(p0), q1 = lds_read_tr16(p0 + 4 * kTrPitch);
+    const int oc = c0 + 16 * wave + i, orow = r0 + rb;
+    if (oc < S.cols && orow < S.rows) stg16(dst + (long)oc * S.rows + orow, u32x4{q0[0], q0[1], q1[0], q1[1]});
   }
 }
 
@@ -67,15 +96,6 @@ constexpr int kWgCols = 64;     // columns of x / dY per workgroup
 constexpr int kWgPitch = 80;    // LDS row pitch in 16-bit elements: 40 banks, so any eight
                                 // consecutive rows start 8 banks apart and tile the 64 banks
 constexpr int kWgSlots = 64;    // gathered rows (four tiles) per wave and loop step
-
-// Transposing LDS read of gfx950: within each 16 lanes, lane i names a "row" of
-// four 16-bit elements M[i][0..3]; lane 4a+b receives M[a][b], M[4+a][b],
-// M[8+a][b], M[12+a][b].
-typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 lds_tr_f16x4;
-__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_addr) {
-  typedef __attribute__((address_space(3))) lds_tr_f16x4 lds_vec;
-  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_vec*)lds_addr));
-}
 
 // LDS row of gathered-row slot s of a step: bits 2 and 3 of s change places, so
 // that the eight rows one half-wave reads together (slots 8g+4h+{0..3}, g = 0,1)
