@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SMLM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|rmsnorm]
 
 A step is one pass of the hot path over one synthetic batch: the tile plan is
 built from the batch's (segment, adapter-id) arrays, then every projection of
@@ -94,6 +94,95 @@ def backward_bytes(w, h_in, h_out):
     return n * (h_out + 2 * h_in) * 2 + 2 * rsum * (h_in + h_out) * 2 + 3 * n * w["r"] * 2
 
 
+def rmsnorm_bench(args, torch, K):
+    """RMSNorm forward + backward on the rows of the fine-tune + serve batch (4224 x 4096, bf16):
+    the other native operator of the reference's model (rms_norm_cutlass.cu, kernel_utils.py:149-176).
+    A step = forward over all rows + backward over the 4096 training rows."""
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    T, n_train, n, tdt = 4224, 4096, 4096, torch.bfloat16
+    fwd_bytes = T * n * 2 * 2 + n * 2 + T * 4
+    bwd_bytes = n_train * n * 2 * 3 + n * 2 * 2 + n_train * 4
+    R = max(2, math.ceil(640e6 / (T * n * 2 * 2 + n_train * n * 2 * 2)))
+    gen = torch.Generator(device="cpu").manual_seed(7)
+    sets = []
+    for _ in range(R):
+        x = torch.randn(T, n, generator=gen).to(dev).to(tdt)
+        sets.append(dict(x=x, w=(1 + 0.1 * torch.randn(n, generator=gen)).to(dev).to(tdt), o=torch.empty_like(x),
+                         m=torch.empty(T, 1, dtype=torch.float32, device=dev),
+                         g=torch.randn(n_train, n, generator=gen).to(dev).to(tdt),
+                         dx=torch.empty(n_train, n, dtype=tdt, device=dev), dw=torch.empty(n, dtype=tdt, device=dev)))
+
+    def fwd(s):
+        K.rms_norm(s["o"], s["m"], s["x"], s["w"], 1e-5)
+
+    def bwd(s):
+        K.rms_norm_backward(s["dx"], s["dw"], s["g"], s["x"][:n_train], s["w"], s["m"][:n_train])
+
+    cap = torch.cuda.Stream()
+    with torch.cuda.stream(cap):
+        for s_ in sets:
+            fwd(s_), bwd(s_)
+    torch.cuda.synchronize()
+
+    def graph_of(fn, n_rep):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=cap):
+            for i in range(n_rep):
+                fn(sets[i % R])
+        return g
+
+    def timed(g, reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b)
+
+    g_step = graph_of(lambda s_: (fwd(s_), bwd(s_)), R)
+    timed(g_step, max(1, args.warmup // R))
+    n_rep = max(1, args.steps // R)
+    ms_per_step = timed(g_step, n_rep) / (n_rep * R)
+    g_f, g_b = graph_of(fwd, R), graph_of(bwd, R)
+    timed(g_f, 2), timed(g_b, 2)
+    fwd_us = timed(g_f, 10) * 1e3 / (10 * R)
+    bwd_us = timed(g_b, 10) * 1e3 / (10 * R)
+    achieved = fwd_bytes / (fwd_us * 1e-6) / 1e9
+    cpu = None
+    if not args.no_cpu_baseline:
+        import numpy as np
+        from oracle import smlm_oracle as O
+        xs = sets[0]["x"][:64].float().cpu().numpy()
+        ws = sets[0]["w"].float().cpu().numpy()
+        gs = sets[0]["g"][:64].float().cpu().numpy()
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < 10.0:
+            _, rms = O.rms_norm_fwd(xs, ws, 1e-5, "bf16")
+            O.rms_norm_bwd(gs, xs, ws, rms, "bf16")
+            reps += 1
+        el = time.perf_counter() - t0
+        cpu = dict(value=round(64 * reps / el, 1), unit="tokens/s", cores=1, kind="port",
+                   sample=f"{reps} passes of forward + backward over 64 rows x 4096 ({el:.1f} s), "
+                          "oracle/rms_norm_oracle.c, scalar C")
+    print(json.dumps({
+        "metric": "RMSNorm tokens/s + HBM GB/s (% of 8 TB/s), Llama-2-7B hidden size, 1 GPU",
+        "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": n_rep * R, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "rmsnorm: forward over 4224 rows x 4096 + backward over the 4096 training rows, "
+                               "bf16", "buffer_sets_rotated": R, "graph_replay": True},
+        "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
+        "step_hbm_gbps": round((fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9, 1),
+        "roofline": dict(kernel="rms_fwd_kernel", bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
+                         unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+                         us_per_launch=round(fwd_us, 3), algorithmic_bytes=fwd_bytes),
+        "kernels": {"fwd_us": round(fwd_us, 3), "fwd_gbps": round(achieved, 1), "bwd_us": round(bwd_us, 3),
+                    "bwd_gbps": round(bwd_bytes / (bwd_us * 1e-6) / 1e9, 1)},
+        "cpu_baseline": cpu}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -120,6 +209,8 @@ def main():
     from loquetier_amd import _lib
     from loquetier_amd.ops import _kernels as K
     _lib.load()  # no fallback: raises when the HIP library is missing
+    if args.config == "rmsnorm":
+        return rmsnorm_bench(args, torch, K)
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

@@ -189,6 +189,31 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
                            size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out,
                            int r, int dtype, const float* part_scale, void* stream);
 
+/*
+ * RMSNorm forward.  Replaces dispatch_rms_norm / rms_norm<T>
+ * (kernel_src/csrc/loquetier_ops.cc:326-358,
+ * kernel_src/csrc/rms_norm/rms_norm_cutlass.cu:81-186):
+ *   rms[t] = 1 / sqrt(mean_j x[t,j]^2 + eps)   (float, kept for the backward)
+ *   out[t,j] = x[t,j] * rms[t] * w[j]          (float arithmetic, rounded once)
+ * out, x: [rows, cols] of `dtype`; w: [cols] of `dtype`; rms: float [rows].
+ * cols a multiple of 8 (as in the reference) and at most 16384.
+ */
+SMLM_API int smlm_rms_norm_fwd(void* out, float* rms, const void* x, const void* w, int rows,
+                               int cols, float eps, int dtype, void* stream);
+
+/*
+ * RMSNorm backward.  Replaces the tensor expressions of rms_norm.backward
+ * (src/loquetier_src/kernel_utils.py:169-176), evaluated in float in one pass:
+ *   dot[t] = sum_j g*w*x,  dx = (g*w - x*dot*rms^2/cols) * rms,
+ *   dw[j] = sum_t x*rms*g   (summed in a fixed order, no atomics)
+ * dx, g, x: [rows, cols]; w, dw: [cols]; rms: float [rows] from the forward.
+ * The workspace holds the per-workgroup partial sums of dw.
+ */
+SMLM_API int smlm_rms_norm_bwd_workspace_size(int rows, int cols, size_t* bytes);
+SMLM_API int smlm_rms_norm_bwd(void* dx, void* dw, const void* g, const void* x, const void* w,
+                               const float* rms, void* workspace, size_t workspace_bytes, int rows,
+                               int cols, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

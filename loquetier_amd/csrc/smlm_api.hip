@@ -5,6 +5,7 @@
 
 #include <cstdlib>
 
+#include "rms_norm.hpp"
 #include "smlm.h"
 #include "smlm_backward.hpp"
 #include "smlm_common.hpp"
@@ -729,6 +730,96 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   const bool split = n_rows / NA >= 256;
   return dtype == SMLM_DTYPE_F16 ? launch_wgrad<SMLM_DTYPE_F16>(nbj, split, grid, st, wa)
                                  : launch_wgrad<SMLM_DTYPE_BF16>(nbj, split, grid, st, wa);
+}
+
+// workgroups of the RMSNorm backward: enough to fill the chip, each with several rows so that
+// the partial sums of dw stay small next to x and g
+// workgroups of the RMSNorm kernels: the forward gives every row group its own workgroup; the
+// backward walks four turns per workgroup (the next rows are fetched while the current ones are
+// worked on), so that its partial sums of dw stay small next to x and g
+static int rms_blocks(int rows, int cols, bool backward) {
+  const int rows_per_step = cols <= kRmsWaveCols ? 4 : 1;
+  int nb = ceil_div(rows, rows_per_step * (backward ? tune("SMLM_TUNE_RMS_ROWS", 4) : 1));
+  const int cap = backward ? tune("SMLM_TUNE_RMS_CAP", 512) : (1 << 22);
+  if (nb > cap) nb = cap;
+  return nb < 1 ? 1 : nb;
+}
+static int rms_bwd_blocks(int rows, int cols) { return rms_blocks(rows, cols, true); }
+
+static int rms_check(int rows, int cols, int dtype) {
+  if (rows < 0 || cols <= 0) return SMLM_ERR_ARG;
+  if (dtype != SMLM_DTYPE_F16 && dtype != SMLM_DTYPE_BF16) return SMLM_ERR_DTYPE;
+  if (cols & 7) return SMLM_ERR_ALIGN;
+  if (cols > kRmsMaxCols || rows > (1 << 30)) return SMLM_ERR_LIMIT;
+  return SMLM_OK;
+}
+
+SMLM_API int smlm_rms_norm_fwd(void* out, float* rms, const void* x, const void* w, int rows,
+                               int cols, float eps, int dtype, void* stream) {
+  int rc = rms_check(rows, cols, dtype);
+  if (rc) return rc;
+  if (rows == 0) return SMLM_OK;
+  if (!out || !rms || !x || !w) return SMLM_ERR_ARG;
+  if (!aligned16(out) || !aligned16(x) || !aligned16(w)) return SMLM_ERR_ALIGN;
+  const RmsFwdArgs a{reinterpret_cast<uint16_t*>(out), rms, reinterpret_cast<const uint16_t*>(x),
+                     reinterpret_cast<const uint16_t*>(w), rows, cols, eps};
+  hipStream_t st = (hipStream_t)stream;
+  const bool f16 = dtype == SMLM_DTYPE_F16;
+  const int nb = rms_blocks(rows, cols, false);
+  const dim3 grid((unsigned)nb);
+  const int rows_per_step = cols <= kRmsWaveCols ? 4 : 1;
+  const bool one_turn = (long)nb * rows_per_step >= rows;  // every workgroup sees one row group
+  if (cols <= kRmsWaveCols) {
+    if (one_turn)
+      return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, true>, grid, dim3(256), st, a)
+                 : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 1, true>, grid, dim3(256), st, a);
+    return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, false>, grid, dim3(256), st, a)
+               : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 1, false>, grid, dim3(256), st, a);
+  }
+  if (one_turn)
+    return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 4, true>, grid, dim3(256), st, a)
+               : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 4, true>, grid, dim3(256), st, a);
+  return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 4, false>, grid, dim3(256), st, a)
+             : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 4, false>, grid, dim3(256), st, a);
+}
+
+SMLM_API int smlm_rms_norm_bwd_workspace_size(int rows, int cols, size_t* bytes) {
+  if (!bytes) return SMLM_ERR_ARG;
+  int rc = rms_check(rows, cols, SMLM_DTYPE_F16);
+  if (rc) return rc;
+  *bytes = align_up((size_t)rms_bwd_blocks(rows > 0 ? rows : 1, cols) * cols * 4, 256);
+  return SMLM_OK;
+}
+
+SMLM_API int smlm_rms_norm_bwd(void* dx, void* dw, const void* g, const void* x, const void* w,
+                               const float* rms, void* workspace, size_t workspace_bytes, int rows,
+                               int cols, int dtype, void* stream) {
+  int rc = rms_check(rows, cols, dtype);
+  if (rc) return rc;
+  if (!dx || !dw || !g || !x || !w || !rms || !workspace) return SMLM_ERR_ARG;
+  if (!aligned16(dx) || !aligned16(dw) || !aligned16(g) || !aligned16(x) || !aligned16(w) ||
+      !aligned16(workspace))
+    return SMLM_ERR_ALIGN;
+  if (rows == 0) return SMLM_ERR_ARG;  // dw would have nothing to sum
+  const int nb = rms_bwd_blocks(rows, cols);
+  if (workspace_bytes < (size_t)nb * cols * 4) return SMLM_ERR_WORKSPACE;
+  hipStream_t st = (hipStream_t)stream;
+  const bool f16 = dtype == SMLM_DTYPE_F16;
+  const RmsBwdArgs a{reinterpret_cast<uint16_t*>(dx), reinterpret_cast<float*>(workspace),
+                     reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const uint16_t*>(x),
+                     reinterpret_cast<const uint16_t*>(w), rms, rows, cols};
+  const dim3 grid((unsigned)nb);
+  if (cols <= kRmsWaveCols)
+    rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 1>, grid, dim3(256), st, a)
+             : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 1>, grid, dim3(256), st, a);
+  else
+    rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 4>, grid, dim3(256), st, a)
+             : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 4>, grid, dim3(256), st, a);
+  if (rc) return rc;
+  const RmsFoldArgs fa{reinterpret_cast<uint16_t*>(dw), reinterpret_cast<const float*>(workspace), nb, cols};
+  const dim3 fgrid((unsigned)ceil_div(cols, 64));
+  return f16 ? launch(rms_fold_kernel<SMLM_DTYPE_F16>, fgrid, dim3(256), st, fa)
+             : launch(rms_fold_kernel<SMLM_DTYPE_BF16>, fgrid, dim3(256), st, fa);
 }
 
 }  // extern "C"

@@ -1,7 +1,8 @@
 """Host-side mirror of src/loquetier_src/kernel_utils.py for the SMLM path:
 `BatchLenInfo` (row layout of the flat batch) and the `add_lora` autograd
 Function, with the reference's positional arguments and `None`-padded backward
-tuple, running on the HIP kernels.
+tuple, running on the HIP kernels; and the `rms_norm` autograd Function
+(kernel_utils.py:149-176).
 """
 from __future__ import annotations
 
@@ -187,3 +188,26 @@ class add_lora(Function):
         grad_x, grads = lora_backward(grad_output, x, v, weight_list, ctx.tp, ctx.rank)
         return (None, grad_x, None, None, None, None, None, None, *grads)
 
+
+
+class rms_norm(Function):
+    """RMSNorm with the reference's call signature `rms_norm.apply(x, w, eps)`
+    (src/loquetier_src/kernel_utils.py:149-176).  x: [rows, cols] fp16/bf16,
+    w: [cols].  The backward runs as one fused kernel in float instead of the
+    reference's chain of 16-bit tensor expressions."""
+
+    @staticmethod
+    def forward(ctx: FunctionCtx, x: torch.Tensor, w: torch.Tensor, eps: float = 1e-6):
+        m = torch.empty((x.size(0), 1), dtype=torch.float32, device=x.device)
+        o = torch.empty_like(x)
+        kernel.rms_norm(o, m, x, w, eps)
+        ctx.save_for_backward(x, w, m)
+        return o
+
+    @staticmethod
+    def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
+        x, w, rms_1 = ctx.saved_tensors
+        dx = torch.empty_like(x)
+        d_weight = torch.empty_like(w)
+        kernel.rms_norm_backward(dx, d_weight, grad_output.contiguous(), x, w, rms_1)
+        return dx, d_weight, None

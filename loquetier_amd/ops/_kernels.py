@@ -287,3 +287,62 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                                        ws.numel(), n_rows, plan.S, NA, h_in, h_out, rank, code,
                                        _ptr(part_scale), _stream(dev))
     _lib.check(rc, "smlm_lora_backward")
+
+
+def rms_norm(output: torch.Tensor, rms_output: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
+             epsilon: float) -> None:
+    """output = input * rms * weight, rms_output = 1 / sqrt(mean(input^2) + epsilon) per row.
+
+    Same arguments and checks as dispatch_rms_norm
+    (kernel_src/csrc/loquetier_ops.cc:326-358): input/output [rows, cols] fp16
+    or bf16, weight [cols] of the same dtype, rms_output float32 [rows, 1].
+    """
+    for t, n in ((output, "output"), (rms_output, "rms_output"), (input, "input"), (weight, "weight")):
+        _check_input(t, n)
+    _check_dim(2, input, "input")
+    _check_dim(2, rms_output, "rms_output")
+    _check_dim(1, weight, "weight")
+    if output.shape != input.shape:
+        raise RuntimeError("output and input must have the same shape")
+    if rms_output.size(0) != input.size(0) or rms_output.size(1) != 1:
+        raise RuntimeError("rms_output must be [rows, 1]")
+    if rms_output.dtype != torch.float32:
+        raise RuntimeError("rms_output must be float32")
+    if weight.size(0) != input.size(1):
+        raise RuntimeError("weight must have one entry per column of input")
+    if input.dtype != weight.dtype or input.dtype != output.dtype:
+        raise RuntimeError("input, weight and output must share one dtype")
+    rows, cols = input.shape
+    if input.dtype not in _DTYPE_CODE or cols % 8 != 0:
+        raise RuntimeError(f"No suitable kernel. dtype={input.dtype} columns={cols}")
+    dev = input.device
+    with torch.cuda.device(dev):
+        rc = _lib.load().smlm_rms_norm_fwd(output.data_ptr(), rms_output.data_ptr(), input.data_ptr(),
+                                           weight.data_ptr(), rows, cols, float(epsilon),
+                                           _DTYPE_CODE[input.dtype], _stream(dev))
+    _lib.check(rc, "rms_norm")
+
+
+def rms_norm_backward(dx: torch.Tensor, dw: torch.Tensor, grad_output: torch.Tensor, x: torch.Tensor,
+                      w: torch.Tensor, rms: torch.Tensor) -> None:
+    """dx [rows, cols] and dw [cols] of RMSNorm from the upstream gradient and the
+    forward's saved tensors (the reference computes them with tensor expressions,
+    src/loquetier_src/kernel_utils.py:169-176)."""
+    for t, n in ((dx, "dx"), (dw, "dw"), (grad_output, "grad_output"), (x, "x"), (w, "w"), (rms, "rms")):
+        _check_input(t, n)
+    if dx.shape != x.shape or grad_output.shape != x.shape or dw.shape != w.shape:
+        raise RuntimeError("dx / grad_output must match x and dw must match w")
+    if rms.dtype != torch.float32 or rms.numel() != x.size(0):
+        raise RuntimeError("rms must be float32 with one entry per row")
+    if not (dx.dtype == dw.dtype == grad_output.dtype == x.dtype == w.dtype):
+        raise RuntimeError("dx, dw, grad_output, x, w must share one dtype")
+    rows, cols = x.shape
+    code = _dtype_code(x)
+    dev = x.device
+    with torch.cuda.device(dev):
+        need = _lib.size_query("smlm_rms_norm_bwd_workspace_size", rows, cols)
+        ws = _workspace(dev, need)
+        rc = _lib.load().smlm_rms_norm_bwd(dx.data_ptr(), dw.data_ptr(), grad_output.data_ptr(),
+                                           x.data_ptr(), w.data_ptr(), rms.data_ptr(), ws.data_ptr(),
+                                           ws.numel(), rows, cols, code, _stream(dev))
+    _lib.check(rc, "rms_norm_backward")

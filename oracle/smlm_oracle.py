@@ -22,8 +22,8 @@ DTYPES = {"fp32": 0, "fp16": 1, "bf16": 2}
 
 def build(force: bool = False) -> str:
     """Compile the C oracle with gcc (no GPU toolchain involved)."""
-    src = os.path.join(_HERE, "smlm_oracle.c")
-    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+    newest = max(os.path.getmtime(os.path.join(_HERE, f)) for f in ("smlm_oracle.c", "rms_norm_oracle.c"))
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < newest:
         subprocess.run(["make", "-C", _HERE, "-B" if force else "-s", "all"], check=True,
                        stdout=subprocess.DEVNULL)
     return _LIB_PATH
@@ -41,7 +41,7 @@ def lib() -> C.CDLL:
         for name in ("oracle_smlm_gemm", "oracle_add_lora_forward", "oracle_mixed_lora_linear",
                      "oracle_lora_fused", "oracle_add_lora_backward_rowmajor",
                      "oracle_add_lora_backward", "oracle_build_segments", "oracle_batch_len_info",
-                     "oracle_prepare_weight"):
+                     "oracle_prepare_weight", "oracle_rms_norm_fwd", "oracle_rms_norm_bwd"):
             getattr(_lib, name).restype = C.c_int
         _lib.oracle_round.restype = None
     return _lib
@@ -235,3 +235,25 @@ def prepare_weight(w, rank_dim: int, rank: int, scaling: Optional[float], dtype:
                                        C.c_float(0.0 if scaling is None else scaling), DTYPES[dtype]),
            "oracle_prepare_weight")
     return out
+
+
+def rms_norm_fwd(x, w, eps: float, dtype: str, acc64: bool = True) -> Tuple[np.ndarray, np.ndarray]:
+    """Returns (out [rows, cols], rms [rows]); reference: rms_norm_cutlass.cu:81-159."""
+    x, w = _f32(x), _f32(w)
+    rows, cols = x.shape
+    out = np.zeros((rows, cols), np.float32)
+    rms = np.zeros(max(rows, 1), np.float32)
+    _check(lib().oracle_rms_norm_fwd(_fp(out), _fp(rms), _fp(x), _fp(w), rows, cols, C.c_float(eps),
+                                     DTYPES[dtype], int(acc64)), "oracle_rms_norm_fwd")
+    return out, rms[:rows]
+
+
+def rms_norm_bwd(g, x, w, rms, dtype: str, literal: bool = False) -> Tuple[np.ndarray, np.ndarray]:
+    """Returns (dx [rows, cols], dw [cols]); reference: kernel_utils.py:169-176."""
+    g, x, w, rms = _f32(g), _f32(x), _f32(w), _f32(rms)
+    rows, cols = x.shape
+    dx = np.zeros((rows, cols), np.float32)
+    dw = np.zeros(cols, np.float32)
+    _check(lib().oracle_rms_norm_bwd(_fp(dx), _fp(dw), _fp(g), _fp(x), _fp(w), _fp(rms), rows, cols,
+                                     DTYPES[dtype], int(literal)), "oracle_rms_norm_bwd")
+    return dx, dw

@@ -85,6 +85,24 @@ def test_argument_validation_codes(lib):
                            None, None) == -4
 
 
+def test_rms_norm_argument_validation_codes(lib):
+    L = lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256  # aligned fake "device" address; never dereferenced
+    fwd = lambda **k: L.smlm_rms_norm_fwd(k.get("out", p), p, p, p, k.get("rows", 4), k.get("cols", 64), 1e-6,
+                                          k.get("dtype", 0), None)
+    assert fwd(dtype=2) == -2
+    assert fwd(cols=60) == -3          # the reference refuses columns % 8 != 0 (rms_norm_cutlass.cu:166-168)
+    assert fwd(cols=16392) == -6       # beyond four waves' worth of registers per row
+    assert fwd(out=None) == -1
+    assert fwd(out=p + 2) == -3
+    assert fwd(rows=0) == 0            # nothing to do, no launch
+    assert fwd(rows=-1) == -1
+    assert lib.size_query("smlm_rms_norm_bwd_workspace_size", 4096, 4096) >= 4096 * 4
+    assert L.smlm_rms_norm_bwd(p, p, p, p, p, p, p, 16, 64, 4096, 0, None) == -4   # workspace too small
+    assert L.smlm_rms_norm_bwd(p, p, p, p, p, p, None, 1 << 30, 64, 4096, 0, None) == -1
+
+
 def test_python_surface_rejects_host_tensors(lib):
     from loquetier_amd.ops import _kernels as K
     y, x = torch.zeros(4, 8, dtype=torch.float16), torch.zeros(4, 16, dtype=torch.float16)
