@@ -116,7 +116,7 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   want = tune("SMLM_TUNE_KSPLIT", want);
   int max_split = d_in / (c.NW * kq);
   if (max_split < 1) max_split = 1;
-  if (max_split > 16) max_split = 16;
+  if (max_split > kMaxKsplit) max_split = kMaxKsplit;
   const int ks = want < 1 ? 1 : (want > max_split ? max_split : want);
   c.k_per_wave = round_up(ceil_div(d_in, c.NW * ks), kq);
   c.ksplit = ceil_div(d_in, c.NW * c.k_per_wave);

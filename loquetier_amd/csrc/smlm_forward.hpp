@@ -352,6 +352,8 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #undef SMLM_TICK
 }
 
+constexpr int kMaxKsplit = 16;  // upper bound of the k split over workgroups
+
 struct ReduceProj {
   const float* partial;  // [ksplit, T, d_out]
   uint16_t* out;         // [T, d_out]
@@ -383,9 +385,17 @@ __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
     const int row = a.plan.tile_row[tile * kTileRows + c];
     if (row < 0) continue;
     const float scale = a.seg_scale ? a.seg_scale[a.plan.tile_rseg[tile * kTileRows + c]] : 1.0f;
+    const float* zf = reinterpret_cast<const float*>(a.plan.hdr + kHdrZeros);
     for (int n = 4 * q; n < a.d_out; n += 64) {
-      f32x4 sum = ldg_f4(P.partial + (long)row * a.d_out + n);
-      for (int z = 1; z < P.ksplit; ++z) sum += ldg_f4(P.partial + ((long)z * a.T + row) * a.d_out + n);
+      // all partials are requested before the first add waits for one; past ksplit the loads
+      // read zeros (the k split never exceeds kMaxKsplit)
+      f32x4 part[kMaxKsplit];
+#pragma unroll
+      for (int z = 0; z < kMaxKsplit; ++z)
+        part[z] = ldg_f4(z < P.ksplit ? P.partial + ((long)z * a.T + row) * a.d_out + n : zf);
+      f32x4 sum = part[0];
+#pragma unroll
+      for (int z = 1; z < kMaxKsplit; ++z) sum += part[z];
       store4<DT>(P.out + (long)row * a.d_out + n, sum, scale, a.beta);
     }
   }
