@@ -294,8 +294,21 @@ __global__ __launch_bounds__(256) void rms_fold_kernel(RmsFoldArgs a) {
   const int rg = threadIdx.x >> 4, c4 = threadIdx.x & 15;
   const int col = (int)blockIdx.x * 64 + c4 * 4;
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
-  if (col < a.cols)
-    for (int p = rg; p < a.n_part; p += kRmsFoldRows) s += ldg_f4(a.partial + (long)p * a.cols + col);
+  if (col < a.cols) {
+    // eight partial rows are requested at a time; rows past the end re-read row rg and are dropped
+    for (int p0 = rg; p0 < a.n_part; p0 += 8 * kRmsFoldRows) {
+      f32x4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int p = p0 + j * kRmsFoldRows;
+        v[j] = ldg_f4(a.partial + (long)(p < a.n_part ? p : rg) * a.cols + col);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (p0 + j * kRmsFoldRows < a.n_part) s += v[j];
+    }
+  }
   red[rg][c4] = s;
   __syncthreads();
   if (rg == 0 && col < a.cols) {
