@@ -381,6 +381,67 @@ def test_forward_dyadic_bit_exact_larger(K, oracle, gpu_device, shape, dt):
     _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
 
 
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [
+    # T, S, NA, h_in, h_out, r: few rows and a long k -> sixteen-wave shrink with k split over
+    # two workgroups, partial sums folded by the expand kernel
+    (1, 1, 1, 4096, 512, 16),
+    (17, 17, 5, 4096, 1024, 8),
+    (256, 256, 32, 4096, 640, 16),
+    (200, 23, 9, 11008, 512, 32),     # k not a multiple of the waves' share: ragged last batch
+    (1000, 61, 7, 2048, 1536, 64),    # shortest k that takes the sixteen-wave route at rank 64
+    (96, 10, 3, 4104, 264, 24),       # k and rank off the round sizes
+    (300, 30, 4, 2040, 512, 16),      # just below the route's minimum k: four-wave shrink
+], ids=["one-row", "r8", "decode-256", "k11008", "r64-k2048", "odd-sizes", "below-min-k"])
+def test_forward_dyadic_bit_exact_decode_route(K, oracle, gpu_device, shape, dt):
+    T, S, NA, h_in, h_out, r = shape
+    rng = np.random.default_rng(41)
+    seg = list(range(T + 1)) if S == T else _ragged_segments(rng, T, S)
+    ids = rng.integers(0, NA, S).tolist()
+    x, A, B = make_case(oracle, 203, T, seg, ids, NA, h_in, h_out, r, dt, dy=True)
+    base = dyadic(rng, (T, h_out), 16, 8)
+    _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
+
+
+def test_multi_projection_mixed_routes_equal_single_calls(K, oracle, gpu_device):
+    """Projections of one launch with different k: all long (sixteen-wave route with a different
+    k split each) and one short (which sends the whole launch down the four-wave route)."""
+    d, dt = gpu_device, "fp16"
+    T, r, NA, S = 120, 16, 5, 14
+    rng = np.random.default_rng(43)
+    seg = _ragged_segments(rng, T, S)
+    ids = rng.integers(0, NA, S).tolist()
+    s = torch.tensor(seg, dtype=torch.int32, device=d)
+    plan = K.SegmentPlan(s, torch.tensor(ids, dtype=torch.int32, device=d), T)
+    sc = torch.full((S,), 2.0, device=d)
+    for dims in ([(4096, 512), (11008, 256), (2048, 1024)], [(4096, 512), (512, 512)]):
+        projs = []
+        for hi, ho in dims:
+            A = [dev_t(dyadic(rng, (r, hi), 8, 64), dt, d) for _ in range(NA)]
+            B = [dev_t(dyadic(rng, (ho, r), 8, 8), dt, d) for _ in range(NA)]
+            projs.append(dict(x=dev_t(dyadic(rng, (T, hi), 16, 8), dt, d), a=ptrs(A, d), b=ptrs(B, d), A=A, B=B,
+                              y0=dev_t(dyadic(rng, (T, ho), 16, 8), dt, d)))
+        single, single_v = [], []
+        for p in projs:
+            y, v = p["y0"].clone(), torch.zeros(T, r, dtype=TDT[dt], device=d)
+            K.smlm_lora_forward(y, p["x"], p["a"], p["b"], plan, r, seg_scale=sc, beta=1.0, v_out=v)
+            single.append(y)
+            single_v.append(v)
+        ys = [p["y0"].clone() for p in projs]
+        vs = [torch.zeros(T, r, dtype=TDT[dt], device=d) for _ in projs]
+        K.smlm_lora_forward_multi(ys, [p["x"] for p in projs], [p["a"] for p in projs],
+                                  [p["b"] for p in projs], plan, r, seg_scale=sc, beta=1.0, v_out=vs)
+        for a, b in zip(single + single_v, ys + vs):
+            assert torch.equal(a, b)
+        # and without the copy of v, and as two separately issued stages
+        ys2 = [p["y0"].clone() for p in projs]
+        args = ([p["x"] for p in projs], [p["a"] for p in projs], [p["b"] for p in projs], plan, r)
+        K.smlm_lora_forward_multi(ys2, *args, seg_scale=sc, beta=1.0, stages=1)
+        K.smlm_lora_forward_multi(ys2, *args, seg_scale=sc, beta=1.0, stages=2)
+        for a, b in zip(single, ys2):
+            assert torch.equal(a, b)
+
+
 def test_multi_projection_equals_single_calls(K, oracle, gpu_device):
     """q/k/v/o-style batched launch: bit-identical to one call per projection,
     with different widths per projection and a shared x for three of them."""
@@ -426,6 +487,8 @@ BWD_CASES = [
     ("empty-part", [0, 17, 17, 50], [0, 1, 2], 3, 0, 256, 128, 32),
     ("rank64", [0, 33, 90], [0, 1], 2, 4, 192, 320, 64),
     ("long", [0, 300, 700], [1, 0], 2, 20, 512, 384, 16),
+    # few rows and long k: the sixteen-wave shrink (k split in two, folded by a launch) for v and dV
+    ("long-k", [0, 30, 75], [1, 0], 2, 4, 4096, 2048, 16),
 ]
 
 
