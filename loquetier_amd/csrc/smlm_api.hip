@@ -98,9 +98,8 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   const int cols = d_out >= 64 ? 64 : d_out;
   c.NB = cols <= 16 ? 1 : (cols <= 32 ? 2 : 4);
   c.MT = tiles_per_wave(T);
-  // 32-wide k steps per load batch; tile blocks hold four tiles of operands per batch and two
-  // batches at a time, so their batches are shorter
-  c.U = (c.NB == 4 ? 2 : 4) / (c.MT > 1 ? 2 : 1);
+  // 32-wide k steps per load batch (the tile-block kernel stages four per batch in LDS)
+  c.U = c.MT > 1 ? 4 : (c.NB == 4 ? 2 : 4);
   const int kq = 32 * c.U;
   c.NW = nw;
   const int units = ceil_div(T > 0 ? T : 1, kTileRows * c.MT);
@@ -151,24 +150,31 @@ inline dim3 item_grid(const ItemSpace& sp, long items) {
   return dim3((unsigned)rows, (unsigned)sp.units_max, (unsigned)sp.nproj);
 }
 
-template <int DT, int MT, int NW, bool RM, bool DIRECT>
+template <int DT, int NW, bool RM, bool DIRECT>
 int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
-  const dim3 block(NW * kWaveSize);
-  constexpr int UD = MT > 1 ? 2 : 1;  // must match shrink_cfg
-  if (NB == 1) return launch(shrink_kernel<DT, 1, 4 / UD, MT, NW, RM, DIRECT>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_kernel<DT, 2, 4 / UD, MT, NW, RM, DIRECT>, grid, block, st, a);
-  return launch(shrink_kernel<DT, 4, 2 / UD, MT, NW, RM, DIRECT>, grid, block, st, a);
+  const dim3 block(NW * kWaveSize);  // U must match shrink_cfg
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, 1, NW, RM, DIRECT>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, 1, NW, RM, DIRECT>, grid, block, st, a);
+  return launch(shrink_kernel<DT, 4, 2, 1, NW, RM, DIRECT>, grid, block, st, a);
+}
+
+template <int DT, bool DIRECT>
+int launch_shrink_block(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
+  const dim3 block(kFwdThreads);
+  if (NB == 1) return launch(shrink_block_kernel<DT, 1, 4, DIRECT>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_kernel<DT, 2, 4, DIRECT>, grid, block, st, a);
+  return launch(shrink_block_kernel<DT, 4, 4, DIRECT>, grid, block, st, a);
 }
 
 template <int DT, bool DIRECT>
 int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStream_t st,
                      const ShrinkArgs& a) {
   if (row_major)  // the slow layout
-    return launch_shrink_nb<DT, 1, kFwdWaves, true, DIRECT>(NB, grid, st, a);
+    return launch_shrink_nb<DT, kFwdWaves, true, DIRECT>(NB, grid, st, a);
   if (MT == 1)
-    return NW == 16 ? launch_shrink_nb<DT, 1, 16, false, DIRECT>(NB, grid, st, a)
-                    : launch_shrink_nb<DT, 1, kFwdWaves, false, DIRECT>(NB, grid, st, a);
-  return launch_shrink_nb<DT, kBlkTiles, kFwdWaves, false, DIRECT>(NB, grid, st, a);
+    return NW == 16 ? launch_shrink_nb<DT, 16, false, DIRECT>(NB, grid, st, a)
+                    : launch_shrink_nb<DT, kFwdWaves, false, DIRECT>(NB, grid, st, a);
+  return launch_shrink_block<DT, DIRECT>(NB, grid, st, a);
 }
 
 // all projections of one launch share NB / U / MT / NW (same rank, same T)

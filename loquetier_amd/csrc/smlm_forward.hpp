@@ -352,6 +352,118 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #undef SMLM_TICK
 }
 
+// Shrink for tile blocks (batches of 1024 rows and more).  Work item -> (projection, k
+// slice, 64-column block, tile block) as above, but here wave w owns tile w of the block
+// and all four waves walk the whole k slice together: each 32*U-wide batch of the weight
+// rows is staged once in LDS (two buffers in turn, one barrier a batch) and shared by the
+// four tiles, while every wave loads the x fragments of its own tile straight into
+// registers one batch ahead.  Against the kernel above with MT = 4 this reads the weights
+// from L2 once per workgroup instead of once per wave and needs no cross-wave sum.
+template <int DT, int NB, int U, bool DIRECT>
+__global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a) {
+  constexpr int KB = 32 * U;                 // k per batch
+  constexpr int kPitch = KB + 8;             // LDS row pitch: rows 16 bytes apart mod 128
+  constexpr int kRowsW = 16 * NB;            // weight rows (output columns) per workgroup
+  constexpr int kPieces = kRowsW * (KB / 8); // 16-byte pieces of one staged batch
+  constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
+  __shared__ __attribute__((aligned(16))) uint16_t wlds[2][kRowsW * kPitch];
+  const int units = DIRECT ? 0 : tile_units<kBlkTiles>(a.plan, 0);
+  const WorkRange wr = item_range<DIRECT>(a.items, units);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
+
+  for (int V = wr.first; V < wr.last; V += wr.step) {
+    int pj, yy, tb;
+    if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tb)) break;
+    const ShrinkProj P = a.p[pj];
+    const int kz = yy % P.ksplit, zb = yy / P.ksplit;
+    int t0, cnt, wid;
+    pick_tiles<kBlkTiles>(a.plan, tb, &t0, &cnt, &wid);
+    if (cnt == 0) continue;  // uniform over the workgroup
+    const int n0 = zb * 64;
+    const bool active = wave < cnt;
+    const int slot = (t0 + (active ? wave : 0)) * kTileRows + c;
+    const int row = active ? a.plan.tile_row[slot] : -1;
+    const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+    const int kbeg = kz * kFwdWaves * P.k_per_wave;
+    const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
+    const uint16_t* xrow = P.x + (long)(row < 0 ? 0 : row) * P.d_in;
+
+    auto load_x = [&](int kb, u32x4 (&xf)[U]) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kk = kb + 32 * u + 8 * g;
+        xf[u] = ldg16_or(xrow + kk, row >= 0 && kk < kend, zeros);
+      }
+    };
+    auto load_w = [&](int kb, u32x4 (&st)[kPer]) {
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int idx = threadIdx.x + j * kFwdThreads;
+        const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
+        st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
+                         idx < kPieces && n0 + nl < P.d_out && kb + k8 < kend, zeros);
+      }
+    };
+    auto stage_w = [&](int buf, const u32x4 (&st)[kPer]) {
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int idx = threadIdx.x + j * kFwdThreads;
+        const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
+        if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[buf][nl * kPitch + k8]) = st[j];
+      }
+    };
+
+    f32x4 acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 xf[U], wst[kPer];
+    load_x(kbeg, xf);
+    load_w(kbeg, wst);
+    __syncthreads();  // every wave is done with both LDS buffers of the previous item
+    stage_w(0, wst);
+    int buf = 0;
+#pragma unroll 1
+    for (int kb = kbeg; kb < kend; kb += KB) {
+      u32x4 xn[U], wn[kPer];
+      // the next batch is requested before this one is multiplied (past the end: zeros)
+      load_x(kb + KB, xn);
+      load_w(kb + KB, wn);
+      __syncthreads();  // buffer `buf` is written; buffer `buf ^ 1` is no longer read
+      if (active) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const u32x4 wf = *reinterpret_cast<const u32x4*>(&wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
+            acc[nb] = Num<DT>::mfma(wf, xf[u], acc[nb]);
+          }
+      }
+      stage_w(buf ^ 1, wn);
+      buf ^= 1;
+#pragma unroll
+      for (int u = 0; u < U; ++u) xf[u] = xn[u];
+    }
+
+    if (row >= 0) {
+      const bool as_partial = P.ksplit > 1 || P.to_partial;
+      float scale = 1.0f;
+      if (!as_partial && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
+        if (n >= P.d_out) continue;
+        if (as_partial)
+          *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + row) * P.d_out + n) = acc[nb];
+        else
+          store4<DT>(P.out + (long)row * P.d_out + n, acc[nb], scale, a.beta);
+      }
+    }
+  }
+}
+
 constexpr int kMaxKsplit = 16;  // upper bound of the k split over workgroups
 
 struct ReduceProj {
