@@ -687,13 +687,20 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 // tiles instead of once per tile.
 template <int DT, int NQ, int KS, bool DIRECT>
 __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a) {
+  static_assert(NQ % 2 == 0, "the output is written 64 columns at a time");
   constexpr int kPitch = 32 * KS + 8;  // LDS row pitch in 16-bit elements: rows 16 bytes apart mod 128
+  constexpr int kOPitch = 64 + 4;      // floats: output staging rows 4 banks apart
   __shared__ __attribute__((aligned(16))) uint16_t wlds[32 * NQ * kPitch];
+  __shared__ __attribute__((aligned(16))) float olds[kFwdWaves][kTileRows * kOPitch];
   const int units = DIRECT ? 0 : tile_units<kBlkTiles>(a.plan, 0);
   const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
   const int mrow = 8 * (c >> 2) + (c & 3);
+  // y is read and written a full 128-byte line per row and instruction: lane -> (row lane/8
+  // (+8), 8 columns at (lane%8)*8 of a 64-column half chunk).  The accumulators come out of
+  // the MFMA as 64-byte pieces per row, so they change layout through LDS on the way.
+  const int orow = lane >> 3, ocol = (lane & 7) * 8;
 
   for (int V = wr.first; V < wr.last; V += wr.step) {
     int pj, yy, tb;
@@ -705,9 +712,16 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
     if (cnt == 0) continue;  // past the last block (direct mode); uniform over the workgroup
     const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, t0));
     const bool active = wave < cnt;
-    const int slot = (t0 + (active ? wave : 0)) * kTileRows + c;
-    const int row = active ? a.plan.tile_row[slot] : -1;
-    const int rseg = (a.seg_scale && active) ? a.plan.tile_rseg[slot] : -1;  // -1 on empty slots too
+    const int tslot = (t0 + (active ? wave : 0)) * kTileRows;
+    const int slot = tslot + c;
+    const int row = active ? a.plan.tile_row[slot] : -1;  // row of the MFMA column this lane feeds
+    int srow[2], sseg[2];                                  // rows this lane reads and writes in y
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      srow[j] = active ? a.plan.tile_row[tslot + orow + 8 * j] : -1;
+      sseg[j] = (a.seg_scale && active) ? a.plan.tile_rseg[tslot + orow + 8 * j] : -1;  // -1 on empty slots
+    }
+    const int rseg = (a.pt_a && a.seg_scale && active) ? a.plan.tile_rseg[slot] : -1;
     const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
 
     // Every load of the item is issued before anything waits for one (predicated-off loads
@@ -727,27 +741,34 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
 #endif
                           , zeros);
     }
-    u32x4 yold[NQ];
-    uint16_t* yrow = P.y + (long)(row < 0 ? 0 : row) * P.d_out + ncol0 + 8 * g;
     bool read_y = a.beta != 0.0f;
 #ifdef SMLM_TUNING
     if (a.dbg & 2) read_y = false;
 #endif
+    u32x4 yold[NQ / 2][2];
+    uint16_t* yrow[2];
 #pragma unroll
-    for (int q = 0; q < NQ; ++q)
-      yold[q] = ldg16_or(yrow + 32 * q, read_y && row >= 0 && ncol0 + 32 * q + 8 * g < P.d_out, zeros);
+    for (int j = 0; j < 2; ++j) {
+      yrow[j] = P.y + (long)(srow[j] < 0 ? 0 : srow[j]) * P.d_out + ncol0 + ocol;
+#pragma unroll
+      for (int h = 0; h < NQ / 2; ++h)
+        yold[h][j] = ldg16_or(yrow[j] + 64 * h, read_y && srow[j] >= 0 && ncol0 + 64 * h + ocol < P.d_out, zeros);
+    }
     u32x4 vf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int kk = 32 * ks + 8 * g;
       vf[ks] = ldg16_or(P.v + (long)row * P.d_in + kk, kk < P.d_in && row >= 0, zeros);
     }
-    const float scale = (rseg >= 0 && row >= 0) ? a.seg_scale[rseg] : 1.0f;
-    if (yy == 0 && active) {
+    float scale[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) scale[j] = (sseg[j] >= 0 && srow[j] >= 0) ? a.seg_scale[sseg[j]] : 1.0f;
+    if (yy == 0 && active) {  // by-products for the backward (v copy, transposed scaled copies)
+      const float sc = (rseg >= 0 && row >= 0) ? a.seg_scale[rseg] : 1.0f;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int kk = 32 * ks + 8 * g;
-        if (kk < P.d_in) write_side<DT>(a, P, slot, row, kk, vf[ks], scale);
+        if (kk < P.d_in) write_side<DT>(a, P, slot, row, kk, vf[ks], sc);
       }
     }
 
@@ -773,7 +794,48 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
           const u32x4 wf = *reinterpret_cast<const u32x4*>(&wlds[(32 * q + 4 * p + mrow) * kPitch + 32 * ks + 8 * g]);
           acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
         }
-    if (row >= 0) store_tile<DT, NQ>(yrow, ncol0 + 8 * g, P.d_out, acc, yold, scale, a.beta);
+
+    // accumulators -> LDS (this wave's area) -> full-line layout, 64 columns at a time
+    float* stg = olds[wave];
+#pragma unroll
+    for (int h = 0; h < NQ / 2; ++h) {
+#pragma unroll
+      for (int qq = 0; qq < 2; ++qq) {
+        *reinterpret_cast<f32x4*>(&stg[c * kOPitch + 32 * qq + 8 * g]) = acc[2 * h + qq][0];
+        *reinterpret_cast<f32x4*>(&stg[c * kOPitch + 32 * qq + 8 * g + 4]) = acc[2 * h + qq][1];
+      }
+      // a wave's own LDS accesses are served in order; the compiler must keep them in order too
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      f32x4 lo4[2], hi4[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        lo4[j] = *reinterpret_cast<const f32x4*>(&stg[(orow + 8 * j) * kOPitch + ocol]);
+        hi4[j] = *reinterpret_cast<const f32x4*>(&stg[(orow + 8 * j) * kOPitch + ocol + 4]);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (srow[j] < 0 || ncol0 + 64 * h + ocol >= P.d_out) continue;
+        const u32x4 old = yold[h][j];
+        const float sc = scale[j], beta = a.beta;
+        u32x4 o;
+        if (beta != 0.0f) {
+          o[0] = pack2<DT>(beta * Num<DT>::lo(old[0]) + sc * lo4[j][0], beta * Num<DT>::hi(old[0]) + sc * lo4[j][1]);
+          o[1] = pack2<DT>(beta * Num<DT>::lo(old[1]) + sc * lo4[j][2], beta * Num<DT>::hi(old[1]) + sc * lo4[j][3]);
+          o[2] = pack2<DT>(beta * Num<DT>::lo(old[2]) + sc * hi4[j][0], beta * Num<DT>::hi(old[2]) + sc * hi4[j][1]);
+          o[3] = pack2<DT>(beta * Num<DT>::lo(old[3]) + sc * hi4[j][2], beta * Num<DT>::hi(old[3]) + sc * hi4[j][3]);
+        } else {
+          o[0] = pack2<DT>(sc * lo4[j][0], sc * lo4[j][1]);
+          o[1] = pack2<DT>(sc * lo4[j][2], sc * lo4[j][3]);
+          o[2] = pack2<DT>(sc * hi4[j][0], sc * hi4[j][1]);
+          o[3] = pack2<DT>(sc * hi4[j][2], sc * hi4[j][3]);
+        }
+        stg16(yrow[j] + 64 * h, o);
+      }
+    }
   }
 }
 
