@@ -158,12 +158,12 @@ int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   return launch(shrink_kernel<DT, 4, 2, 1, NW, RM, DIRECT>, grid, block, st, a);
 }
 
-template <int DT, bool DIRECT>
+template <int DT, bool DIRECT, bool WKN>
 int launch_shrink_block(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   const dim3 block(kFwdThreads);
-  if (NB == 1) return launch(shrink_block_kernel<DT, 1, 4, DIRECT>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_block_kernel<DT, 2, 4, DIRECT>, grid, block, st, a);
-  return launch(shrink_block_kernel<DT, 4, 4, DIRECT>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_block_kernel<DT, 1, 4, DIRECT, WKN>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_kernel<DT, 2, 4, DIRECT, WKN>, grid, block, st, a);
+  return launch(shrink_block_kernel<DT, 4, 4, DIRECT, WKN>, grid, block, st, a);
 }
 
 template <int DT, bool DIRECT>
@@ -174,7 +174,8 @@ int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStrea
   if (MT == 1)
     return NW == 16 ? launch_shrink_nb<DT, 16, false, DIRECT>(NB, grid, st, a)
                     : launch_shrink_nb<DT, kFwdWaves, false, DIRECT>(NB, grid, st, a);
-  return launch_shrink_block<DT, DIRECT>(NB, grid, st, a);
+  return a.w_kn ? launch_shrink_block<DT, DIRECT, true>(NB, grid, st, a)
+                : launch_shrink_block<DT, DIRECT, false>(NB, grid, st, a);
 }
 
 // all projections of one launch share NB / U / MT / NW (same rank, same T)
@@ -224,12 +225,12 @@ int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipS
                      const ExpandArgs& a) {
   if (row_major)
     return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
-  if (block && nq == 8)
-    return KS == 1 ? launch(expand_block_kernel<DT, 8, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
-                   : launch(expand_block_kernel<DT, 8, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
+  if (block && a.w_kn)
+    return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, true>, grid, dim3(kFwdThreads), st, a)
+                   : launch(expand_block_kernel<DT, 4, 2, DIRECT, true>, grid, dim3(kFwdThreads), st, a);
   if (block)
-    return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT>, grid, dim3(kFwdThreads), st, a)
-                   : launch(expand_block_kernel<DT, 4, 2, DIRECT>, grid, dim3(kFwdThreads), st, a);
+    return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, false>, grid, dim3(kFwdThreads), st, a)
+                   : launch(expand_block_kernel<DT, 4, 2, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
   const bool vfold = a.p[0].vsplit > 0;  // set for all projections of a launch or for none
   return nq == 4 ? launch_expand_wave<DT, 4, DIRECT>(KS, vfold, grid, st, a)
                  : launch_expand_wave<DT, 2, DIRECT>(KS, vfold, grid, st, a);
@@ -243,7 +244,7 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   if (row_major) nq = 2;
   if (block) nq = 4;
   nq = tune("SMLM_TUNE_NQ", nq);
-  if (block && nq != 8) nq = 4;
+  if (block) nq = 4;
   const int chunk = block ? 32 * nq : kFwdWaves * 32 * nq;  // columns per workgroup
   a.items.nproj = nproj;
 #ifdef SMLM_TUNING
@@ -297,8 +298,9 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
-               const float* seg_scale, hipStream_t st, bool fold = true) {
+               const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false) {
   ShrinkArgs a{};
+  a.w_kn = w_kn ? 1 : 0;
   a.plan = tile_args(pv);
   a.seg_scale = seg_scale;
   a.beta = beta;
@@ -670,12 +672,15 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   PlanView pv{};
   plan_carve(const_cast<void*>(plan), n_rows, P, &pv);
 
-  // 1. transposed copies of the training adapters' weights: At [h_in, r], Bt [r, h_out]
-  TransposeArgs ta{};
-  ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
-  ta.set[1] = TransposeSet{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
-  ta.NA = NA;
-  {
+  // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The
+  // tile-block kernels (1024 rows and more) read the weights as they lie in memory; smaller
+  // batches work on transposed copies At [h_in, r], Bt [r, h_out] made here.
+  const bool in_place = tiles_per_wave(n_rows) > 1;
+  if (!in_place) {
+    TransposeArgs ta{};
+    ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
+    ta.set[1] = TransposeSet{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
+    ta.NA = NA;
     const int gx = ceil_div(h_in > h_out ? h_in : h_out, 64), gy = ceil_div(r, 64);
     if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
   }
@@ -690,9 +695,10 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   }
 
   // 3. dV = round16(dY B)
-  const void* const* btp = bt_ptrs;
-  if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &h_out,
-                       0.0f, nullptr, st)))
+  const void* const* btp = in_place ? b_ptrs : bt_ptrs;
+  const int b_ld = in_place ? r : h_out;
+  if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
+                       0.0f, nullptr, st, true, in_place)))
     return rc;
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
@@ -708,9 +714,10 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
     ExpandProj& E = ea.p[0];
     E.y = reinterpret_cast<uint16_t*>(dx);
     E.v = reinterpret_cast<const uint16_t*>(dv16);
-    E.w_ptrs = at_ptrs;
-    E.d_in = r; E.d_out = h_in; E.ldw = r;
+    E.w_ptrs = in_place ? a_ptrs : at_ptrs;
+    E.d_in = r; E.d_out = h_in; E.ldw = in_place ? h_in : r;
   }
+  ea.w_kn = in_place ? 1 : 0;
   if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, NA, 1, r, st,
                           ea)))
     return rc;

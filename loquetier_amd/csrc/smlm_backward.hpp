@@ -24,15 +24,6 @@ struct TransposeArgs {
 
 constexpr int kTrPitch = 80;  // LDS row pitch in 16-bit elements (40 banks: see kWgPitch)
 
-// Transposing LDS read of gfx950: within each 16 lanes, lane i names a "row" of
-// four 16-bit elements M[i][0..3]; lane 4a+b receives M[a][b], M[4+a][b],
-// M[8+a][b], M[12+a][b].
-typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 lds_tr_f16x4;
-__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_addr) {
-  typedef __attribute__((address_space(3))) lds_tr_f16x4 lds_vec;
-  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_vec*)lds_addr));
-}
-
 // 64x64 tiles through LDS, 16-byte global accesses on both sides: rows of the
 // source tile are written to LDS as they are and read back down the columns
 // with the transposing LDS read.  grid (tiles along the hidden dimension, tiles

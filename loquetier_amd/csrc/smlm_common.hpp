@@ -102,6 +102,15 @@ __device__ __forceinline__ u32x4 ldg16_or(const uint16_t* p, bool ok, const uint
 }
 constexpr int kHdrZeros = 12;  // header words 12..15 are always zero
 
+// Transposing LDS read of gfx950: within each 16 lanes, lane i names a "row" of
+// four 16-bit elements M[i][0..3]; lane 4a+b receives M[a][b], M[4+a][b],
+// M[8+a][b], M[12+a][b].
+typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 lds_tr_f16x4;
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_addr) {
+  typedef __attribute__((address_space(3))) lds_tr_f16x4 lds_vec;
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_vec*)lds_addr));
+}
+
 // Reads of plan tables and pointer tables at a wave-uniform index.  These are
 // written by an earlier kernel and never by the kernel that reads them, so they
 // may go through the scalar (constant) path: the loads then cost no vector

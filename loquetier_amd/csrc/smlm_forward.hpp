@@ -173,6 +173,7 @@ struct ShrinkProj {
   int to_partial;             // write the fp32 partial even when ksplit == 1 (the consumer rounds)
 };
 
+
 struct ShrinkArgs {
   TileArgs plan;
   ShrinkProj p[kMaxProj];
@@ -180,6 +181,7 @@ struct ShrinkArgs {
   float beta;
   int T;
   ItemSpace items;            // chunk rows of projection p: ksplit*zblocks
+  int w_kn;                   // tile-block kernel only: weights are stored [k][n]
 #ifdef SMLM_TUNING
   int dbg;                    // experiments: 1 = no weight loads, 2 = no x loads, 4 = no partial/output store
 #endif
@@ -359,14 +361,19 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 // four tiles, while every wave loads the x fragments of its own tile straight into
 // registers one batch ahead.  Against the kernel above with MT = 4 this reads the weights
 // from L2 once per workgroup instead of once per wave and needs no cross-wave sum.
-template <int DT, int NB, int U, bool DIRECT>
+//
+// WKN: the weight matrices are stored [k][n] (k rows of d_out contiguous columns, as B
+// [h_out, r] is for the backward's dV = dY B) instead of [n][k]: a batch is then staged as
+// it lies in memory and the MFMA operand, which wants eight consecutive k of one column,
+// is read out of LDS with the transposing read.
+template <int DT, int NB, int U, bool DIRECT, bool WKN>
 __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a) {
   constexpr int KB = 32 * U;                 // k per batch
-  constexpr int kPitch = KB + 8;             // LDS row pitch: rows 16 bytes apart mod 128
   constexpr int kRowsW = 16 * NB;            // weight rows (output columns) per workgroup
+  constexpr int kPitch = WKN ? kRowsW + 8 : KB + 8;  // LDS row pitch in elements
   constexpr int kPieces = kRowsW * (KB / 8); // 16-byte pieces of one staged batch
   constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
-  __shared__ __attribute__((aligned(16))) uint16_t wlds[2][kRowsW * kPitch];
+  __shared__ __attribute__((aligned(16))) uint16_t wlds[2][(WKN ? KB : kRowsW) * kPitch];
   const int units = DIRECT ? 0 : tile_units<kBlkTiles>(a.plan, 0);
   const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -401,18 +408,35 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
 #pragma unroll
       for (int j = 0; j < kPer; ++j) {
         const int idx = threadIdx.x + j * kFwdThreads;
-        const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
-        st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
-                         idx < kPieces && n0 + nl < P.d_out && kb + k8 < kend, zeros);
+        if (WKN) {
+          const int kl = idx / (kRowsW / 8), n8 = (idx % (kRowsW / 8)) * 8;
+          st[j] = ldg16_or(W + (long)(kb + kl) * P.ldw + n0 + n8,
+                           idx < kPieces && n0 + n8 < P.d_out && kb + kl < kend, zeros);
+        } else {
+          const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
+          st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
+                           idx < kPieces && n0 + nl < P.d_out && kb + k8 < kend, zeros);
+        }
       }
     };
     auto stage_w = [&](int buf, const u32x4 (&st)[kPer]) {
 #pragma unroll
       for (int j = 0; j < kPer; ++j) {
         const int idx = threadIdx.x + j * kFwdThreads;
-        const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
-        if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[buf][nl * kPitch + k8]) = st[j];
+        const int r_ = WKN ? idx / (kRowsW / 8) : idx / (KB / 8);
+        const int c_ = WKN ? (idx % (kRowsW / 8)) * 8 : (idx % (KB / 8)) * 8;
+        if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[buf][r_ * kPitch + c_]) = st[j];
       }
+    };
+    auto weight_frag = [&](int buf, int u, int nb) -> u32x4 {
+      if (WKN) {
+        // lane c names k row 32u + 8g (+4) + c/4 and columns 16nb + 4(c%4) .. +3; it receives
+        // column 16nb + c of four consecutive k rows per read
+        const uint16_t* base = &wlds[buf][(32 * u + 8 * g + (c >> 2)) * kPitch + 16 * nb + 4 * (c & 3)];
+        const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 4 * kPitch);
+        return u32x4{q0[0], q0[1], q1[0], q1[1]};
+      }
+      return *reinterpret_cast<const u32x4*>(&wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
     };
 
     f32x4 acc[NB];
@@ -437,8 +461,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
         for (int u = 0; u < U; ++u)
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
-            const u32x4 wf = *reinterpret_cast<const u32x4*>(&wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
-            acc[nb] = Num<DT>::mfma(wf, xf[u], acc[nb]);
+            acc[nb] = Num<DT>::mfma(weight_frag(buf, u, nb), xf[u], acc[nb]);
           }
       }
       stage_w(buf ^ 1, wn);
@@ -536,6 +559,7 @@ struct ExpandArgs {
   float beta;
   int T, nt_max;
   ItemSpace items;           // chunk rows of projection p: its column chunks
+  int w_kn;                  // tile-block kernel only: weights are stored [k][n]
 #ifdef SMLM_TUNING
   int dbg;                   // experiments: 1 = no weights / multiply, 2 = no read of y
 #endif
@@ -738,11 +762,13 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 // stages the chunk's weight rows in LDS once; wave w then multiplies tile w of
 // the block with them, so an adapter's B chunk is read from L2 once per four
 // tiles instead of once per tile.
-template <int DT, int NQ, int KS, bool DIRECT>
+// WKN: weights stored [k][n] (A [r, h_in] for the backward's dX = dV A): the chunk is staged
+// as it lies in memory and read out of LDS with the transposing read.
+template <int DT, int NQ, int KS, bool DIRECT, bool WKN>
 __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a) {
   static_assert(NQ % 2 == 0, "the output is written 64 columns at a time");
-  constexpr int kPitch = 32 * KS + 8;  // LDS row pitch in 16-bit elements: rows 16 bytes apart mod 128
-  __shared__ __attribute__((aligned(16))) uint16_t wlds[32 * NQ * kPitch];
+  constexpr int kPitch = WKN ? 32 * NQ + 8 : 32 * KS + 8;  // LDS row pitch in 16-bit elements
+  __shared__ __attribute__((aligned(16))) uint16_t wlds[(WKN ? 32 * KS : 32 * NQ) * kPitch];
   __shared__ __attribute__((aligned(16))) float olds[kFwdWaves][kTileRows * kOPitch];
   const int units = DIRECT ? 0 : tile_units<kBlkTiles>(a.plan, 0);
   const WorkRange wr = item_range<DIRECT>(a.items, units);
@@ -785,13 +811,19 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int idx = threadIdx.x + j * kFwdThreads;
-      const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
-      stage[j] = ldg16_or(W + (long)(ncol0 + nl) * P.ldw + k8,
-                          idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in
+      if (WKN) {
+        const int kl = idx / (4 * NQ), n8 = (idx % (4 * NQ)) * 8;
+        stage[j] = ldg16_or(W + (long)kl * P.ldw + ncol0 + n8,
+                            idx < kPieces && ncol0 + n8 < P.d_out && kl < P.d_in, zeros);
+      } else {
+        const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
+        stage[j] = ldg16_or(W + (long)(ncol0 + nl) * P.ldw + k8,
+                            idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in
 #ifdef SMLM_TUNING
-                              && !(a.dbg & 1)
+                                && !(a.dbg & 1)
 #endif
-                          , zeros);
+                            , zeros);
+      }
     }
     bool read_y = a.beta != 0.0f;
 #ifdef SMLM_TUNING
@@ -820,8 +852,9 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int idx = threadIdx.x + j * kFwdThreads;
-      const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
-      if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[nl * kPitch + k8]) = stage[j];
+      const int r_ = WKN ? idx / (4 * NQ) : idx / (4 * KS);
+      const int c_ = WKN ? (idx % (4 * NQ)) * 8 : (idx % (4 * KS)) * 8;
+      if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[r_ * kPitch + c_]) = stage[j];
     }
     __syncthreads();
     if (!active) continue;  // whole waves only (MFMA runs with every lane); barriers are behind us
@@ -835,7 +868,16 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
       for (int q = 0; q < NQ; ++q)
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-          const u32x4 wf = *reinterpret_cast<const u32x4*>(&wlds[(32 * q + 4 * p + mrow) * kPitch + 32 * ks + 8 * g]);
+          u32x4 wf;
+          if (WKN) {
+            // lane c names k row 32ks + 8g (+4) + c/4 and columns 32q + 4p + 8(c%4) .. +3; it
+            // receives column 32q + 4p + 8(c/4) + c%4 (its MFMA row's column) of four k rows
+            const uint16_t* base = &wlds[(32 * ks + 8 * g + (c >> 2)) * kPitch + 32 * q + 4 * p + 8 * (c & 3)];
+            const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 4 * kPitch);
+            wf = u32x4{q0[0], q0[1], q1[0], q1[1]};
+          } else {
+            wf = *reinterpret_cast<const u32x4*>(&wlds[(32 * q + 4 * p + mrow) * kPitch + 32 * ks + 8 * g]);
+          }
           acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
         }
 
