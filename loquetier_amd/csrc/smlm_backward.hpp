@@ -110,7 +110,7 @@ template <int DT, int NBJ, int NW, bool IS_A>
 __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   constexpr int kWgWaves = NW;
   constexpr int kStageElems = kWgSlots * kWgPitch;
-  constexpr int kStageBytes = kWgWaves * kStageElems * 2;
+  constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
 
   const int ad = blockIdx.y;
   constexpr bool is_a = IS_A;
@@ -118,8 +118,6 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   const int h = is_a ? a.h_in : a.h_out;
   const uint16_t* Q = is_a ? a.q_a : a.q_b;
   const uint16_t* PT = is_a ? a.pt_a : a.pt_b;
-  // an address read from a table has no known address space; say it is global
-  typedef __attribute__((address_space(1))) u32x2 global_u32x2;
   uint16_t* out = reinterpret_cast<uint16_t*>(is_a ? a.da_ptrs[ad] : a.db_ptrs[ad]);
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -240,47 +238,92 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
     for (int jb = 0; jb < NBJ; ++jb) pf[jb][0] = pf_next[jb][0], pf[jb][1] = pf_next[jb][1];
   }
 
-  // cross-wave sum in wave order, one rank block at a time, then store
+  // cross-wave sum in wave order, one rank block at a time; wave 0 ends up with the totals
   f32x4(*red)[4][kWaveSize] = reinterpret_cast<f32x4(*)[4][kWaveSize]>(smem);
-  if (NW > 1) __syncthreads();  // every wave is done with its staging area, which red overlays
-  for (int jb = 0; jb < NBJ; ++jb) {
-    if (NW > 1) {
+  if (NW > 1) {
+    __syncthreads();  // every wave is done with its staging area, which red overlays
+    for (int jb = 0; jb < NBJ; ++jb) {
 #pragma unroll
       for (int nb = 0; nb < 4; ++nb) red[wave][nb][lane] = acc[jb][nb];
       __syncthreads();
-    }
-    if (wave == 0) {
+      if (wave == 0) {
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) {
-        f32x4 s = acc[jb][nb];
-        if (NW > 1) {
-          s = red[0][nb][lane];
+        for (int nb = 0; nb < 4; ++nb) {
+          f32x4 part[kWgWaves];
 #pragma unroll
-          for (int w = 1; w < kWgWaves; ++w) s += red[w][nb][lane];
-        }
-        u32x2 o;
-        o[0] = pack2<DT>(s[0], s[1]);
-        o[1] = pack2<DT>(s[2], s[3]);
-        if (is_a) {
-          // D[m = x column 16nb + 4g + i][n = rank 16jb + c]
-          const int j = 16 * jb + c, n = n0 + 16 * nb + 4 * g;
-          if (j < a.r && n < h) *(global_u32x2*)(out + (long)j * h + n) = o;
-        } else {
-          // D[m = rank 16jb + 4g + i][n = dY column 16nb + c]
-          const int j = 16 * jb + 4 * g, n = n0 + 16 * nb + c;
-          if (j < a.r && n < h) *(global_u32x2*)(out + (long)n * a.r + j) = o;
+          for (int w = 0; w < kWgWaves; ++w) part[w] = red[w][nb][lane];
+          f32x4 sum = part[0];
+#pragma unroll
+          for (int w = 1; w < kWgWaves; ++w) sum += part[w];
+          acc[jb][nb] = sum;
         }
       }
+      __syncthreads();
     }
-    if (NW > 1) __syncthreads();
+    if (wave != 0) return;  // no barrier follows
+  }
+
+  // Store.  The MFMA leaves 32-byte pieces per output row; the totals go through LDS once
+  // more (an area of their own behind `red`) so that every store instruction writes full
+  // rows: lane -> output row lane/8 (+8), eight elements at (lane%8)*8.
+  constexpr int kSPitch = 64 + 4;  // floats; conflict-free for the writes below and the reads
+  float* sto = reinterpret_cast<float*>(smem + (NW > 1 ? kRedBytes : 0));
+  const int orow = lane >> 3, ocol = (lane & 7) * 8;
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto read_and_pack = [&](int row) -> u32x4 {
+    const f32x4 lo4 = *reinterpret_cast<const f32x4*>(&sto[row * kSPitch + ocol]);
+    const f32x4 hi4 = *reinterpret_cast<const f32x4*>(&sto[row * kSPitch + ocol + 4]);
+    return u32x4{pack2<DT>(lo4[0], lo4[1]), pack2<DT>(lo4[2], lo4[3]), pack2<DT>(hi4[0], hi4[1]),
+                 pack2<DT>(hi4[2], hi4[3])};
+  };
+  if (is_a) {
+    // dA [r, h]: per rank block, 16 rank rows x 64 columns; lane (c, g) holds rank row c,
+    // columns 16nb + 4g .. +3
+#pragma unroll
+    for (int jb = 0; jb < NBJ; ++jb) {
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * nb + 4 * g]) = acc[jb][nb];
+      wave_sync();
+      u32x4 o[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) o[i] = read_and_pack(orow + 8 * i);
+      wave_sync();
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int j = 16 * jb + orow + 8 * i, n = n0 + ocol;
+        if (j < a.r && n < h) stg16(out + (long)j * h + n, o[i]);
+      }
+    }
+  } else {
+    // dB [h, r]: per 16 columns of dY (output rows), all ranks; lane (c, g) holds output row
+    // 16nb + c, ranks 16jb + 4g .. +3
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+#pragma unroll
+      for (int jb = 0; jb < NBJ; ++jb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * jb + 4 * g]) = acc[jb][nb];
+      wave_sync();
+      u32x4 o[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) o[i] = read_and_pack(orow + 8 * i);
+      wave_sync();
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int n = n0 + 16 * nb + orow + 8 * i;
+        if (ocol < a.r && n < h) stg16(out + (long)n * a.r + ocol, o[i]);
+      }
+    }
   }
 }
 
 template <int DT, int NBJ, int NW>
 __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
   constexpr int kStageBytes = NW * kWgSlots * kWgPitch * 2;
-  constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
-  __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+  constexpr int kTailBytes = (NW > 1 ? NW * 4 * kWaveSize * 16 : 0) + 16 * (64 + 4) * 4;  // red + store staging
+  __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kTailBytes ? kStageBytes : kTailBytes];
   if ((int)blockIdx.x < a.chunks_a)  // uniform over the workgroup
     wgrad_body<DT, NBJ, NW, true>(a, smem);
   else
