@@ -227,6 +227,8 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
 
   SMLM_TICK();
   // gathered-row position of every sorted segment, group heads
+  int32_t* gpos = len0;  // group -> sorted position of its first segment (len0 is read before the scan
+                         // below, gpos written after it)
   constexpr uint64_t kRowMask = 0xffffffffull;  // rows in the low half, group heads in the high half
   int seg = 0, len = 0;
   uint64_t gk = 0;
@@ -254,11 +256,13 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
       grow[G] = rows_before;
       gseg[G] = seg;
       gid[G] = (int32_t)(uint32_t)gk;
+      gpos[G] = tid;
     }
   }
   if (tid == 0) {
     rowpos[S] = rows_total;
     grow[NG] = rows_total;
+    gpos[NG] = S;
     pv.rowpos[S] = rows_total;
   }
   __syncthreads();
@@ -297,6 +301,10 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   __syncthreads();
 
   SMLM_TICK();
+  // tile -> group table (the sort keys' first copy is free by now)
+  uint16_t* gt = reinterpret_cast<uint16_t*>(K0);
+  for (int tile = tid; tile < n_tiles; tile += blockDim.x) gt[tile] = (uint16_t)last_le(gtile, NG, tile);
+  __syncthreads();
   // tile blocks; entries past the last one say "no tiles" (kernels launched over an
   // upper bound of the block count stop there without reading the header)
   for (int b = tid; b < pv.nt_max; b += blockDim.x) {
@@ -310,15 +318,18 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     pv.blk[b] = packed;
   }
 
-  // fill: one thread per tile slot; tiles past the last one get weight index -1
+  // fill: one thread per tile slot; tiles past the last one get weight index -1.  The group
+  // of a tile comes from the table above and the segment of a row is searched among the
+  // group's own segments only, which keeps the chains of dependent LDS reads short.
   for (int tile = n_tiles + tid; tile < pv.nt_max; tile += blockDim.x) pv.tile_wid[tile] = -1;
   for (int slot = tid; slot < n_tiles * kTileRows; slot += blockDim.x) {
     const int tile = slot / kTileRows, c = slot % kTileRows;
-    const int G = last_le(gtile, NG, tile);
+    const int G = gt[tile];
     const int q = grow[G] + (tile - gtile[G]) * kTileRows + c;
     int row = -1, rseg = -1;
     if (q < grow[G + 1]) {
-      const int a = last_le(rowpos, S, q);
+      const int a0 = gpos[G];
+      const int a = a0 + last_le(rowpos + a0, gpos[G + 1] - a0, q);
       rseg = sseg[a];
       row = start0[rseg] + (q - rowpos[a]);
     }
