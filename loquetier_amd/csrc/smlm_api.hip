@@ -153,9 +153,9 @@ inline dim3 item_grid(const ItemSpace& sp, long items) {
 template <int DT, int NW, bool RM, bool DIRECT>
 int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   const dim3 block(NW * kWaveSize);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, 1, NW, RM, DIRECT>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, 1, NW, RM, DIRECT>, grid, block, st, a);
-  return launch(shrink_kernel<DT, 4, 2, 1, NW, RM, DIRECT>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, NW, RM, DIRECT>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, NW, RM, DIRECT>, grid, block, st, a);
+  return launch(shrink_kernel<DT, 4, 2, NW, RM, DIRECT>, grid, block, st, a);
 }
 
 template <int DT, bool DIRECT, bool WKN>

@@ -1,26 +1,25 @@
 // Shrink (skinny-N, long-K) and expand (skinny-K, wide-N) tile kernels.
 //
 // Both take the place of the CUTLASS GemmGrouped instantiations of
-// kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:84-171.  One wave owns
-// up to MT 16-row plan tiles of one adapter and drives v_mfma_f32_16x16x32 with
-// the tokens as the MFMA *columns* and the weight rows as the MFMA *rows*: each
-// lane then ends up with consecutive output columns of one token, which is what
-// a coalesced store of y needs.  Operand fragments are 16-byte global loads
-// straight into registers (x and the weights are both contiguous along the
-// contraction); a weight fragment is loaded once and used for all MT tiles.
+// kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:84-171.  The unit of
+// work is a 16-row plan tile of one adapter (or a tile block of up to four).
+// v_mfma_f32_16x16x32 runs with the tokens as the MFMA *columns* and the weight
+// rows as the MFMA *rows*, so a lane ends up with consecutive output columns of
+// one token.  x fragments are 16-byte global loads straight into registers (x
+// is contiguous along the contraction); weight fragments come straight from
+// global memory in the one-tile kernels and from an LDS-staged chunk shared by
+// the tiles of a block in the tile-block kernels.
 //
 // Every output element is produced by the same sequence of MFMA steps over k
-// whatever other rows share its tile or its wave, so regrouping or
+// whatever other rows share its tile or its workgroup, so regrouping or
 // re-segmenting rows never changes a bit of any row.
 //
-// Launches are one-dimensional and persistent: the number of work items (tiles
-// x column chunks | k slices x projections) is only known on the device, in the
-// plan header, so a fixed grid walks the items.  Workgroups are handed to the 8
-// XCDs round robin by their linear id, and each XCD has its own L2; work_range()
-// gives each XCD one contiguous range of (projection, column chunk | k slice,
-// tile block) items: all tile blocks that read one slice of an adapter's weights
-// run on the same XCD close in time, so that slice is fetched from HBM once
-// instead of once per XCD.
+// The number of tiles is only known on the device (plan header).  Launches are
+// sized on the host over an upper bound of it, one work item per workgroup
+// ("direct" mode); items past the real count find an empty entry in the plan
+// and leave.  A persistent one-dimensional walk over the exact count (one
+// contiguous range of items per XCD, or plain round robin) remains as the
+// fallback for batches beyond the direct grid's limits.
 #pragma once
 #include "smlm_common.hpp"
 
@@ -173,7 +172,6 @@ struct ShrinkProj {
   int to_partial;             // write the fp32 partial even when ksplit == 1 (the consumer rounds)
 };
 
-
 struct ShrinkArgs {
   TileArgs plan;
   ShrinkProj p[kMaxProj];
@@ -187,70 +185,49 @@ struct ShrinkArgs {
 #endif
 };
 
-// Work item -> (projection, k slice, 64-column block, tile block).  The NW
-// waves of a workgroup take consecutive k ranges; their accumulators are summed
-// through LDS in wave order and written either as an fp32 partial (ksplit > 1)
-// or as the final 16-bit value.  NW = 16 lets one workgroup cover all of k, so
-// no partial sums leave the CU.
-template <int DT, int NB, int U, int MT, int NW, bool ROWMAJOR, bool DIRECT>
+// Shrink for single tiles (batches below 1024 rows).  Work item -> (projection, k
+// slice, 64-column block, tile).  The NW waves of a workgroup take consecutive k
+// ranges; their accumulators are summed through LDS in wave order and written
+// either as an fp32 partial (k split over workgroups, or a consumer that folds)
+// or as the final 16-bit value.  NW = 16 is for decode batches: few tiles, long k.
+template <int DT, int NB, int U, int NW, bool ROWMAJOR, bool DIRECT>
 __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
-  constexpr int TP = (MT * NB > 8) ? 8 / NB : MT;  // tiles per cross-wave reduction pass
-  __shared__ f32x4 red[NW][TP][NB][kWaveSize];
-  const int units = DIRECT ? 0 : tile_units<MT>(a.plan, 0);
+  __shared__ f32x4 red[NW][NB][kWaveSize];
+  const int units = DIRECT ? 0 : tile_units<1>(a.plan, 0);
   const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
 
-#ifdef SMLM_TUNING
-  long long tick[6];
-  tick[0] = wall_clock64();
-#define SMLM_TICK(i) tick[i] = wall_clock64()
-#else
-#define SMLM_TICK(i) do {} while (0)
-#endif
   for (int V = wr.first; V < wr.last; V += wr.step) {
-    int pj, yy, tb;
-    if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tb)) break;
+    int pj, yy, tile;
+    if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tile)) break;
     const ShrinkProj P = a.p[pj];
     const int kz = yy % P.ksplit, zb = yy / P.ksplit;
-    int t0, cnt, wid;
-    pick_tiles<MT>(a.plan, tb, &t0, &cnt, &wid);
-    if (cnt == 0) continue;  // uniform over the workgroup
+    const int wid = uload(a.plan.tile_wid, tile);
+    if (wid < 0) continue;  // past the last tile (direct mode); uniform over the workgroup
     const int n0 = zb * 64;
-
-    int row[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) row[i] = i < cnt ? a.plan.tile_row[(t0 + i) * kTileRows + c] : -1;
+    const int slot = tile * kTileRows + c;
+    const int row = a.plan.tile_row[slot];
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
-#ifdef SMLM_TUNING
-    SMLM_TICK(1);
-    if (row[0] == -12345 || W == nullptr) continue;  // keeps the tick after the metadata loads
-#endif
 
     const int kbeg = (kz * NW + wave) * P.k_per_wave;
     const int kend = min(kbeg + P.k_per_wave, P.d_in);
     const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
 
-    f32x4 acc[MT][NB];
+    f32x4 acc[NB];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // k loop, two load batches in turn: the loads of one batch are on their way while the
-    // other batch is multiplied
-    auto load_batch = [&](int k, u32x4 (&xf)[MT][U], u32x4 (&wf)[NB][U]) {
+    auto load_batch = [&](int k, u32x4 (&xf)[U], u32x4 (&wf)[NB][U]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int kk = k + 32 * u + 8 * g;
         const bool kin = kk < kend;
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-          xf[i][u] = ldg16_or(P.x + (long)row[i] * P.d_in + kk, kin && row[i] >= 0
+        xf[u] = ldg16_or(P.x + (long)row * P.d_in + kk, kin && row >= 0
 #ifdef SMLM_TUNING
-                                                                         && !(a.dbg & 2)
+                                                            && !(a.dbg & 2)
 #endif
-                              , zeros);
+                         , zeros);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const int n = n0 + 16 * nb + c;
@@ -262,18 +239,15 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         }
       }
     };
-    auto multiply = [&](const u32x4 (&xf)[MT][U], const u32x4 (&wf)[NB][U]) {
+    auto multiply = [&](const u32x4 (&xf)[U], const u32x4 (&wf)[NB][U]) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-          if (i < cnt) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) acc[i][nb] = Num<DT>::mfma(wf[nb][u], xf[i][u], acc[i][nb]);
-          }
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(wf[nb][u], xf[u], acc[nb]);
     };
     if (NW < 16) {
-      u32x4 xa[MT][U], wa[NB][U], xb[MT][U], wb[NB][U];
+      // two load batches in turn: one is on its way while the other is multiplied
+      u32x4 xa[U], wa[NB][U], xb[U], wb[NB][U];
       load_batch(kbeg, xa, wa);
 #pragma unroll 1
       for (int k = kbeg; k < kend; k += 64 * U) {
@@ -287,71 +261,45 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
     } else {  // sixteen waves share the VGPR file: one batch at a time (k is usually one batch)
 #pragma unroll 1
       for (int k = kbeg; k < kend; k += 32 * U) {
-        u32x4 xf[MT][U], wf[NB][U];
+        u32x4 xf[U], wf[NB][U];
         load_batch(k, xf, wf);
         multiply(xf, wf);
       }
     }
 
+    // cross-wave sum in wave order; wave 0 writes the tile
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) red[wave][nb][lane] = acc[nb];
+    __syncthreads();
+    if (wave == 0 && row >= 0) {
+      float scale = 1.0f;
+      const bool as_partial = P.ksplit > 1 || P.to_partial;
+      if (!as_partial && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        // all NW reads are issued before the first add waits for one (left to itself the
+        // compiler keeps two in flight, and the sixteen-wave kernel spends as long here as
+        // in its k loop)
+        f32x4 part[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) part[w] = red[w][nb][lane];
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 sum = part[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sum += part[w];
+        const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
+        if (n >= P.d_out) continue;
 #ifdef SMLM_TUNING
-    SMLM_TICK(2);
-    if (acc[0][0][0] == -12345.678f) continue;  // keeps the tick after the MFMA loop
+        if ((a.dbg & 4) && sum[0] != 12345.f) continue;
 #endif
-    // cross-wave sum, TP tiles per pass, wave j finishing tile j of the pass
-#pragma unroll
-    for (int pass = 0; pass < MT / TP; ++pass) {
-      if (pass * TP >= cnt) break;  // uniform over the workgroup
-#pragma unroll
-      for (int j = 0; j < TP; ++j)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) red[wave][j][nb][lane] = acc[pass * TP + j][nb];
-      __syncthreads();
-      const int i = pass * TP + wave;
-      if (wave < TP && i < cnt) {
-        const int slot = (t0 + i) * kTileRows + c;
-        int r = row[0];  // row of tile i, picked from registers
-#pragma unroll
-        for (int j = 1; j < MT; ++j) r = (i == j) ? row[j] : r;
-        if (r >= 0) {
-          float scale = 1.0f;
-          const bool as_partial = P.ksplit > 1 || P.to_partial;
-          if (!as_partial && a.seg_scale) scale = a.seg_scale[a.plan.tile_rseg[slot]];
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            // all NW reads are issued before the first add waits for one (left to itself the
-            // compiler keeps two in flight, and the sixteen-wave kernel spends as long here
-            // as in its k loop)
-            f32x4 part[NW];
-#pragma unroll
-            for (int w = 0; w < NW; ++w) part[w] = red[w][wave][nb][lane];
-            __builtin_amdgcn_sched_barrier(0);
-            f32x4 sum = part[0];
-#pragma unroll
-            for (int w = 1; w < NW; ++w) sum += part[w];
-            const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
-            if (n >= P.d_out) continue;
-#ifdef SMLM_TUNING
-            if ((a.dbg & 4) && sum[0] != 12345.f) continue;
-#endif
-            if (as_partial)
-              *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + r) * P.d_out + n) = sum;
-            else
-              store4<DT>(P.out + (long)r * P.d_out + n, sum, scale, a.beta);
-          }
-        }
+        if (as_partial)
+          *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + row) * P.d_out + n) = sum;
+        else
+          store4<DT>(P.out + (long)row * P.d_out + n, sum, scale, a.beta);
       }
-      __syncthreads();
     }
-
-#ifdef SMLM_TUNING
-    SMLM_TICK(3);
-    if (threadIdx.x == 0 && blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0) {
-      int32_t* dbg = const_cast<int32_t*>(a.plan.hdr);
-      for (int i = 1; i < 4; ++i) dbg[8 + i - 1] = (int)(tick[i] - tick[i - 1]);
-    }
-#endif
+    __syncthreads();  // red is free again (persistent walk)
   }
-#undef SMLM_TICK
 }
 
 // Shrink for tile blocks (batches of 1024 rows and more).  Work item -> (projection, k
@@ -359,8 +307,8 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 // and all four waves walk the whole k slice together: each 32*U-wide batch of the weight
 // rows is staged once in LDS (two buffers in turn, one barrier a batch) and shared by the
 // four tiles, while every wave loads the x fragments of its own tile straight into
-// registers one batch ahead.  Against the kernel above with MT = 4 this reads the weights
-// from L2 once per workgroup instead of once per wave and needs no cross-wave sum.
+// registers one batch ahead.  The weights are read from L2 once per workgroup, not once per
+// wave, and there is no cross-wave sum.
 //
 // WKN: the weight matrices are stored [k][n] (k rows of d_out contiguous columns, as B
 // [h_out, r] is for the backward's dV = dY B) instead of [n][k]: a batch is then staged as

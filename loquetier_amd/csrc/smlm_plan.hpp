@@ -159,14 +159,6 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   __shared__ int bad_key, wide_key;
   const PlanView pv = args.pv;
   const int S = args.S, tid = threadIdx.x;  // blockDim.x >= S
-#ifdef SMLM_TUNING
-  long long tick[8];
-  int ntick = 0;
-#define SMLM_TICK() do { __syncthreads(); tick[ntick++] = wall_clock64(); } while (0)
-#else
-#define SMLM_TICK() do {} while (0)
-#endif
-  SMLM_TICK();
 
   uint64_t raw = 0;
   int s0 = 0, s1 = 0;
@@ -188,7 +180,6 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     len0[tid] = s1 > s0 ? s1 - s0 : 0;
   }
   __syncthreads();
-  SMLM_TICK();
   const int kind = bad_key ? SMLM_KEY_NONE : args.key_kind;
   uint64_t mine = ~0ull;
   if (tid < S) {
@@ -225,7 +216,6 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   }
   __syncthreads();
 
-  SMLM_TICK();
   // gathered-row position of every sorted segment, group heads
   int32_t* gpos = len0;  // group -> sorted position of its first segment (len0 is read before the scan
                          // below, gpos written after it)
@@ -300,7 +290,6 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   }
   __syncthreads();
 
-  SMLM_TICK();
   // tile -> group table (the sort keys' first copy is free by now)
   uint16_t* gt = reinterpret_cast<uint16_t*>(K0);
   for (int tile = tid; tile < n_tiles; tile += blockDim.x) gt[tile] = (uint16_t)last_le(gtile, NG, tile);
@@ -337,12 +326,6 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     pv.tile_rseg[slot] = rseg;
     if (c == 0) pv.tile_wid[tile] = (kind == SMLM_KEY_I32) ? gid[G] : gseg[G];
   }
-  SMLM_TICK();
-#ifdef SMLM_TUNING
-  if (tid == 0)
-    for (int i = 1; i < ntick; ++i) pv.hdr[8 + i - 1] = (int)(tick[i] - tick[i - 1]);
-#endif
-#undef SMLM_TICK
 }
 
 // --------------------------------------------------------------- two launches
