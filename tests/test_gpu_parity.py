@@ -403,6 +403,19 @@ def test_forward_dyadic_bit_exact_decode_route(K, oracle, gpu_device, shape, dt)
     _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
 
 
+def test_forward_beyond_the_direct_grid(K, oracle, gpu_device):
+    """More than 65535 tile units: the launches fall back to the persistent walk over the
+    plan's exact tile count (and the plan to its two-launch route).  Bit-exact on dyadic
+    inputs, narrow matrices so that a million rows stay small."""
+    T, S, NA, h_in, h_out, r, dt = 1_050_000, 64, 5, 64, 64, 8, "bf16"
+    rng = np.random.default_rng(47)
+    seg = _ragged_segments(rng, T, S)
+    ids = rng.integers(0, NA, S).tolist()
+    x, A, B = make_case(oracle, 204, T, seg, ids, NA, h_in, h_out, r, dt, dy=True)
+    base = dyadic(rng, (T, h_out), 16, 8)
+    _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
+
+
 def test_multi_projection_mixed_routes_equal_single_calls(K, oracle, gpu_device):
     """Projections of one launch with different k: all long (sixteen-wave route with a different
     k split each) and one short (which sends the whole launch down the four-wave route)."""
