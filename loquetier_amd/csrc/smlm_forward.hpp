@@ -349,7 +349,11 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int kk = kb + 32 * u + 8 * g;
-        xf[u] = ldg16_or(xrow + kk, row >= 0 && kk < kend, zeros);
+        xf[u] = ldg16_or(xrow + kk, row >= 0 && kk < kend
+#ifdef SMLM_TUNING
+                                        && !(a.dbg & 2)
+#endif
+                         , zeros);
       }
     };
     auto load_w = [&](int kb, u32x4 (&st)[kPer]) {
@@ -363,7 +367,11 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
         } else {
           const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
           st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
-                           idx < kPieces && n0 + nl < P.d_out && kb + k8 < kend, zeros);
+                           idx < kPieces && n0 + nl < P.d_out && kb + k8 < kend
+#ifdef SMLM_TUNING
+                               && !(a.dbg & 1)
+#endif
+                           , zeros);
         }
       }
     };
@@ -426,6 +434,9 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
       for (int nb = 0; nb < NB; ++nb) {
         const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
         if (n >= P.d_out) continue;
+#ifdef SMLM_TUNING
+        if ((a.dbg & 4) && acc[nb][0] != 12345.f) continue;
+#endif
         if (as_partial)
           *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + row) * P.d_out + n) = acc[nb];
         else
