@@ -199,6 +199,12 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
 }
 
 int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
+  const int row_tiles = ceil_div(a.T, kTileRows);
+  if (!a.seg_scale && row_tiles <= kMaxGridY * 64) {  // no scale to look up: fold row by row
+    const dim3 grid((unsigned)row_tiles, (unsigned)a.nproj);
+    if (dtype == SMLM_DTYPE_F16) return launch(reduce_rows_kernel<SMLM_DTYPE_F16>, grid, dim3(256), st, a);
+    return launch(reduce_rows_kernel<SMLM_DTYPE_BF16>, grid, dim3(256), st, a);
+  }
   const int units = tile_units_max(a.T, S, groups, 1);
   const long items = (long)units * a.nproj;
   a.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;

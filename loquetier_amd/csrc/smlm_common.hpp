@@ -144,6 +144,7 @@ __device__ __forceinline__ u32x4 ldg_strided8(const uint16_t* p, long stride) {
 // Views into a plan buffer (all int32).  Sizes are functions of (T, S) only.
 struct PlanView {
   int32_t* hdr;         // [16]: 0 n_tiles, 1 n_groups, 2 rows covered, 3 key kind used, 4 n_blocks,
+                        //       5 first covered row (the covered rows are [hdr[5], hdr[5] + hdr[2])),
                         //       12..15 zero (16 zero bytes for predicated-off loads to read)
   int32_t* sorted_seg;  // [S]   segment at sorted position p
   int32_t* rowpos;      // [S+1] first gathered-row index of sorted position p

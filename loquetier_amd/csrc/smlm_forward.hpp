@@ -495,6 +495,31 @@ __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
   }
 }
 
+// The same fold without a scale, walking the rows in order instead of through the plan's
+// tiles: grid (ceil(T / 16), projections), a workgroup folds 16 consecutive rows.  Nothing is
+// looked up before the partials are requested; the rows that belong to a segment are the
+// range [hdr[5], hdr[5] + hdr[2]) (segments lie end to end) and only those are stored.
+template <int DT>
+__global__ __launch_bounds__(256) void reduce_rows_kernel(ReduceArgs a) {
+  const ReduceProj P = a.p[blockIdx.y];
+  if (P.ksplit <= 1) return;
+  const int c = threadIdx.x >> 4, q = threadIdx.x & 15;
+  const int row = (int)blockIdx.x * kTileRows + c;
+  const int first = uload(a.plan.hdr, 5), count = uload(a.plan.hdr, 2);
+  const bool in_batch = row < a.T;
+  const float* zf = reinterpret_cast<const float*>(a.plan.hdr + kHdrZeros);
+  for (int n = 4 * q; n < a.d_out; n += 64) {
+    f32x4 part[kMaxKsplit];
+#pragma unroll
+    for (int z = 0; z < kMaxKsplit; ++z)
+      part[z] = ldg_f4((in_batch && z < P.ksplit) ? P.partial + ((long)z * a.T + row) * a.d_out + n : zf);
+    f32x4 sum = part[0];
+#pragma unroll
+    for (int z = 1; z < kMaxKsplit; ++z) sum += part[z];
+    if (row >= first && row < first + count) store4<DT>(P.out + (long)row * a.d_out + n, sum, 1.0f, a.beta);
+  }
+}
+
 // ------------------------------------------------------------------ expand --
 struct ExpandProj {
   uint16_t* y;                // [T, d_out]

@@ -285,6 +285,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     pv.hdr[2] = rows_total;
     pv.hdr[3] = kind;
     pv.hdr[4] = n_blocks;
+    pv.hdr[5] = start0[0];  // segments lie end to end: the covered rows start at s[0]
 #pragma unroll
     for (int i = 0; i < 4; ++i) pv.hdr[kHdrZeros + i] = 0;
   }
@@ -398,6 +399,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
     pv.hdr[1] = NG;
     pv.hdr[2] = rows_total;
     pv.hdr[3] = kind;
+    pv.hdr[5] = s[0];  // segments lie end to end: the covered rows start at s[0]
 #pragma unroll
     for (int i = 0; i < 4; ++i) pv.hdr[kHdrZeros + i] = 0;
   }

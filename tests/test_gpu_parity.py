@@ -85,6 +85,7 @@ FWD_CASES = [
     ("one-segment", 16, [0, 16], [0], 1, 128, 128, 16),
     ("ragged", 77, [0, 1, 18, 18, 50, 51, 52, 77], [3, 1, 2, 1, 0, 3, 1], 4, 256, 320, 32),
     ("uncovered-rows", 40, [3, 10, 31], [1, 0], 2, 64, 64, 16),
+    ("uncovered-rows-long-k", 75, [5, 22, 22, 60], [1, 0, 1], 2, 4096, 64, 16),  # k split and folded
     ("rank64", 45, [0, 20, 45], [0, 1], 2, 512, 256, 64),
     ("rank24", 33, [0, 33], [0], 1, 96, 136, 24),
     ("decode", 64, list(range(65)), [i % 5 for i in range(64)], 5, 512, 512, 16),
