@@ -214,6 +214,23 @@ SMLM_API int smlm_rms_norm_bwd(void* dx, void* dw, const void* g, const void* x,
                                const float* rms, void* workspace, size_t workspace_bytes, int rows,
                                int cols, int dtype, void* stream);
 
+/*
+ * Run-length segments of a flat batch, built on the device.  Replaces the host
+ * loop of ModelGeneration.generate (src/loquetier_src/model_generation.py:267-283):
+ * consecutive requests with the same adapter id merge into one segment; its
+ * length is the sum of their token counts, seg_indptr the running sum from 0.
+ *   req_adapter, req_len : int32 [R] on the device (negative lengths count as 0)
+ *   seg_adapter, seg_len : int32 [R];  seg_indptr : int32 [R + 1];  n_seg : int32 [2]
+ * The segment count stays on the device (n_seg[0]; n_seg[1] = total rows), so the
+ * outputs have capacity R: entries past the last segment are empty segments
+ * (indptr = total rows, length 0, the last request's adapter id).  Pass them on
+ * with S = R; empty segments cost nothing in the plan.  R == 0 writes
+ * seg_indptr[0] = 0 and n_seg = {0, 0}.
+ */
+SMLM_API int smlm_segments_build(const int32_t* req_adapter, const int32_t* req_len, int R,
+                                 int32_t* seg_adapter, int32_t* seg_len, int32_t* seg_indptr,
+                                 int32_t* n_seg, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

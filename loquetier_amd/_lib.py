@@ -45,6 +45,7 @@ SIGNATURES = {
     "smlm_rms_norm_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "smlm_rms_norm_bwd_workspace_size": (_i, [_i, _i, _psz]),
     "smlm_rms_norm_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),
+    "smlm_segments_build": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -6,6 +6,7 @@
 #include <cstdlib>
 
 #include "rms_norm.hpp"
+#include "segments.hpp"
 #include "smlm.h"
 #include "smlm_backward.hpp"
 #include "smlm_common.hpp"
@@ -839,6 +840,16 @@ SMLM_API int smlm_rms_norm_bwd(void* dx, void* dw, const void* g, const void* x,
   const dim3 fgrid((unsigned)ceil_div(cols, 64));
   return f16 ? launch(rms_fold_kernel<SMLM_DTYPE_F16>, fgrid, dim3(256), st, fa)
              : launch(rms_fold_kernel<SMLM_DTYPE_BF16>, fgrid, dim3(256), st, fa);
+}
+
+SMLM_API int smlm_segments_build(const int32_t* req_adapter, const int32_t* req_len, int R,
+                                 int32_t* seg_adapter, int32_t* seg_len, int32_t* seg_indptr,
+                                 int32_t* n_seg, void* stream) {
+  if (R < 0 || !seg_indptr || !n_seg) return SMLM_ERR_ARG;
+  if (R > 0 && (!req_adapter || !req_len || !seg_adapter || !seg_len)) return SMLM_ERR_ARG;
+  if (R > kMaxSegments) return SMLM_ERR_LIMIT;
+  const SegmentsArgs a{req_adapter, req_len, seg_adapter, seg_len, seg_indptr, n_seg, R};
+  return launch(segments_kernel, dim3(1), dim3(kPlanThreads), (hipStream_t)stream, a);
 }
 
 }  // extern "C"

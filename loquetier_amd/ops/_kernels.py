@@ -346,3 +346,32 @@ def rms_norm_backward(dx: torch.Tensor, dw: torch.Tensor, grad_output: torch.Ten
                                            x.data_ptr(), w.data_ptr(), rms.data_ptr(), ws.data_ptr(),
                                            ws.numel(), rows, cols, code, _stream(dev))
     _lib.check(rc, "rms_norm_backward")
+
+
+def segments_build(req_adapter: torch.Tensor, req_len: torch.Tensor):
+    """Run-length segments from per-request (adapter id, token count), on the device.
+
+    The device version of the loop in ModelGeneration.generate
+    (src/loquetier_src/model_generation.py:267-283).  Both inputs are int32 [R]
+    device tensors.  Returns (seg_adapter [R], seg_len [R], seg_indptr [R+1],
+    n_seg [2]) as int32 device tensors; n_seg holds (segment count, total rows)
+    and is not read back here, so nothing waits for the device.  Entries past
+    n_seg[0] are empty segments; pass the arrays on whole (S = R)."""
+    for t, n in ((req_adapter, "req_adapter"), (req_len, "req_len")):
+        _check_input(t, n)
+        _check_dim(1, t, n)
+        if t.dtype != torch.int32:
+            raise RuntimeError(f"{n} must be int32")
+    if req_adapter.numel() != req_len.numel():
+        raise RuntimeError("req_adapter and req_len must have one entry per request")
+    dev, R = req_adapter.device, req_adapter.numel()
+    seg_adapter = torch.empty(R, dtype=torch.int32, device=dev)
+    seg_len = torch.empty(R, dtype=torch.int32, device=dev)
+    seg_indptr = torch.empty(R + 1, dtype=torch.int32, device=dev)
+    n_seg = torch.empty(2, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().smlm_segments_build(_ptr(req_adapter), _ptr(req_len), R, _ptr(seg_adapter),
+                                             _ptr(seg_len), seg_indptr.data_ptr(), n_seg.data_ptr(),
+                                             _stream(dev))
+    _lib.check(rc, "segments_build")
+    return seg_adapter, seg_len, seg_indptr, n_seg

@@ -29,3 +29,14 @@ def build_segments(req_lora_id: Sequence[int], req_len: Sequence[int], device
     segment = torch.cumsum(torch.tensor([0] + lora_lens, dtype=torch.int32, device=device), dim=0,
                            dtype=torch.int32)
     return lora_ids, lora_len, segment
+
+
+def build_segments_device(req_lora_id: torch.Tensor, req_len: torch.Tensor
+                          ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The same merge for request arrays that already live on the GPU (int32
+    [R] each): returns (lora_ids [R], lora_len [R], segment [R+1], n_seg [2])
+    as device tensors without waiting for the GPU.  n_seg = (segment count,
+    total rows); the arrays keep the capacity R and describe empty segments
+    past the count, so they are handed on whole."""
+    from .ops import _kernels
+    return _kernels.segments_build(req_lora_id, req_len)

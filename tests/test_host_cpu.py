@@ -158,3 +158,14 @@ def test_prepare_weight_mirror(oracle):
             assert np.array_equal(got, oracle.prepare_weight(w.T.copy(), 1, 16, scaling, dt))
         same = prepare_weight(torch.from_numpy(w), 8, tdt, "cpu", 0, None)
         assert same.shape == (8, 32)
+
+
+def test_segments_build_argument_validation_codes(lib):
+    L = lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256  # fake "device" address; never dereferenced
+    assert L.smlm_segments_build(p, p, -1, p, p, p, p, None) == -1
+    assert L.smlm_segments_build(None, p, 4, p, p, p, p, None) == -1
+    assert L.smlm_segments_build(p, p, 4, p, p, None, p, None) == -1
+    assert L.smlm_segments_build(p, p, 4, p, p, p, None, None) == -1
+    assert L.smlm_segments_build(p, p, (1 << 20) + 1, p, p, p, p, None) == -6   # beyond the plan's segment limit
