@@ -190,6 +190,39 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
                            int r, int dtype, const float* part_scale, void* stream);
 
 /*
+ * Dropout of the training rows of x inside the LoRA operator.  Replaces the
+ * per-partition nn.Dropout calls and the torch.cat in MixedLoraLinear.forward
+ * (src/loquetier_src/models/mixed_lora.py:185-192) and autograd's mask multiply
+ * on the way back: no dropped copy of x and no mask are stored, the mask is
+ * regenerated from (seed, offset, row, column) wherever x or dX pass through
+ * registers.  Element (t, j) of a row t < rows whose segment has p > 0 is dropped
+ * when 16-bit piece j % 8 of
+ *   philox4x32_10(counter = (t, j / 8, offset_lo, offset_hi), key = (seed_lo, seed_hi))
+ * is below floor(p * 65536); kept elements become round(x * (1 / (1 - p))).
+ *   seg_p  : device float [S], the dropout probability of each segment's adapter
+ *            (indexed like seg_scale: by the plan's segments); NULL = no dropout
+ *   rows   : training rows are [0, rows) of the batch; later rows are never dropped
+ *   seed, offset : the stream; the same pair must be passed to the forward and to
+ *            the backward of one layer.  Projection i of a multi-projection call
+ *            uses offset + i.
+ */
+typedef struct smlm_dropout {
+  const float* seg_p;
+  int rows;
+  uint64_t seed;
+  uint64_t offset;
+} smlm_dropout;
+
+/* smlm_lora_fwd_multi with dropout of x (NULL descriptor: identical to it). */
+SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void* const* x,
+                                         void* const* v_out, const void* const* const* a_ptrs,
+                                         const void* const* const* b_ptrs, int n_weights,
+                                         const int* h_in, const int* h_out, const void* plan,
+                                         void* workspace, size_t workspace_bytes, int T, int S, int r,
+                                         int dtype, float beta, const float* seg_scale, int stages,
+                                         const smlm_dropout* dropout, void* stream);
+
+/*
  * RMSNorm forward.  Replaces dispatch_rms_norm / rms_norm<T>
  * (kernel_src/csrc/loquetier_ops.cc:326-358,
  * kernel_src/csrc/rms_norm/rms_norm_cutlass.cu:81-186):

@@ -22,6 +22,13 @@ _psz = C.POINTER(C.c_size_t)
 _pi = C.POINTER(C.c_int)
 _pvp = C.POINTER(C.c_void_p)
 
+class Dropout(C.Structure):
+    """struct smlm_dropout of include/smlm.h."""
+    _fields_ = [("seg_p", C.c_void_p), ("rows", C.c_int), ("seed", C.c_uint64), ("offset", C.c_uint64)]
+
+
+_pdrop = C.POINTER(Dropout)
+
 # name -> (restype, argtypes); must list every symbol include/smlm.h declares
 SIGNATURES = {
     "smlm_abi_version": (_i, []),
@@ -39,6 +46,8 @@ SIGNATURES = {
     "smlm_lora_fwd_multi_workspace_size": (_i, [_i, _i, _pi, _i, _psz]),
     "smlm_lora_fwd_multi": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _i, _pi, _pi, _vp, _vp, _sz, _i, _i, _i,
                                  _i, _f, _vp, _i, _vp]),
+    "smlm_lora_fwd_multi_dropout": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _i, _pi, _pi, _vp, _vp, _sz, _i, _i,
+                                         _i, _i, _f, _vp, _i, _pdrop, _vp]),
     "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
     "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
                            _i, _vp, _vp]),

@@ -1,0 +1,89 @@
+// Dropout of the training rows of x, regenerated wherever x (or dX) passes through registers.
+//
+// The reference drops x before the LoRA term, one nn.Dropout(p) per adapter
+// (src/loquetier_src/models/mixed_lora.py:185-192): a dropped copy of every training partition
+// plus a torch.cat of the whole batch, and autograd's mask multiply on the way back.  Here no
+// dropped copy and no mask are stored: the mask is a pure function of (seed, offset, row,
+// column), so the shrink kernels apply it to the x fragments they load, the weight-gradient
+// kernel to the x fragments it loads, and the dX kernel to the values it stores.
+//
+// Mask: the eight 16-bit pieces of philox4x32_10(counter = (row, col / 8, offset), key = seed)
+// decide elements col .. col + 7 of a row; an element is dropped when its piece is below
+// floor(p * 65536).  Kept elements become round(x * (1 / (1 - p))) (float product, as torch's
+// dropout computes it), dropped ones +0.  Rows at or past `rows` (inference rows) and segments
+// with p <= 0 pass through untouched.
+#pragma once
+#include "smlm_common.hpp"
+
+namespace smlm {
+
+struct DropArgs {
+  const float* seg_p;  // [S] dropout probability of each segment's adapter; nullptr: no dropout
+  int rows;            // training rows are [0, rows)
+  uint32_t k0, k1;     // seed
+  uint32_t o0, o1;     // offset (distinguishes layers / steps)
+};
+
+// the arguments of projection pj of a launch over several projections: offset + pj
+__device__ __forceinline__ DropArgs drop_proj(DropArgs d, int pj) {
+  const uint64_t off = (((uint64_t)d.o1 << 32) | d.o0) + (uint32_t)pj;
+  d.o0 = (uint32_t)off;
+  d.o1 = (uint32_t)(off >> 32);
+  return d;
+}
+
+struct DropRow {
+  uint32_t thresh;  // pieces below it are dropped
+  float scale;      // factor of kept elements
+  bool on;
+};
+
+// the row's dropout parameters; seg is only read for training rows
+__device__ __forceinline__ DropRow drop_row(const DropArgs& d, int row, const int32_t* seg_of_slot, int slot) {
+  DropRow r{0u, 1.0f, false};
+  if (row >= 0 && row < d.rows) {
+    const float p = d.seg_p[seg_of_slot[slot]];
+    if (p > 0.0f) {
+      r.on = true;
+      r.thresh = p >= 1.0f ? 65536u : (uint32_t)(p * 65536.0f);
+      r.scale = p >= 1.0f ? 0.0f : 1.0f / (1.0f - p);
+    }
+  }
+  return r;
+}
+
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                              uint32_t k1, uint32_t (&out)[4]) {
+#pragma unroll
+  for (int i = 0; i < 10; ++i) {
+    if (i) {
+      k0 += 0x9E3779B9u;
+      k1 += 0xBB67AE85u;
+    }
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+  }
+  out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
+}
+
+// eight consecutive elements of one row (columns 8*colblk .. +7), packed two to a word
+template <int DT>
+__device__ __forceinline__ u32x4 drop8(u32x4 v, const DropArgs& d, const DropRow& r, int row, int colblk) {
+  if (__builtin_amdgcn_ballot_w64(r.on) == 0) return v;  // uniform over the wave
+  uint32_t w[4];
+  philox4x32_10((uint32_t)row, (uint32_t)colblk, d.o0, d.o1, d.k0, d.k1, w);
+  u32x4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t scaled = pack2<DT>(Num<DT>::lo(v[e]) * r.scale, Num<DT>::hi(v[e]) * r.scale);
+    const uint32_t keep = ((w[e] & 0xffffu) >= r.thresh ? 0x0000ffffu : 0u) | ((w[e] >> 16) >= r.thresh ? 0xffff0000u : 0u);
+    o[e] = r.on ? (scaled & keep) : v[e];
+  }
+  return o;
+}
+
+}  // namespace smlm

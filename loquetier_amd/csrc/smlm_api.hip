@@ -151,20 +151,20 @@ inline dim3 item_grid(const ItemSpace& sp, long items) {
   return dim3((unsigned)rows, (unsigned)sp.units_max, (unsigned)sp.nproj);
 }
 
-template <int DT, int NW, bool RM, bool DIRECT>
+template <int DT, int NW, bool RM, bool DIRECT, bool DROP = false>
 int launch_shrink_nb(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   const dim3 block(NW * kWaveSize);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, NW, RM, DIRECT>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, NW, RM, DIRECT>, grid, block, st, a);
-  return launch(shrink_kernel<DT, 4, 2, NW, RM, DIRECT>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_kernel<DT, 1, 4, NW, RM, DIRECT, DROP>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_kernel<DT, 2, 4, NW, RM, DIRECT, DROP>, grid, block, st, a);
+  return launch(shrink_kernel<DT, 4, 2, NW, RM, DIRECT, DROP>, grid, block, st, a);
 }
 
-template <int DT, bool DIRECT, bool WKN>
+template <int DT, bool DIRECT, bool WKN, bool DROP = false>
 int launch_shrink_block(int NB, dim3 grid, hipStream_t st, const ShrinkArgs& a) {
   const dim3 block(kFwdThreads);
-  if (NB == 1) return launch(shrink_block_kernel<DT, 1, 4, DIRECT, WKN>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_block_kernel<DT, 2, 4, DIRECT, WKN>, grid, block, st, a);
-  return launch(shrink_block_kernel<DT, 4, 4, DIRECT, WKN>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_block_kernel<DT, 1, 4, DIRECT, WKN, DROP>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_kernel<DT, 2, 4, DIRECT, WKN, DROP>, grid, block, st, a);
+  return launch(shrink_block_kernel<DT, 4, 4, DIRECT, WKN, DROP>, grid, block, st, a);
 }
 
 template <int DT, bool DIRECT>
@@ -172,6 +172,12 @@ int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStrea
                      const ShrinkArgs& a) {
   if (row_major)  // the slow layout
     return launch_shrink_nb<DT, kFwdWaves, true, DIRECT>(NB, grid, st, a);
+  if (a.drop.seg_p) {  // dropout of the training rows: x in the usual layout, weights [n][k]
+    if (MT == 1)
+      return NW == 16 ? launch_shrink_nb<DT, 16, false, DIRECT, true>(NB, grid, st, a)
+                      : launch_shrink_nb<DT, kFwdWaves, false, DIRECT, true>(NB, grid, st, a);
+    return launch_shrink_block<DT, DIRECT, false, true>(NB, grid, st, a);
+  }
   if (MT == 1)
     return NW == 16 ? launch_shrink_nb<DT, 16, false, DIRECT>(NB, grid, st, a)
                     : launch_shrink_nb<DT, kFwdWaves, false, DIRECT>(NB, grid, st, a);
@@ -305,8 +311,11 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
-               const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false) {
+               const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false,
+               const DropArgs* drop = nullptr) {
+  if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
   ShrinkArgs a{};
+  if (drop) a.drop = *drop;
   a.w_kn = w_kn ? 1 : 0;
   a.plan = tile_args(pv);
   a.seg_scale = seg_scale;
@@ -539,14 +548,40 @@ SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_
   return SMLM_OK;
 }
 
+// the library's view of the caller's dropout descriptor; nullptr or seg_p == nullptr: none
+static int drop_args(const smlm_dropout* d, DropArgs* out) {
+  *out = DropArgs{};
+  if (!d || !d->seg_p) return SMLM_OK;
+  if (d->rows < 0) return SMLM_ERR_ARG;
+  out->seg_p = d->seg_p;
+  out->rows = d->rows;
+  out->k0 = (uint32_t)d->seed; out->k1 = (uint32_t)(d->seed >> 32);
+  out->o0 = (uint32_t)d->offset; out->o1 = (uint32_t)(d->offset >> 32);
+  return SMLM_OK;
+}
+
 SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* x,
                                  void* const* v_out, const void* const* const* a_ptrs,
                                  const void* const* const* b_ptrs, int n_weights, const int* h_in,
                                  const int* h_out, const void* plan, void* workspace,
                                  size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
                                  const float* seg_scale, int stages, void* stream) {
+  return smlm_lora_fwd_multi_dropout(n_proj, y, x, v_out, a_ptrs, b_ptrs, n_weights, h_in, h_out, plan,
+                                     workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale, stages,
+                                     nullptr, stream);
+}
+
+SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void* const* x,
+                                         void* const* v_out, const void* const* const* a_ptrs,
+                                         const void* const* const* b_ptrs, int n_weights,
+                                         const int* h_in, const int* h_out, const void* plan,
+                                         void* workspace, size_t workspace_bytes, int T, int S, int r,
+                                         int dtype, float beta, const float* seg_scale, int stages,
+                                         const smlm_dropout* dropout, void* stream) {
   int rc = check_common(T, S, dtype);
   if (rc) return rc;
+  DropArgs drop;
+  if ((rc = drop_args(dropout, &drop))) return rc;
   if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
     return SMLM_ERR_ARG;
   if (stages < 1 || stages > (SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND)) return SMLM_ERR_ARG;
@@ -595,7 +630,7 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
   }
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                    0.0f, nullptr, st, !expand_folds);
+                    0.0f, nullptr, st, !expand_folds, false, &drop);
     if (rc) return rc;
   }
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;

@@ -21,6 +21,7 @@
 // contiguous range of items per XCD, or plain round robin) remains as the
 // fallback for batches beyond the direct grid's limits.
 #pragma once
+#include "dropout.hpp"
 #include "smlm_common.hpp"
 
 namespace smlm {
@@ -180,6 +181,7 @@ struct ShrinkArgs {
   int T;
   ItemSpace items;            // chunk rows of projection p: ksplit*zblocks
   int w_kn;                   // tile-block kernel only: weights are stored [k][n]
+  DropArgs drop;              // DROP kernels: dropout of the training rows of x
 #ifdef SMLM_TUNING
   int dbg;                    // experiments: 1 = no weight loads, 2 = no x loads, 4 = no partial/output store
 #endif
@@ -190,7 +192,7 @@ struct ShrinkArgs {
 // ranges; their accumulators are summed through LDS in wave order and written
 // either as an fp32 partial (k split over workgroups, or a consumer that folds)
 // or as the final 16-bit value.  NW = 16 is for decode batches: few tiles, long k.
-template <int DT, int NB, int U, int NW, bool ROWMAJOR, bool DIRECT>
+template <int DT, int NB, int U, int NW, bool ROWMAJOR, bool DIRECT, bool DROP = false>
 __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
   __shared__ f32x4 red[NW][NB][kWaveSize];
   const int units = DIRECT ? 0 : tile_units<1>(a.plan, 0);
@@ -209,6 +211,9 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+    DropRow dr{};
+    DropArgs dp{};
+    if (DROP) dp = drop_proj(a.drop, pj), dr = drop_row(dp, row, a.plan.tile_rseg, slot);
 
     const int kbeg = (kz * NW + wave) * P.k_per_wave;
     const int kend = min(kbeg + P.k_per_wave, P.d_in);
@@ -239,11 +244,13 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         }
       }
     };
-    auto multiply = [&](const u32x4 (&xf)[U], const u32x4 (&wf)[NB][U]) {
+    auto multiply = [&](int k, const u32x4 (&xf)[U], const u32x4 (&wf)[NB][U]) {
 #pragma unroll
-      for (int u = 0; u < U; ++u)
+      for (int u = 0; u < U; ++u) {
+        const u32x4 xu = DROP ? drop8<DT>(xf[u], dp, dr, row, (k + 32 * u + 8 * g) >> 3) : xf[u];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(wf[nb][u], xf[u], acc[nb]);
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(wf[nb][u], xu, acc[nb]);
+      }
     };
     if (NW < 16) {
       // two load batches in turn: one is on its way while the other is multiplied
@@ -253,17 +260,17 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
       for (int k = kbeg; k < kend; k += 64 * U) {
         const bool more = k + 32 * U < kend;  // uniform over the wave
         if (more) load_batch(k + 32 * U, xb, wb);
-        multiply(xa, wa);
+        multiply(k, xa, wa);
         if (!more) break;
         if (k + 64 * U < kend) load_batch(k + 64 * U, xa, wa);
-        multiply(xb, wb);
+        multiply(k + 32 * U, xb, wb);
       }
     } else {  // sixteen waves share the VGPR file: one batch at a time (k is usually one batch)
 #pragma unroll 1
       for (int k = kbeg; k < kend; k += 32 * U) {
         u32x4 xf[U], wf[NB][U];
         load_batch(k, xf, wf);
-        multiply(xf, wf);
+        multiply(k, xf, wf);
       }
     }
 
@@ -314,7 +321,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 // [h_out, r] is for the backward's dV = dY B) instead of [n][k]: a batch is then staged as
 // it lies in memory and the MFMA operand, which wants eight consecutive k of one column,
 // is read out of LDS with the transposing read.
-template <int DT, int NB, int U, bool DIRECT, bool WKN>
+template <int DT, int NB, int U, bool DIRECT, bool WKN, bool DROP = false>
 __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a) {
   constexpr int KB = 32 * U;                 // k per batch
   constexpr int kRowsW = 16 * NB;            // weight rows (output columns) per workgroup
@@ -344,6 +351,9 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
     const int kbeg = kz * kFwdWaves * P.k_per_wave;
     const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
     const uint16_t* xrow = P.x + (long)(row < 0 ? 0 : row) * P.d_in;
+    DropRow dr{};
+    DropArgs dp{};
+    if (DROP) dp = drop_proj(a.drop, pj), dr = drop_row(dp, row, a.plan.tile_rseg, slot);
 
     auto load_x = [&](int kb, u32x4 (&xf)[U]) {
 #pragma unroll
@@ -414,11 +424,11 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
       __syncthreads();  // buffer `buf` is written; buffer `buf ^ 1` is no longer read
       if (active) {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+        for (int u = 0; u < U; ++u) {
+          const u32x4 xu = DROP ? drop8<DT>(xf[u], dp, dr, row, (kb + 32 * u + 8 * g) >> 3) : xf[u];
 #pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            acc[nb] = Num<DT>::mfma(weight_frag(buf, u, nb), xf[u], acc[nb]);
-          }
+          for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(weight_frag(buf, u, nb), xu, acc[nb]);
+        }
       }
       stage_w(buf ^ 1, wn);
       buf ^= 1;

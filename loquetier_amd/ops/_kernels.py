@@ -198,23 +198,51 @@ def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, pl
     _lib.check(rc, "smlm_gemm_planned")
 
 
+class DropoutSpec:
+    """Dropout of the training rows of x inside the operator (struct smlm_dropout):
+    seg_p float32 [S] on the device, the dropout probability of each segment's
+    adapter; rows = number of training rows (they come first in the batch);
+    (seed, offset) name the mask stream -- the backward of a layer must be given
+    the pair its forward used.  Replaces the nn.Dropout calls and the torch.cat of
+    MixedLoraLinear.forward (src/loquetier_src/models/mixed_lora.py:185-192)."""
+
+    def __init__(self, seg_p: torch.Tensor, rows: int, seed: int, offset: int):
+        _check_input(seg_p, "seg_p")
+        if seg_p.dtype != torch.float32 or seg_p.dim() != 1:
+            raise RuntimeError("seg_p must be a 1D float32 tensor")
+        if rows < 0:
+            raise RuntimeError("rows must not be negative")
+        self.seg_p, self.rows = seg_p, int(rows)
+        self.seed, self.offset = int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1)
+
+    def with_offset(self, offset: int) -> "DropoutSpec":
+        return DropoutSpec(self.seg_p, self.rows, self.seed, offset)
+
+    def struct(self, plan: "SegmentPlan"):
+        if self.seg_p.size(0) != plan.S or self.seg_p.device != plan.segment.device:
+            raise RuntimeError("seg_p must have one entry per segment of the plan, on its device")
+        return _lib.Dropout(self.seg_p.data_ptr(), self.rows, self.seed, self.offset)
+
+
 def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_ptrs: torch.Tensor,
                       plan: SegmentPlan, rank: int, seg_scale: Optional[torch.Tensor] = None,
-                      beta: float = 0.0, v_out: Optional[torch.Tensor] = None) -> None:
+                      beta: float = 0.0, v_out: Optional[torch.Tensor] = None,
+                      dropout: Optional[DropoutSpec] = None) -> None:
     """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call (two launches).
     a_ptrs / b_ptrs are indexed by adapter id when the plan was built from int32
     adapter ids, by segment otherwise."""
     smlm_lora_forward_multi([y], [x], [a_ptrs], [b_ptrs], plan, rank, seg_scale=seg_scale, beta=beta,
-                            v_out=None if v_out is None else [v_out])
+                            v_out=None if v_out is None else [v_out], dropout=dropout)
 
 
 def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
-                            v_out=None, stages: int = 3) -> None:
+                            v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
     in two launches.  Lists of equal length; entries of xs may be the same tensor.
     stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
-    arguments on the same stream), 3 = both."""
+    arguments on the same stream), 3 = both.  dropout: the training rows of x are
+    dropped inside the shrink kernel; projection i uses the stream offset + i."""
     n = len(ys)
     if not (1 <= n <= 8) or len(xs) != n or len(a_ptrs) != n or len(b_ptrs) != n or \
             (v_out is not None and len(v_out) != n):
@@ -245,12 +273,13 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
         _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(n, plan.T, h_in, rank, C.byref(need)),
                    "smlm_lora_fwd_multi_workspace_size")
         ws = _workspace(dev, need.value)
-        rc = _lib.load().smlm_lora_fwd_multi(
+        drop = None if dropout is None else C.byref(dropout.struct(plan))
+        rc = _lib.load().smlm_lora_fwd_multi_dropout(
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
             min(t.size(0) for t in list(a_ptrs) + list(b_ptrs)), h_in, h_out,
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
-            _ptr(seg_scale), int(stages), _stream(dev))
+            _ptr(seg_scale), int(stages), drop, _stream(dev))
     _lib.check(rc, "smlm_lora_forward")
 
 

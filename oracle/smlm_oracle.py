@@ -22,7 +22,7 @@ DTYPES = {"fp32": 0, "fp16": 1, "bf16": 2}
 
 def build(force: bool = False) -> str:
     """Compile the C oracle with gcc (no GPU toolchain involved)."""
-    newest = max(os.path.getmtime(os.path.join(_HERE, f)) for f in ("smlm_oracle.c", "rms_norm_oracle.c"))
+    newest = max(os.path.getmtime(os.path.join(_HERE, f)) for f in ("smlm_oracle.c", "rms_norm_oracle.c", "dropout_oracle.c"))
     if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < newest:
         subprocess.run(["make", "-C", _HERE, "-B" if force else "-s", "all"], check=True,
                        stdout=subprocess.DEVNULL)
@@ -41,9 +41,11 @@ def lib() -> C.CDLL:
         for name in ("oracle_smlm_gemm", "oracle_add_lora_forward", "oracle_mixed_lora_linear",
                      "oracle_lora_fused", "oracle_add_lora_backward_rowmajor",
                      "oracle_add_lora_backward", "oracle_build_segments", "oracle_batch_len_info",
-                     "oracle_prepare_weight", "oracle_rms_norm_fwd", "oracle_rms_norm_bwd"):
+                     "oracle_prepare_weight", "oracle_rms_norm_fwd", "oracle_rms_norm_bwd",
+                     "oracle_dropout_mask", "oracle_dropout_rows"):
             getattr(_lib, name).restype = C.c_int
         _lib.oracle_round.restype = None
+        _lib.oracle_philox4x32_10.restype = None
     return _lib
 
 
@@ -257,3 +259,34 @@ def rms_norm_bwd(g, x, w, rms, dtype: str, literal: bool = False) -> Tuple[np.nd
     _check(lib().oracle_rms_norm_bwd(_fp(dx), _fp(dw), _fp(g), _fp(x), _fp(w), _fp(rms), rows, cols,
                                      DTYPES[dtype], int(literal)), "oracle_rms_norm_bwd")
     return dx, dw
+
+
+def philox4x32_10(ctr: Sequence[int], key: Sequence[int]) -> List[int]:
+    c = (C.c_uint32 * 4)(*ctr)
+    k = (C.c_uint32 * 2)(*key)
+    o = (C.c_uint32 * 4)()
+    lib().oracle_philox4x32_10(c, k, o)
+    return list(o)
+
+
+def dropout_mask(rows: int, cols: int, row_p, seed: int, offset: int, row0: int = 0) -> np.ndarray:
+    """keep[t, j] of the counter-based dropout mask (1 = kept)."""
+    rp = _f32(row_p)
+    assert rp.shape == (rows,)
+    keep = np.zeros((rows, cols), np.uint8)
+    _check(lib().oracle_dropout_mask(keep.ctypes.data_as(C.c_void_p), rows, cols, row0, _fp(rp),
+                                     C.c_uint64(seed), C.c_uint64(offset)), "oracle_dropout_mask")
+    return keep
+
+
+def dropout_rows(x, row_p, seed: int, offset: int, dtype: str, row0: int = 0) -> np.ndarray:
+    """nn.Dropout on the rows of x (row t with probability row_p[t]), mask from the
+    counter-based generator; see dropout_oracle.c."""
+    x = _f32(x)
+    rp = _f32(row_p)
+    assert rp.shape == (x.shape[0],)
+    out = np.empty_like(x)
+    _check(lib().oracle_dropout_rows(_fp(out), _fp(x), x.shape[0], x.shape[1], row0, _fp(rp),
+                                     C.c_uint64(seed), C.c_uint64(offset), DTYPES[dtype]),
+           "oracle_dropout_rows")
+    return out
