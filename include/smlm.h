@@ -223,6 +223,24 @@ SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void*
                                          const smlm_dropout* dropout, void* stream);
 
 /*
+ * smlm_lora_bwd for a forward that ran with dropout (NULL descriptor: identical
+ * to smlm_lora_bwd).  seg_p is indexed by the backward plan's partitions and the
+ * partitions of one adapter must carry the same probability; (seed, offset) are
+ * the pair the forward of this projection used (offset + i for projection i of a
+ * multi-projection call); rows >= n_rows.  x is the caller's x before dropout: v
+ * (when not passed) and dA are taken against the regenerated dropped x, and dx is
+ * the gradient with respect to x before its dropout (the mask and factor applied
+ * once more, as autograd's dropout backward does after add_lora.backward).
+ */
+SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* db_ptrs,
+                                   const void* dy, const void* x, const void* v,
+                                   const void* const* a_ptrs, const void* const* b_ptrs,
+                                   const void* plan, void* workspace, size_t workspace_bytes,
+                                   int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
+                                   const float* part_scale, const smlm_dropout* dropout,
+                                   void* stream);
+
+/*
  * RMSNorm forward.  Replaces dispatch_rms_norm / rms_norm<T>
  * (kernel_src/csrc/loquetier_ops.cc:326-358,
  * kernel_src/csrc/rms_norm/rms_norm_cutlass.cu:81-186):

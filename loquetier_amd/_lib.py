@@ -51,6 +51,8 @@ SIGNATURES = {
     "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
     "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
                            _i, _vp, _vp]),
+    "smlm_lora_bwd_dropout": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i,
+                                   _i, _i, _vp, _pdrop, _vp]),
     "smlm_rms_norm_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "smlm_rms_norm_bwd_workspace_size": (_i, [_i, _i, _psz]),
     "smlm_rms_norm_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),

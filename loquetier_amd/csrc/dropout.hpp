@@ -38,18 +38,21 @@ struct DropRow {
   bool on;
 };
 
-// the row's dropout parameters; seg is only read for training rows
-__device__ __forceinline__ DropRow drop_row(const DropArgs& d, int row, const int32_t* seg_of_slot, int slot) {
+// threshold and factor of dropout probability p (p <= 0: off)
+__device__ __forceinline__ DropRow drop_params(float p) {
   DropRow r{0u, 1.0f, false};
-  if (row >= 0 && row < d.rows) {
-    const float p = d.seg_p[seg_of_slot[slot]];
-    if (p > 0.0f) {
-      r.on = true;
-      r.thresh = p >= 1.0f ? 65536u : (uint32_t)(p * 65536.0f);
-      r.scale = p >= 1.0f ? 0.0f : 1.0f / (1.0f - p);
-    }
+  if (p > 0.0f) {
+    r.on = true;
+    r.thresh = p >= 1.0f ? 65536u : (uint32_t)(p * 65536.0f);
+    r.scale = p >= 1.0f ? 0.0f : 1.0f / (1.0f - p);
   }
   return r;
+}
+
+// the row's dropout parameters; its segment is only looked up for training rows
+__device__ __forceinline__ DropRow drop_row(const DropArgs& d, int row, const int32_t* seg_of_slot, int slot) {
+  if (row >= 0 && row < d.rows) return drop_params(d.seg_p[seg_of_slot[slot]]);
+  return DropRow{0u, 1.0f, false};
 }
 
 __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,

@@ -238,6 +238,18 @@ int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipS
                      const ExpandArgs& a) {
   if (row_major)
     return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
+  if (a.drop.seg_p) {  // the backward's dX with the dropout of x undone: one projection, no fold
+    const dim3 bl(kFwdThreads);
+    if (block)  // launch_expand admits only [k][n] weights here
+      return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, true, true>, grid, bl, st, a)
+                     : launch(expand_block_kernel<DT, 4, 2, DIRECT, true, true>, grid, bl, st, a);
+    if (KS == 0) return SMLM_ERR_LIMIT;  // the backward stops at rank 64
+    if (nq == 4)
+      return KS == 1 ? launch(expand_wave_kernel<DT, 4, 1, false, DIRECT, false, true>, grid, bl, st, a)
+                     : launch(expand_wave_kernel<DT, 4, 2, false, DIRECT, false, true>, grid, bl, st, a);
+    return KS == 1 ? launch(expand_wave_kernel<DT, 2, 1, false, DIRECT, false, true>, grid, bl, st, a)
+                   : launch(expand_wave_kernel<DT, 2, 2, false, DIRECT, false, true>, grid, bl, st, a);
+  }
   if (block && a.w_kn)
     return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, true>, grid, dim3(kFwdThreads), st, a)
                    : launch(expand_block_kernel<DT, 4, 2, DIRECT, true>, grid, dim3(kFwdThreads), st, a);
@@ -254,6 +266,7 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
                   hipStream_t st, ExpandArgs& a) {
   const int KS = max_d_in <= 32 ? 1 : (max_d_in <= 64 ? 2 : 0);
   const bool block = !row_major && MT > 1 && KS > 0;  // tile blocks with the weights staged in LDS
+  if (a.drop.seg_p && (row_major || nproj != 1 || a.p[0].vsplit > 0 || (block && !a.w_kn))) return SMLM_ERR_ARG;
   if (row_major) nq = 2;
   if (block) nq = 4;
   nq = tune("SMLM_TUNE_NQ", nq);
@@ -357,6 +370,16 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
 
 template <int DT>
 int launch_wgrad(int nbj, bool split, dim3 grid, hipStream_t st, const WgradArgs& wa) {
+  if (wa.drop.seg_p) {
+    if (split) {
+      if (nbj == 1) return launch(wgrad_kernel<DT, 1, 4, true>, grid, dim3(256), st, wa);
+      if (nbj == 2) return launch(wgrad_kernel<DT, 2, 4, true>, grid, dim3(256), st, wa);
+      return launch(wgrad_kernel<DT, 4, 4, true>, grid, dim3(256), st, wa);
+    }
+    if (nbj == 1) return launch(wgrad_kernel<DT, 1, 1, true>, grid, dim3(64), st, wa);
+    if (nbj == 2) return launch(wgrad_kernel<DT, 2, 1, true>, grid, dim3(64), st, wa);
+    return launch(wgrad_kernel<DT, 4, 1, true>, grid, dim3(64), st, wa);
+  }
   if (split) {
     if (nbj == 1) return launch(wgrad_kernel<DT, 1, 4>, grid, dim3(256), st, wa);
     if (nbj == 2) return launch(wgrad_kernel<DT, 2, 4>, grid, dim3(256), st, wa);
@@ -685,8 +708,22 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
                            const void* const* b_ptrs, const void* plan, void* workspace,
                            size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out,
                            int r, int dtype, const float* part_scale, void* stream) {
+  return smlm_lora_bwd_dropout(dx, da_ptrs, db_ptrs, dy, x, v, a_ptrs, b_ptrs, plan, workspace,
+                               workspace_bytes, n_rows, P, NA, h_in, h_out, r, dtype, part_scale, nullptr,
+                               stream);
+}
+
+SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* db_ptrs,
+                                   const void* dy, const void* x, const void* v,
+                                   const void* const* a_ptrs, const void* const* b_ptrs,
+                                   const void* plan, void* workspace, size_t workspace_bytes,
+                                   int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
+                                   const float* part_scale, const smlm_dropout* dropout,
+                                   void* stream) {
   int rc = check_common(n_rows, P, dtype);
   if (rc) return rc;
+  DropArgs drop;
+  if ((rc = drop_args(dropout, &drop))) return rc;
   if (NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
   if ((h_in & 7) || (h_out & 7) || (r & 7)) return SMLM_ERR_ALIGN;
   if (r > 64) return SMLM_ERR_LIMIT;
@@ -731,7 +768,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
   if (!vv) {
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
-                         0.0f, nullptr, st)))
+                         0.0f, nullptr, st, true, false, &drop)))  // v of the dropped x, as the forward made it
       return rc;
     vv = reinterpret_cast<const uint16_t*>(v16);
   }
@@ -760,6 +797,7 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
     E.d_in = r; E.d_out = h_in; E.ldw = in_place ? h_in : r;
   }
   ea.w_kn = in_place ? 1 : 0;
+  ea.drop = drop;  // dX is the gradient with respect to x before its dropout
   if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, NA, 1, r, st,
                           ea)))
     return rc;
@@ -779,6 +817,8 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
   wa.pitch = L.pitch;
   wa.h_in = h_in; wa.h_out = h_out; wa.r = r;
   wa.chunks_a = ceil_div(h_in, kWgCols);
+  wa.grp_seg = pv.grp_seg;
+  wa.drop = drop;  // dA against the dropped x
   dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA);
   const int nbj = ceil_div(r, 16);
   // four waves splitting the rows of an adapter pay off when adapters have many rows each

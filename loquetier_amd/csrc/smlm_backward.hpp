@@ -5,6 +5,7 @@
 // (src/loquetier_src/kernel_utils.py:139-145); its C++ side has no backward
 // (kernel_src/csrc/loquetier_ops.cc:321-322).
 #pragma once
+#include "dropout.hpp"
 #include "smlm_common.hpp"
 
 namespace smlm {
@@ -81,6 +82,8 @@ struct WgradArgs {
   void* const* db_ptrs;  // [NA] -> [h_out, r]
   long pitch;
   int h_in, h_out, r, chunks_a;  // chunks_a = ceil(h_in/64): blockIdx.x below it works on dA
+  const int32_t* grp_seg;  // DROP kernels: first segment of every group (its adapter's dropout probability)
+  DropArgs drop;           // DROP kernels: dA is taken against the dropped x, regenerated while x is staged
 };
 
 constexpr int kWgCols = 64;     // columns of x / dY per workgroup
@@ -106,7 +109,11 @@ __device__ __forceinline__ int wg_lds_row(int s) {
 // token-innermost with the transposing LDS read; no workgroup barrier is needed
 // inside the loop, and the rows of the next step are already on their way from
 // memory while the current step is multiplied.
-template <int DT, int NBJ, int NW, bool IS_A>
+//
+// DROP (dA only): the forward multiplied the dropped x, so dA = dV^T dropout(x).  The mask is
+// regenerated while the rows are staged; every row of the workgroup belongs to one adapter,
+// whose probability is read once from the group's first segment.
+template <int DT, int NBJ, int NW, bool IS_A, bool DROP = false>
 __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   constexpr int kWgWaves = NW;
   constexpr int kStageElems = kWgSlots * kWgPitch;
@@ -125,7 +132,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 
   // group of this adapter (ids are distinct): every lane looks at one group
   const int NG = uload(a.hdr, 1);
-  int t_beg = 0, t_end = 0;
+  int t_beg = 0, t_end = 0, seg0 = -1;
   for (int base = 0; base < NG; base += kWaveSize) {
     const int G = base + lane;
     const bool hit = G < NG && a.grp_id[G] == ad;
@@ -134,6 +141,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       const int Gh = base + __builtin_ctzll(m);
       t_beg = uload(a.grp_tile, Gh);
       t_end = uload(a.grp_tile, Gh + 1);
+      if (DROP) seg0 = uload(a.grp_seg, Gh);
       break;
     }
   }
@@ -187,20 +195,43 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       }
   };
 
-  int32_t row_next[8];
+  DropRow dr{0u, 1.0f, false};  // uniform over the workgroup; .on is set per row below
+  bool drop_on = false;
+  if (DROP && seg0 >= 0) {
+    dr = drop_params(a.drop.seg_p[seg0]);
+    drop_on = dr.on;
+  }
+
+  int32_t row_next[8], row_cur[DROP ? 8 : 1];
   u32x4 val[8], pf[NBJ][2];
   load_rows(wave, row_next);
   load_data(row_next, val);
   load_p(wave, pf);
+  if (DROP) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) row_cur[u] = row_next[u];
+  }
   load_rows(wave + kWgWaves, row_next);
 
   for (int step = wave; step < n_steps; step += kWgWaves) {
     // the next step's rows and token-side operand start their way from memory now
     u32x4 val_next[8], pf_next[NBJ][2];
+    int32_t row_keep[DROP ? 8 : 1];
     load_data(row_next, val_next);
     load_p(step + kWgWaves, pf_next);
+    if (DROP) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) row_keep[u] = row_next[u];
+    }
     load_rows(step + 2 * kWgWaves, row_next);
 
+    if (DROP && drop_on) {  // uniform over the workgroup
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        dr.on = row_cur[u] >= 0 && row_cur[u] < a.drop.rows;
+        val[u] = drop8<DT>(val[u], a.drop, dr, row_cur[u], (n0 + lcol) >> 3);
+      }
+    }
 #pragma unroll
     for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4*>(st + (8 * u + rlow) * kWgPitch + lcol) = val[u];
     // the wave's own LDS accesses are served in order; only the compiler must not move
@@ -234,6 +265,10 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int u = 0; u < 8; ++u) val[u] = val_next[u];
+    if (DROP) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) row_cur[u] = row_keep[u];
+    }
 #pragma unroll
     for (int jb = 0; jb < NBJ; ++jb) pf[jb][0] = pf_next[jb][0], pf[jb][1] = pf_next[jb][1];
   }
@@ -319,13 +354,13 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   }
 }
 
-template <int DT, int NBJ, int NW>
+template <int DT, int NBJ, int NW, bool DROP = false>
 __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
   constexpr int kStageBytes = NW * kWgSlots * kWgPitch * 2;
   constexpr int kTailBytes = (NW > 1 ? NW * 4 * kWaveSize * 16 : 0) + 16 * (64 + 4) * 4;  // red + store staging
   __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kTailBytes ? kStageBytes : kTailBytes];
   if ((int)blockIdx.x < a.chunks_a)  // uniform over the workgroup
-    wgrad_body<DT, NBJ, NW, true>(a, smem);
+    wgrad_body<DT, NBJ, NW, true, DROP>(a, smem);
   else
     wgrad_body<DT, NBJ, NW, false>(a, smem);
 }

@@ -554,6 +554,7 @@ struct ExpandArgs {
   int T, nt_max;
   ItemSpace items;           // chunk rows of projection p: its column chunks
   int w_kn;                  // tile-block kernel only: weights are stored [k][n]
+  DropArgs drop;             // DROP kernels (the backward's dX): the mask and factor applied to the stored values
 #ifdef SMLM_TUNING
   int dbg;                   // experiments: 1 = no weights / multiply, 2 = no read of y
 #endif
@@ -597,6 +598,7 @@ struct LineLane {
   int srow[2];        // the two y rows of the lane, -1 = none
   float scale[2];
   uint16_t* yrow[2];  // &y[srow[j]][chunk column + ocol]
+  DropRow drop[2];    // DROP kernels: dropout parameters of the two rows
 };
 
 template <int NQ>
@@ -609,9 +611,12 @@ __device__ __forceinline__ void load_y_lines(u32x4 (&yold)[NQ / 2][2], const Lin
       yold[h][j] = ldg16_or(L.yrow[j] + 64 * h, read_y && L.srow[j] >= 0 && ncol0 + 64 * h + L.ocol < d_out, zeros);
 }
 
-template <int DT, int NQ>
+// DROP: what is stored is the gradient with respect to x before its dropout: the value as it
+// would be stored otherwise, times the row's factor where the element was kept, zero elsewhere
+template <int DT, int NQ, bool DROP = false>
 __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ][2], const u32x4 (&yold)[NQ / 2][2],
-                                              const LineLane& L, int c, int g, int ncol0, int d_out, float beta) {
+                                              const LineLane& L, int c, int g, int ncol0, int d_out, float beta,
+                                              const DropArgs* dp = nullptr) {
 #pragma unroll
   for (int h = 0; h < NQ / 2; ++h) {
 #pragma unroll
@@ -648,6 +653,7 @@ __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ]
         o[2] = pack2<DT>(sc * hi4[j][0], sc * hi4[j][1]);
         o[3] = pack2<DT>(sc * hi4[j][2], sc * hi4[j][3]);
       }
+      if (DROP) o = drop8<DT>(o, *dp, L.drop[j], L.srow[j], (ncol0 + 64 * h + L.ocol) >> 3);
       stg16(L.yrow[j] + 64 * h, o);
     }
   }
@@ -659,7 +665,7 @@ __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ]
 // short: KS > 0 unrolls KS 32-wide k steps, KS == 0 is the general loop over k.
 // MFMA row m of column block (q,p) is output column 32q + 8(m/4) + 4p + m%4, so
 // that a lane's eight accumulators for one q are eight consecutive columns.
-template <int DT, int NQ, int KS, bool ROWMAJOR, bool DIRECT, bool VFOLD>
+template <int DT, int NQ, int KS, bool ROWMAJOR, bool DIRECT, bool VFOLD, bool DROP = false>
 __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) {
   __shared__ __attribute__((aligned(16))) float olds[kFwdWaves][kTileRows * kOPitch];
   const int units = DIRECT ? 0 : tile_units<1>(a.plan, 0);
@@ -696,6 +702,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
       L.srow[j] = a.plan.tile_row[tile * kTileRows + L.orow + 8 * j];
       sseg[j] = a.seg_scale ? a.plan.tile_rseg[tile * kTileRows + L.orow + 8 * j] : -1;
       L.yrow[j] = P.y + (long)(L.srow[j] < 0 ? 0 : L.srow[j]) * P.d_out + ncol0 + L.ocol;
+      if (DROP) L.drop[j] = drop_row(a.drop, L.srow[j], a.plan.tile_rseg, tile * kTileRows + L.orow + 8 * j);
     }
     u32x4 yold[NQ / 2][2];
     load_y_lines<NQ>(yold, L, ncol0, P.d_out, a.beta != 0.0f, zeros);
@@ -747,7 +754,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 #pragma unroll
         for (int p = 0; p < 2; ++p) acc[q][p] = Num<DT>::mfma(wf[q][p], vf, acc[q][p]);
     }
-    store_y_lines<DT, NQ>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
+    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta, &a.drop);
   }
 }
 
@@ -758,7 +765,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 // tiles instead of once per tile.
 // WKN: weights stored [k][n] (A [r, h_in] for the backward's dX = dV A): the chunk is staged
 // as it lies in memory and read out of LDS with the transposing read.
-template <int DT, int NQ, int KS, bool DIRECT, bool WKN>
+template <int DT, int NQ, int KS, bool DIRECT, bool WKN, bool DROP = false>
 __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a) {
   static_assert(NQ % 2 == 0, "the output is written 64 columns at a time");
   constexpr int kPitch = WKN ? 32 * NQ + 8 : 32 * KS + 8;  // LDS row pitch in 16-bit elements
@@ -792,6 +799,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
       L.srow[j] = active ? a.plan.tile_row[tslot + L.orow + 8 * j] : -1;
       sseg[j] = (a.seg_scale && active) ? a.plan.tile_rseg[tslot + L.orow + 8 * j] : -1;  // -1 on empty slots
       L.yrow[j] = P.y + (long)(L.srow[j] < 0 ? 0 : L.srow[j]) * P.d_out + ncol0 + L.ocol;
+      if (DROP) L.drop[j] = drop_row(a.drop, L.srow[j], a.plan.tile_rseg, tslot + L.orow + 8 * j);
     }
     const int rseg = (a.pt_a && a.seg_scale && active) ? a.plan.tile_rseg[slot] : -1;
     const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
@@ -875,7 +883,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
           acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
         }
 
-    store_y_lines<DT, NQ>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
+    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta, &a.drop);
   }
 }
 

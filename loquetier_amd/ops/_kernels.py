@@ -286,9 +286,11 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
 def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.Tensor,
                        dy: torch.Tensor, x: torch.Tensor, v: Optional[torch.Tensor],
                        a_ptrs: torch.Tensor, b_ptrs: torch.Tensor, plan: SegmentPlan, rank: int,
-                       part_scale: Optional[torch.Tensor] = None) -> None:
+                       part_scale: Optional[torch.Tensor] = None,
+                       dropout: Optional[DropoutSpec] = None) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
-    `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows)."""
+    `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
+    forward's stream with seg_p per partition; x is the tensor before dropout."""
     for t, n in ((dx, "dx"), (dy, "dy"), (x, "x"), (da_ptrs, "da_ptrs"), (db_ptrs, "db_ptrs"),
                  (a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs")):
         _check_input(t, n)
@@ -310,11 +312,14 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     with torch.cuda.device(dev):
         need = _lib.size_query("smlm_lora_bwd_workspace_size", n_rows, plan.S, NA, h_in, h_out, rank)
         ws = _workspace(dev, need)
-        rc = _lib.load().smlm_lora_bwd(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
-                                       dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
-                                       b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
-                                       ws.numel(), n_rows, plan.S, NA, h_in, h_out, rank, code,
-                                       _ptr(part_scale), _stream(dev))
+        if dropout is not None and dropout.rows < n_rows:
+            raise RuntimeError("the dropout descriptor must cover the backward's rows")
+        drop = None if dropout is None else C.byref(dropout.struct(plan))
+        rc = _lib.load().smlm_lora_bwd_dropout(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
+                                               dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
+                                               b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
+                                               ws.numel(), n_rows, plan.S, NA, h_in, h_out, rank, code,
+                                               _ptr(part_scale), drop, _stream(dev))
     _lib.check(rc, "smlm_lora_backward")
 
 

@@ -140,3 +140,96 @@ def test_forward_dropout_gaussian(K, oracle, gpu_device, dt, p):
     y_stage = np.zeros((T, h_out), np.float32)
     oracle.smlm_gemm(y_stage, to_np(v), [B[j] for j in ids], seg, False, dt)
     close(to_np(y), y_stage)
+
+
+# name, tp, part_ad, NA, h_in, h_out, r, per-adapter p
+BWD_CASES = [
+    ("two-parts", [0, 5, 12], [0, 1], 2, 64, 96, 8, [0.5, 0.5]),
+    ("shared-adapter", [0, 40, 70, 100], [1, 0, 1], 2, 128, 256, 16, [0.5, 0.0]),   # adapter 0 trains without dropout
+    ("empty-part", [0, 17, 17, 50], [0, 1, 2], 3, 256, 128, 32, [0.5, 0.5, 0.5]),
+    ("rank64", [0, 33, 90], [0, 1], 2, 192, 320, 64, [0.5, 0.5]),
+    ("in-place", [0, 500, 520, 1300], [2, 0, 2], 3, 256, 192, 16, [0.5, 0.0, 0.5]),  # 1024 rows and more: no transposes
+    ("many-rows", [0, 1100, 2300], [0, 1], 2, 320, 128, 32, [0.5, 0.5]),             # four-wave weight gradient
+    ("long-k", [0, 30, 75], [1, 0], 2, 4096, 2048, 16, [0.5, 0.5]),
+]
+
+
+def run_backward(K, d, dt, x, A, B, g, tp, part_ad, r, spec, v=None):
+    n_rows = tp[-1]
+    xd, gd = dev_t(x, dt, d), dev_t(g, dt, d)
+    Ad, Bd = [dev_t(a, dt, d) for a in A], [dev_t(b, dt, d) for b in B]
+    dA, dB = [torch.empty_like(a) for a in Ad], [torch.empty_like(b) for b in Bd]
+    dx = torch.full((n_rows + 3, x.shape[1]), 9.0, dtype=TDT[dt], device=d)
+    pi = torch.tensor(tp, dtype=torch.int32, device=d)
+    pa = torch.tensor(part_ad, dtype=torch.int32, device=d)
+    plan = K.SegmentPlan(pi, pa, n_rows)
+    K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), gd, xd, v, ptrs(Ad, d), ptrs(Bd, d), plan, r,
+                         dropout=spec)
+    return to_np(dx), [to_np(t) for t in dA], [to_np(t) for t in dB]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("with_v", [False, True])
+@pytest.mark.parametrize("case", BWD_CASES, ids=[c[0] for c in BWD_CASES])
+def test_backward_dropout_exact(K, oracle, gpu_device, case, dt, with_v):
+    """dX, dA, dB of a forward that ran with dropout: the oracle's backward on the dropped x,
+    then the mask and factor once more on its dX (autograd's dropout backward)."""
+    name, tp, part_ad, NA, h_in, h_out, r, ad_p = case
+    d = gpu_device
+    n_rows = tp[-1]
+    rng = np.random.default_rng(31)
+    x = oracle.round_to(dyadic(rng, (n_rows, h_in), 16, 8), dt)
+    A = [dyadic(rng, (r, h_in), 8, 64) for _ in range(NA)]
+    B = [dyadic(rng, (h_out, r), 8, 8) for _ in range(NA)]
+    g = dyadic(rng, (n_rows, h_out), 16, 8)
+    seg_p = np.array([ad_p[a] for a in part_ad], np.float32)
+    seed, offset = 4242, 9
+    spec = K.DropoutSpec(torch.from_numpy(seg_p).to(d), n_rows, seed, offset)
+    rp = row_probs(tp, seg_p, n_rows, n_rows)
+    xdrop = oracle.dropout_rows(x, rp, seed, offset, dt)
+    v = None
+    if with_v:  # the v the forward saved (of the dropped x)
+        _, vo = oracle.add_lora_forward(xdrop, [A[a] for a in part_ad], [B[a] for a in part_ad], tp, h_out, dt)
+        v = dev_t(vo, dt, d)
+    dx, dA, dB = run_backward(K, d, dt, x, A, B, g, tp, part_ad, r, spec, v)
+    gx, ga, gb = oracle.add_lora_backward(g, xdrop, A, B, tp, part_ad, dt)
+    gx = oracle.dropout_rows(gx, rp, seed, offset, dt)
+    covered = np.zeros(n_rows, bool)
+    for p in range(len(part_ad)):
+        covered[tp[p]:tp[p + 1]] = True
+    assert np.array_equal(dx[:n_rows][covered], gx[covered])
+    assert np.all(dx[n_rows:] == 9.0)
+    for a in range(NA):
+        assert np.array_equal(dA[a], ga[a]), f"dA[{a}]"
+        assert np.array_equal(dB[a], gb[a]), f"dB[{a}]"
+    # and the mask matters: without the descriptor dA differs wherever an adapter drops
+    _, dA_plain, _ = run_backward(K, d, dt, x, A, B, g, tp, part_ad, r, None)
+    for a in set(part_ad):
+        rows = sum(tp[i + 1] - tp[i] for i in range(len(part_ad)) if part_ad[i] == a)
+        if rows:
+            assert np.array_equal(dA_plain[a], dA[a]) == (ad_p[a] == 0.0)
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+def test_backward_dropout_gaussian(K, oracle, gpu_device, dt):
+    tp, part_ad, NA, h_in, h_out, r, ad_p = [0, 200, 500], [0, 1], 2, 512, 384, 16, [0.1, 0.25]
+    d = gpu_device
+    n_rows = tp[-1]
+    rng = np.random.default_rng(32)
+    x = oracle.round_to(rng.standard_normal((n_rows, h_in)), dt)
+    A = [oracle.round_to(rng.standard_normal((r, h_in)) / np.sqrt(h_in), dt) for _ in range(NA)]
+    B = [oracle.round_to(rng.standard_normal((h_out, r)) / np.sqrt(r), dt) for _ in range(NA)]
+    g = oracle.round_to(rng.standard_normal((n_rows, h_out)), dt)
+    seg_p = np.array([ad_p[a] for a in part_ad], np.float32)
+    spec = K.DropoutSpec(torch.from_numpy(seg_p).to(d), n_rows, 1, 2)
+    rp = row_probs(tp, seg_p, n_rows, n_rows)
+    xdrop = oracle.dropout_rows(x, rp, 1, 2, dt)
+    dx, dA, dB = run_backward(K, d, dt, x, A, B, g, tp, part_ad, r, spec)
+    gx, ga, gb = oracle.add_lora_backward(g, xdrop, A, B, tp, part_ad, dt)
+    keep = oracle.dropout_mask(n_rows, h_in, rp, 1, 2).astype(bool)
+    gx = oracle.dropout_rows(gx, rp, 1, 2, dt)
+    assert not dx[:n_rows][~keep].any()               # dropped positions: exactly zero
+    close(dx[:n_rows], gx, atol=ATOL if dt == "fp16" else 6e-3)
+    for a in range(NA):
+        close(dA[a], ga[a], atol=ATOL * max(1.0, float(np.abs(ga[a]).max())))
+        close(dB[a], gb[a], atol=ATOL * max(1.0, float(np.abs(gb[a]).max())))
