@@ -194,6 +194,9 @@ def main():
     ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
     ap.add_argument("--eager", action="store_true",
                     help="launch the steps one by one instead of replaying a graph (for counter runs)")
+    ap.add_argument("--dropout", type=float, default=0.0,
+                    help="dropout probability of the training adapters (workloads with a backward): the "
+                         "kernels regenerate the mask in the forward and the backward; default 0 = off")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a 128 MiB device copy three times before the timed region: a kernel "
                          "of known traffic to scale FETCH_SIZE / WRITE_SIZE readings with")
@@ -272,12 +275,23 @@ def main():
         part_indptr = torch.tensor(w["seg"][:P + 1], dtype=torch.int32, device=dev)
         part_ad = torch.tensor([train.index(a) for a in w["ids"][:P]], dtype=torch.int32, device=dev)
         part_scale = torch.full((P,), 2.0, device=dev)
+    drop_f = drop_b = None
+    if P and args.dropout > 0:
+        seg_p = torch.zeros(S, device=dev)
+        seg_p[:P] = args.dropout
+        # the forward leaves the keep bits of every projection's mask end to end; the backward of
+        # projection i reads its part
+        widths = [hi for _, hi, _ in w["proj"]]
+        bits = torch.empty(K.DropoutSpec.mask_nbytes(n_train, widths), dtype=torch.uint8, device=dev)
+        drop_f = K.DropoutSpec(seg_p, n_train, 1, 0, bits)
+        starts = [K.DropoutSpec.mask_nbytes(n_train, widths[:i]) for i in range(len(widths))]
+        drop_b = [K.DropoutSpec(seg_p[:P].contiguous(), n_train, 1, i, bits[starts[i]:]) for i in range(len(widths))]
 
     def fwd(st, stages=3):
         pr = st["proj"]
         K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
                                   [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
-                                  v_out=[d["v"] for d in pr] if P else None, stages=stages)
+                                  v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f)
 
     def step(st, build_plan=True):
         if build_plan:
@@ -285,9 +299,10 @@ def main():
         fwd(st)
         if P:
             bplan = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
-            for d in st["proj"]:
+            for i, d in enumerate(st["proj"]):
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
-                                     d["ta_tab"], d["tb_tab"], bplan, r, part_scale)
+                                     d["ta_tab"], d["tb_tab"], bplan, r, part_scale,
+                                     dropout=drop_b[i] if drop_b else None)
 
     # eager once on the capture stream (sizes its workspace outside any capture)
     cap_stream = torch.cuda.Stream()
@@ -429,7 +444,8 @@ def main():
         "config": {"workload": w["name"], "tokens_per_step": T, "segments": S, "adapters": NA, "rank": r,
                    "projections": [f"{n}:{a}->{b}" for n, a, b in w["proj"]],
                    "buffer_sets_rotated": R, "step_includes": "plan build + fused forward per projection"
-                   + (" + backward" if P else ""), "graph_replay": not args.eager},
+                   + (" + backward" if P else ""), "graph_replay": not args.eager,
+                   "dropout": args.dropout if P else 0.0},
         "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
         "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),

@@ -205,12 +205,19 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
  *   seed, offset : the stream; the same pair must be passed to the forward and to
  *            the backward of one layer.  Projection i of a multi-projection call
  *            uses offset + i.
+ *   mask_bits : optional device buffer for the keep bits, one byte per eight
+ *            columns of a training row ([rows, h_in / 8] bytes; bit e of a byte =
+ *            element 8*block + e is kept; the projections of a multi-projection call
+ *            lie end to end).  The forward fills it when given (bytes of rows whose
+ *            p is 0 are left alone); the backward reads it when given and otherwise
+ *            regenerates the same bits into its workspace.  NULL is always valid.
  */
 typedef struct smlm_dropout {
   const float* seg_p;
   int rows;
   uint64_t seed;
   uint64_t offset;
+  void* mask_bits;
 } smlm_dropout;
 
 /* smlm_lora_fwd_multi with dropout of x (NULL descriptor: identical to it). */

@@ -24,7 +24,8 @@ _pvp = C.POINTER(C.c_void_p)
 
 class Dropout(C.Structure):
     """struct smlm_dropout of include/smlm.h."""
-    _fields_ = [("seg_p", C.c_void_p), ("rows", C.c_int), ("seed", C.c_uint64), ("offset", C.c_uint64)]
+    _fields_ = [("seg_p", C.c_void_p), ("rows", C.c_int), ("seed", C.c_uint64), ("offset", C.c_uint64),
+                ("mask_bits", C.c_void_p)]
 
 
 _pdrop = C.POINTER(Dropout)

@@ -22,6 +22,8 @@ struct DropArgs {
   int rows;            // training rows are [0, rows)
   uint32_t k0, k1;     // seed
   uint32_t o0, o1;     // offset (distinguishes layers / steps)
+  uint8_t* bits;       // optional [rows, bits_pitch]: keep bits, one byte per eight columns of a row;
+  long bits_pitch;     //   written by the forward's shrink, read by the backward instead of regenerating
 };
 
 // the arguments of projection pj of a launch over several projections: offset + pj
@@ -73,20 +75,70 @@ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
   out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
 }
 
-// eight consecutive elements of one row (columns 8*colblk .. +7), packed two to a word
-template <int DT>
-__device__ __forceinline__ u32x4 drop8(u32x4 v, const DropArgs& d, const DropRow& r, int row, int colblk) {
-  if (__builtin_amdgcn_ballot_w64(r.on) == 0) return v;  // uniform over the wave
+// keep bits (bit e = element e is kept) of the eight elements at columns 8*colblk .. +7 of a row
+__device__ __forceinline__ uint32_t drop_keep8(const DropArgs& d, uint32_t thresh, int row, int colblk) {
   uint32_t w[4];
   philox4x32_10((uint32_t)row, (uint32_t)colblk, d.o0, d.o1, d.k0, d.k1, w);
+  uint32_t keep = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    keep |= ((w[e] & 0xffffu) >= thresh ? 1u << (2 * e) : 0u) | ((w[e] >> 16) >= thresh ? 2u << (2 * e) : 0u);
+  return keep;
+}
+
+// kept elements times the factor (float product, rounded to the 16-bit type), dropped ones +0
+template <int DT>
+__device__ __forceinline__ u32x4 drop_apply8(u32x4 v, uint32_t keep, float scale) {
   u32x4 o;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const uint32_t scaled = pack2<DT>(Num<DT>::lo(v[e]) * r.scale, Num<DT>::hi(v[e]) * r.scale);
-    const uint32_t keep = ((w[e] & 0xffffu) >= r.thresh ? 0x0000ffffu : 0u) | ((w[e] >> 16) >= r.thresh ? 0xffff0000u : 0u);
-    o[e] = r.on ? (scaled & keep) : v[e];
+    const uint32_t scaled = pack2<DT>(Num<DT>::lo(v[e]) * scale, Num<DT>::hi(v[e]) * scale);
+    const uint32_t m = ((0u - ((keep >> (2 * e)) & 1u)) & 0x0000ffffu) | ((0u - ((keep >> (2 * e + 1)) & 1u)) & 0xffff0000u);
+    o[e] = scaled & m;
   }
   return o;
+}
+
+// Eight consecutive elements of one row (columns 8*colblk .. +7), packed two to a word.
+// bits_out (may be nullptr): the row's keep bits, one byte per eight columns, are left there
+// for a later pass that reads them instead of running the generator again (write != false
+// selects the lanes that own the byte).
+template <int DT>
+__device__ __forceinline__ u32x4 drop8(u32x4 v, const DropArgs& d, const DropRow& r, int row, int colblk,
+                                       uint8_t* bits_out = nullptr, long bits_pitch = 0, bool write = false) {
+  if (__builtin_amdgcn_ballot_w64(r.on) == 0) return v;  // uniform over the wave
+  const uint32_t keep = drop_keep8(d, r.thresh, row, colblk);
+  if (bits_out && write && r.on) bits_out[(long)row * bits_pitch + colblk] = (uint8_t)keep;
+  const u32x4 o = drop_apply8<DT>(v, keep, r.scale);
+  return r.on ? o : v;
+}
+
+// the same from stored keep bits
+template <int DT>
+__device__ __forceinline__ u32x4 drop8_bits(u32x4 v, const DropRow& r, uint32_t keep) {
+  if (__builtin_amdgcn_ballot_w64(r.on) == 0) return v;
+  const u32x4 o = drop_apply8<DT>(v, keep, r.scale);
+  return r.on ? o : v;
+}
+
+// Keep bits of every training row of a planned batch, for the kernels that apply a stored
+// mask: workgroup -> tile, thread -> (row slot, column blocks slot-strided by 16).
+struct DropBitsArgs {
+  const int32_t* hdr;        // plan header: [0] = number of tiles
+  const int32_t* tile_row;
+  const int32_t* tile_rseg;
+  DropArgs drop;             // bits / bits_pitch name the output
+};
+
+__global__ __launch_bounds__(256) void drop_bits_kernel(DropBitsArgs a) {
+  const int tile = blockIdx.x;
+  if (tile >= a.hdr[0]) return;
+  const int slot = tile * kTileRows + (threadIdx.x >> 4);
+  const int row = a.tile_row[slot];
+  const DropRow r = drop_row(a.drop, row, a.tile_rseg, slot);
+  if (!r.on) return;  // rows that are not dropped never have their byte read
+  for (int cb = threadIdx.x & 15; cb < a.drop.bits_pitch; cb += 16)
+    a.drop.bits[(long)row * a.drop.bits_pitch + cb] = (uint8_t)drop_keep8(a.drop, r.thresh, row, cb);
 }
 
 }  // namespace smlm

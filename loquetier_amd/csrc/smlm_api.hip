@@ -339,6 +339,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   ReduceArgs ra{};
   bool need_reduce = false;
   ShrinkCfg c0{};
+  size_t bits_off = 0;
   const int nw = row_major ? kFwdWaves : shrink_waves(T, nproj, d_in, d_out);
   for (int i = 0; i < nproj; ++i) {
     const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw);
@@ -351,6 +352,10 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
     P.d_in = d_in[i]; P.d_out = d_out; P.ldw = ldw[i];
     P.k_per_wave = c.k_per_wave; P.ksplit = c.ksplit; P.zblocks = c.zblocks;
     P.to_partial = fold ? 0 : 1;
+    if (drop && drop->bits) {  // projections' masks lie end to end
+      P.drop_bits = drop->bits + bits_off;
+      bits_off += (size_t)drop->rows * (d_in[i] / 8);
+    }
     a.items.row_start[i + 1] = a.items.row_start[i] + c.ksplit * c.zblocks;
     ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit};
     need_reduce = need_reduce || c.ksplit > 1;
@@ -391,7 +396,7 @@ int launch_wgrad(int nbj, bool split, dim3 grid, hipStream_t st, const WgradArgs
 }
 
 struct BwdLayout {
-  size_t at, bt, at_ptrs, bt_ptrs, partial, dv16, v16, pt_a, pt_b, total;
+  size_t at, bt, at_ptrs, bt_ptrs, partial, dv16, v16, pt_a, pt_b, bits, total;
   long pitch;
   ShrinkCfg cfg_dv, cfg_v;
 };
@@ -418,6 +423,7 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
   L.v16 = take((size_t)n_rows * r * 2);
   L.pt_a = take((size_t)r * L.pitch * 2);
   L.pt_b = take((size_t)r * L.pitch * 2);
+  L.bits = take((size_t)n_rows * (h_in / 8));  // keep bits of x's dropout mask when the caller has none
   L.total = off;
   return L;
 }
@@ -580,6 +586,7 @@ static int drop_args(const smlm_dropout* d, DropArgs* out) {
   out->rows = d->rows;
   out->k0 = (uint32_t)d->seed; out->k1 = (uint32_t)(d->seed >> 32);
   out->o0 = (uint32_t)d->offset; out->o1 = (uint32_t)(d->offset >> 32);
+  out->bits = reinterpret_cast<uint8_t*>(d->mask_bits);
   return SMLM_OK;
 }
 
@@ -764,11 +771,24 @@ SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* 
     if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
   }
 
+  // The keep bits of x's dropout mask: the forward's when the caller kept them, else made here
+  // (same stream, same bits) so that the kernels below apply a stored mask either way.
+  if (drop.seg_p) {
+    drop.bits_pitch = h_in / 8;
+    if (!drop.bits) {
+      drop.bits = reinterpret_cast<uint8_t*>(ws + L.bits);
+      const DropBitsArgs ba{pv.hdr, pv.tile_row, pv.tile_rseg, drop};
+      if ((rc = launch(drop_bits_kernel, dim3((unsigned)pv.nt_max), dim3(256), st, ba))) return rc;
+    }
+  }
+
   // 2. v = round16(x A^T) unless the forward saved it
   const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
   if (!vv) {
+    DropArgs vdrop = drop;
+    vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
-                         0.0f, nullptr, st, true, false, &drop)))  // v of the dropped x, as the forward made it
+                         0.0f, nullptr, st, true, false, &vdrop)))  // v of the dropped x, as the forward made it
       return rc;
     vv = reinterpret_cast<const uint16_t*>(v16);
   }

@@ -110,9 +110,10 @@ __device__ __forceinline__ int wg_lds_row(int s) {
 // inside the loop, and the rows of the next step are already on their way from
 // memory while the current step is multiplied.
 //
-// DROP (dA only): the forward multiplied the dropped x, so dA = dV^T dropout(x).  The mask is
-// regenerated while the rows are staged; every row of the workgroup belongs to one adapter,
-// whose probability is read once from the group's first segment.
+// DROP (dA only): the forward multiplied the dropped x, so dA = dV^T dropout(x).  The keep
+// bits (one byte per eight columns, a.drop.bits) travel with the rows and are applied while the
+// rows are staged; every row of the workgroup belongs to one adapter, whose probability is read
+// once from the group's first segment.
 template <int DT, int NBJ, int NW, bool IS_A, bool DROP = false>
 __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   constexpr int kWgWaves = NW;
@@ -175,11 +176,17 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       row[u] = (step < n_steps && tile < t_end) ? a.tile_row[tile * kTileRows + (s & 15)] : -1;
     }
   };
-  auto load_data = [&](const int32_t (&row)[8], u32x4 (&val)[8]) {
+  const uint8_t* zero_bytes = reinterpret_cast<const uint8_t*>(zeros);
+  auto load_data = [&](const int32_t (&row)[8], u32x4 (&val)[8], uint32_t (&keep)[DROP ? 8 : 1]) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const bool ok = row[u] >= 0 && col_ok;
       val[u] = ldg16_or(Q + (long)row[u] * h + n0 + lcol, ok, zeros);
+      if (DROP) {  // rows at or past drop.rows keep everything: their byte is never applied
+        const bool dropped = ok && row[u] < a.drop.rows;
+        keep[u] = *(const SMLM_GLOBAL uint8_t*)(dropped ? a.drop.bits + (long)row[u] * a.drop.bits_pitch + ((n0 + lcol) >> 3)
+                                                        : zero_bytes) | (dropped ? 0u : 0x100u);
+      }
     }
   };
   auto load_p = [&](int step, u32x4 (&pf)[NBJ][2]) {
@@ -202,34 +209,27 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
     drop_on = dr.on;
   }
 
-  int32_t row_next[8], row_cur[DROP ? 8 : 1];
+  int32_t row_next[8];
+  uint32_t keep[DROP ? 8 : 1];  // bit 8 set: the row is not dropped
   u32x4 val[8], pf[NBJ][2];
   load_rows(wave, row_next);
-  load_data(row_next, val);
+  load_data(row_next, val, keep);
   load_p(wave, pf);
-  if (DROP) {
-#pragma unroll
-    for (int u = 0; u < 8; ++u) row_cur[u] = row_next[u];
-  }
   load_rows(wave + kWgWaves, row_next);
 
   for (int step = wave; step < n_steps; step += kWgWaves) {
     // the next step's rows and token-side operand start their way from memory now
     u32x4 val_next[8], pf_next[NBJ][2];
-    int32_t row_keep[DROP ? 8 : 1];
-    load_data(row_next, val_next);
+    uint32_t keep_next[DROP ? 8 : 1];
+    load_data(row_next, val_next, keep_next);
     load_p(step + kWgWaves, pf_next);
-    if (DROP) {
-#pragma unroll
-      for (int u = 0; u < 8; ++u) row_keep[u] = row_next[u];
-    }
     load_rows(step + 2 * kWgWaves, row_next);
 
     if (DROP && drop_on) {  // uniform over the workgroup
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        dr.on = row_cur[u] >= 0 && row_cur[u] < a.drop.rows;
-        val[u] = drop8<DT>(val[u], a.drop, dr, row_cur[u], (n0 + lcol) >> 3);
+        dr.on = (keep[u] & 0x100u) == 0;
+        val[u] = drop8_bits<DT>(val[u], dr, keep[u]);
       }
     }
 #pragma unroll
@@ -267,7 +267,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
     for (int u = 0; u < 8; ++u) val[u] = val_next[u];
     if (DROP) {
 #pragma unroll
-      for (int u = 0; u < 8; ++u) row_cur[u] = row_keep[u];
+      for (int u = 0; u < 8; ++u) keep[u] = keep_next[u];
     }
 #pragma unroll
     for (int jb = 0; jb < NBJ; ++jb) pf[jb][0] = pf_next[jb][0], pf[jb][1] = pf_next[jb][1];

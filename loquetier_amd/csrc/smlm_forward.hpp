@@ -171,6 +171,7 @@ struct ShrinkProj {
   uint16_t* out;              // [T, d_out] when ksplit == 1
   int d_in, d_out, ldw, k_per_wave, ksplit, zblocks;
   int to_partial;             // write the fp32 partial even when ksplit == 1 (the consumer rounds)
+  uint8_t* drop_bits;         // DROP kernels, optional: [rows, d_in / 8] keep bits of this projection's mask
 };
 
 struct ShrinkArgs {
@@ -247,7 +248,8 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
     auto multiply = [&](int k, const u32x4 (&xf)[U], const u32x4 (&wf)[NB][U]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const u32x4 xu = DROP ? drop8<DT>(xf[u], dp, dr, row, (k + 32 * u + 8 * g) >> 3) : xf[u];
+        const int kk = k + 32 * u + 8 * g;
+        const u32x4 xu = DROP ? drop8<DT>(xf[u], dp, dr, row, kk >> 3, P.drop_bits, P.d_in >> 3, zb == 0 && kk < kend) : xf[u];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(wf[nb][u], xu, acc[nb]);
       }
@@ -425,7 +427,8 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
       if (active) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          const u32x4 xu = DROP ? drop8<DT>(xf[u], dp, dr, row, (kb + 32 * u + 8 * g) >> 3) : xf[u];
+          const int kk = kb + 32 * u + 8 * g;
+          const u32x4 xu = DROP ? drop8<DT>(xf[u], dp, dr, row, kk >> 3, P.drop_bits, P.d_in >> 3, zb == 0 && kk < kend) : xf[u];
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(weight_frag(buf, u, nb), xu, acc[nb]);
         }
@@ -598,8 +601,25 @@ struct LineLane {
   int srow[2];        // the two y rows of the lane, -1 = none
   float scale[2];
   uint16_t* yrow[2];  // &y[srow[j]][chunk column + ocol]
-  DropRow drop[2];    // DROP kernels: dropout parameters of the two rows
+  DropRow drop[2];    // DROP kernels: dropout parameters of the two rows ...
+  uint32_t keep[2][2];  // ... and the keep bits of their 64-column pieces [h][j]
 };
+
+// keep bits of the pieces a lane will store (DROP kernels): requested with the other loads of
+// the item; rows that are not dropped read a zero byte that is never applied
+template <int NQ>
+__device__ __forceinline__ void load_keep_bits(LineLane& L, const DropArgs& d, int ncol0, int d_out,
+                                               const uint16_t* zeros) {
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int h = 0; h < NQ / 2; ++h) {
+      const int col = ncol0 + 64 * h + L.ocol;
+      const bool ok = L.srow[j] >= 0 && L.srow[j] < d.rows && col < d_out;  // whatever the row's probability
+      L.keep[h][j] = *(const SMLM_GLOBAL uint8_t*)(ok ? d.bits + (long)L.srow[j] * d.bits_pitch + (col >> 3)
+                                                      : reinterpret_cast<const uint8_t*>(zeros));
+    }
+}
 
 template <int NQ>
 __device__ __forceinline__ void load_y_lines(u32x4 (&yold)[NQ / 2][2], const LineLane& L, int ncol0, int d_out,
@@ -615,8 +635,7 @@ __device__ __forceinline__ void load_y_lines(u32x4 (&yold)[NQ / 2][2], const Lin
 // would be stored otherwise, times the row's factor where the element was kept, zero elsewhere
 template <int DT, int NQ, bool DROP = false>
 __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ][2], const u32x4 (&yold)[NQ / 2][2],
-                                              const LineLane& L, int c, int g, int ncol0, int d_out, float beta,
-                                              const DropArgs* dp = nullptr) {
+                                              const LineLane& L, int c, int g, int ncol0, int d_out, float beta) {
 #pragma unroll
   for (int h = 0; h < NQ / 2; ++h) {
 #pragma unroll
@@ -653,7 +672,7 @@ __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ]
         o[2] = pack2<DT>(sc * hi4[j][0], sc * hi4[j][1]);
         o[3] = pack2<DT>(sc * hi4[j][2], sc * hi4[j][3]);
       }
-      if (DROP) o = drop8<DT>(o, *dp, L.drop[j], L.srow[j], (ncol0 + 64 * h + L.ocol) >> 3);
+      if (DROP) o = drop8_bits<DT>(o, L.drop[j], L.keep[h][j]);
       stg16(L.yrow[j] + 64 * h, o);
     }
   }
@@ -706,6 +725,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     }
     u32x4 yold[NQ / 2][2];
     load_y_lines<NQ>(yold, L, ncol0, P.d_out, a.beta != 0.0f, zeros);
+    if (DROP) load_keep_bits<NQ>(L, a.drop, ncol0, P.d_out, zeros);
 #pragma unroll
     for (int j = 0; j < 2; ++j) L.scale[j] = sseg[j] >= 0 ? a.seg_scale[sseg[j]] : 1.0f;
 
@@ -754,7 +774,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 #pragma unroll
         for (int p = 0; p < 2; ++p) acc[q][p] = Num<DT>::mfma(wf[q][p], vf, acc[q][p]);
     }
-    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta, &a.drop);
+    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
   }
 }
 
@@ -833,6 +853,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
 #endif
     u32x4 yold[NQ / 2][2];
     load_y_lines<NQ>(yold, L, ncol0, P.d_out, read_y, zeros);
+    if (DROP) load_keep_bits<NQ>(L, a.drop, ncol0, P.d_out, zeros);
     u32x4 vf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -883,7 +904,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
           acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
         }
 
-    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta, &a.drop);
+    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
   }
 }
 

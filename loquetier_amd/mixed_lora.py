@@ -107,18 +107,27 @@ class fused_add_lora(Function):
     """result <- result + scale_seg * (x A_seg^T) B_seg^T, in place, one call.
 
     Arguments: (result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-    train_len, train_partition, *weights); the tables hold one address per
-    adapter and the plan is keyed by adapter id.  Returns `result`.
+    train_len, train_partition, dropout, *weights); the tables hold one address
+    per adapter and the plan is keyed by adapter id.  `dropout` (a
+    kernel.DropoutSpec or None) drops the training rows of x inside the kernels,
+    in place of the reference's nn.Dropout calls and torch.cat before the op
+    (src/loquetier_src/models/mixed_lora.py:185-192); x is the tensor before
+    dropout.  Returns `result`.
     Gradients: result -> passed through, x -> dX on train rows (zero elsewhere),
     each trainable weight -> its summed gradient (None when not training)."""
 
     @staticmethod
     def forward(ctx: FunctionCtx, result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-                train_len, train_partition, *weights):
+                train_len, train_partition, dropout, *weights):
         need_v = len(weights) > 0 and train_len > 0
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
+        if dropout is not None and need_v and dropout.mask_bits is None:
+            # the backward reads the forward's keep bits (1/16 of x's bytes) instead of making them again
+            bits = torch.empty(kernel.DropoutSpec.mask_nbytes(dropout.rows, x.size(1)), dtype=torch.uint8,
+                               device=x.device)
+            dropout = kernel.DropoutSpec(dropout.seg_p, dropout.rows, dropout.seed, dropout.offset, bits)
         kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
-                                 beta=1.0, v_out=v)
+                                 beta=1.0, v_out=v, dropout=dropout)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
@@ -127,23 +136,28 @@ class fused_add_lora(Function):
         # scale of each train partition = scale of the segment that starts it;
         # kept as a device gather so nothing is read back to the host
         ctx.part_scale = None
-        if need_v and seg_scale is not None:
+        ctx.part_drop = None
+        if need_v and (seg_scale is not None or dropout is not None):
             starts = torch.tensor([int(t) for t in train_partition][: ctx.n_parts],
                                   dtype=torch.int32, device=x.device)
-            seg_of = torch.searchsorted(plan.segment, starts, right=True) - 1
-            ctx.part_scale = seg_scale[seg_of.clamp_(0, plan.S - 1)].contiguous()
+            seg_of = (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, plan.S - 1)
+            if seg_scale is not None:
+                ctx.part_scale = seg_scale[seg_of].contiguous()
+            if dropout is not None:  # the same stream, probabilities by train partition
+                ctx.part_drop = kernel.DropoutSpec(dropout.seg_p[seg_of].contiguous(), train_len,
+                                                   dropout.seed, dropout.offset, dropout.mask_bits)
         if need_v:
             ctx.save_for_backward(x[:train_len, ...], v[:train_len, ...], *weights)
         return result
 
     @staticmethod
     def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
-        n_fixed = 9
+        n_fixed = 10
         if not ctx.has_v:
             return (grad_output, None) + (None,) * (n_fixed - 2) + (None,) * (2 * ctx.n_parts)
         x, v, *weight_list = ctx.saved_tensors
         grad_x, grads = lora_backward(grad_output, x, v, weight_list, ctx.tp, ctx.rank,
-                                      part_scale=ctx.part_scale)
+                                      part_scale=ctx.part_scale, dropout=ctx.part_drop)
         return (grad_output, grad_x) + (None,) * (n_fixed - 2) + tuple(grads)
 
 
@@ -199,7 +213,19 @@ class MixedLoraLinear(nn.Module):
         train_idx = ctx.train_idx
 
         x = x.to(self.dtype)
-        if blen.tlen > 0:
+        drop_spec = None
+        if blen.tlen > 0 and self.fused:
+            # the kernels drop the training rows themselves: no dropped copy, no torch.cat
+            probs = [float(a.dropout.p) if isinstance(a.dropout, nn.Dropout) and a.dropout.training else 0.0
+                     for a in self.adapters]
+            if any(probs[idx] > 0.0 for idx in train_idx):
+                seg_p = torch.tensor(probs, dtype=torch.float32, device=self.device)[
+                    ctx.seg_adapter(self.device).long()]
+                # the stream: torch's seed, and an offset drawn from torch's generator so that every
+                # call (layer, step) gets its own mask and torch.manual_seed makes runs repeatable
+                offset = int(torch.randint(0, 2 ** 62, (1,)).item())
+                drop_spec = kernel.DropoutSpec(seg_p, blen.tlen, torch.initial_seed(), offset)
+        elif blen.tlen > 0:
             dropped_x = []
             for idx, pi in zip(train_idx, range(len(blen.train_partition) - 1)):
                 start, end = blen.train_partition[pi], blen.train_partition[pi + 1]
@@ -215,7 +241,7 @@ class MixedLoraLinear(nn.Module):
                 x = x.contiguous()
             result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale,
                                           ctx.plan(self.device, x.size(0)), self.rank, blen.tlen,
-                                          blen.train_partition, *weights)
+                                          blen.train_partition, drop_spec, *weights)
             return result.to(torch_result_dtype)
 
         segment = ctx.segment.to(self.device)

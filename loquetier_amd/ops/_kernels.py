@@ -206,22 +206,36 @@ class DropoutSpec:
     the pair its forward used.  Replaces the nn.Dropout calls and the torch.cat of
     MixedLoraLinear.forward (src/loquetier_src/models/mixed_lora.py:185-192)."""
 
-    def __init__(self, seg_p: torch.Tensor, rows: int, seed: int, offset: int):
+    def __init__(self, seg_p: torch.Tensor, rows: int, seed: int, offset: int,
+                 mask_bits: Optional[torch.Tensor] = None):
         _check_input(seg_p, "seg_p")
         if seg_p.dtype != torch.float32 or seg_p.dim() != 1:
             raise RuntimeError("seg_p must be a 1D float32 tensor")
         if rows < 0:
             raise RuntimeError("rows must not be negative")
+        if mask_bits is not None:
+            _check_input(mask_bits, "mask_bits")
+            if mask_bits.dtype != torch.uint8:
+                raise RuntimeError("mask_bits must be a uint8 tensor")
         self.seg_p, self.rows = seg_p, int(rows)
         self.seed, self.offset = int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1)
+        self.mask_bits = mask_bits
+
+    @staticmethod
+    def mask_nbytes(rows: int, h_in) -> int:
+        """Size of mask_bits for `rows` training rows; h_in: one width or one per projection."""
+        widths = [h_in] if isinstance(h_in, int) else list(h_in)
+        return sum(int(rows) * (int(h) // 8) for h in widths)
 
     def with_offset(self, offset: int) -> "DropoutSpec":
-        return DropoutSpec(self.seg_p, self.rows, self.seed, offset)
+        return DropoutSpec(self.seg_p, self.rows, self.seed, offset, self.mask_bits)
 
-    def struct(self, plan: "SegmentPlan"):
+    def struct(self, plan: "SegmentPlan", widths):
         if self.seg_p.size(0) != plan.S or self.seg_p.device != plan.segment.device:
             raise RuntimeError("seg_p must have one entry per segment of the plan, on its device")
-        return _lib.Dropout(self.seg_p.data_ptr(), self.rows, self.seed, self.offset)
+        if self.mask_bits is not None and self.mask_bits.numel() < self.mask_nbytes(self.rows, widths):
+            raise RuntimeError(f"mask_bits needs {self.mask_nbytes(self.rows, widths)} bytes")
+        return _lib.Dropout(self.seg_p.data_ptr(), self.rows, self.seed, self.offset, _ptr(self.mask_bits))
 
 
 def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_ptrs: torch.Tensor,
@@ -273,7 +287,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
         _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(n, plan.T, h_in, rank, C.byref(need)),
                    "smlm_lora_fwd_multi_workspace_size")
         ws = _workspace(dev, need.value)
-        drop = None if dropout is None else C.byref(dropout.struct(plan))
+        drop = None if dropout is None else C.byref(dropout.struct(plan, [x.size(1) for x in xs]))
         rc = _lib.load().smlm_lora_fwd_multi_dropout(
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
@@ -314,7 +328,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
         ws = _workspace(dev, need)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
-        drop = None if dropout is None else C.byref(dropout.struct(plan))
+        drop = None if dropout is None else C.byref(dropout.struct(plan, h_in))
         rc = _lib.load().smlm_lora_bwd_dropout(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
                                                dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
                                                b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),

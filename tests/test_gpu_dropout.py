@@ -94,7 +94,9 @@ def test_forward_dropout_exact(K, oracle, gpu_device, case, dt):
     rng = np.random.default_rng(21)
     x, A, B, xd, Ad, Bd, plan, seg_p = setup(K, rng, case, dt, d)
     seed, offset = 0x5eed5eed5eed, (1 << 32) - 1   # the offset carries into its high word for projection 1
-    spec = K.DropoutSpec(torch.from_numpy(seg_p).to(d), train_rows, seed, offset)
+    bits = torch.full((2, train_rows, h_in // 8), 0xAA, dtype=torch.uint8, device=d)
+    assert bits.numel() == K.DropoutSpec.mask_nbytes(train_rows, [h_in, h_in])
+    spec = K.DropoutSpec(torch.from_numpy(seg_p).to(d), train_rows, seed, offset, mask_bits=bits)
     y0 = dyadic(rng, (T, h_out), 8, 4)
     rp = row_probs(seg, seg_p, T, train_rows)
     # two projections sharing x: each gets its own mask (offset + i), as two modules of the reference would
@@ -113,6 +115,14 @@ def test_forward_dropout_exact(K, oracle, gpu_device, case, dt):
         assert np.array_equal(to_np(vs[i])[covered], vo[covered])
         assert np.array_equal(to_np(ys[i]), yo)
         outs.append(yo)
+        # the keep bits the forward left behind: bit e of byte b of a row = element 8b + e is kept;
+        # rows that are not dropped (p = 0, outside every segment) keep the buffer's old bytes
+        keep = oracle.dropout_mask(train_rows, h_in, rp[:train_rows], seed, offset + i)
+        want_bits = np.packbits(keep, axis=1, bitorder="little")
+        dropped = covered[:train_rows] & (rp[:train_rows] > 0)
+        got_bits = bits[i].cpu().numpy()
+        assert np.array_equal(got_bits[dropped], want_bits[dropped])
+        assert np.all(got_bits[~dropped] == 0xAA)
     assert not np.array_equal(outs[0], outs[1])   # the two masks differ
     # without the descriptor nothing is dropped
     y_plain = dev_t(y0, dt, d)
@@ -169,9 +179,10 @@ def run_backward(K, d, dt, x, A, B, g, tp, part_ad, r, spec, v=None):
 
 
 @pytest.mark.parametrize("dt", ["fp16", "bf16"])
-@pytest.mark.parametrize("with_v", [False, True])
+@pytest.mark.parametrize("with_v,with_bits", [(False, False), (True, False), (True, True)],
+                         ids=["recompute", "saved-v", "saved-v-and-bits"])
 @pytest.mark.parametrize("case", BWD_CASES, ids=[c[0] for c in BWD_CASES])
-def test_backward_dropout_exact(K, oracle, gpu_device, case, dt, with_v):
+def test_backward_dropout_exact(K, oracle, gpu_device, case, dt, with_v, with_bits):
     """dX, dA, dB of a forward that ran with dropout: the oracle's backward on the dropped x,
     then the mask and factor once more on its dX (autograd's dropout backward)."""
     name, tp, part_ad, NA, h_in, h_out, r, ad_p = case
@@ -191,6 +202,15 @@ def test_backward_dropout_exact(K, oracle, gpu_device, case, dt, with_v):
     if with_v:  # the v the forward saved (of the dropped x)
         _, vo = oracle.add_lora_forward(xdrop, [A[a] for a in part_ad], [B[a] for a in part_ad], tp, h_out, dt)
         v = dev_t(vo, dt, d)
+    if with_bits:  # and the keep bits a forward call left (here: the fused forward over the same rows)
+        bits = torch.zeros(n_rows, h_in // 8, dtype=torch.uint8, device=d)
+        spec = K.DropoutSpec(spec.seg_p, n_rows, seed, offset, mask_bits=bits)
+        Ad, Bd = [dev_t(a, dt, d) for a in A], [dev_t(b, dt, d) for b in B]
+        plan = K.SegmentPlan(torch.tensor(tp, dtype=torch.int32, device=d),
+                             torch.tensor(part_ad, dtype=torch.int32, device=d), n_rows)
+        K.smlm_lora_forward(torch.zeros(n_rows, h_out, dtype=TDT[dt], device=d), dev_t(x, dt, d), ptrs(Ad, d),
+                            ptrs(Bd, d), plan, r, dropout=spec)
+        assert bits.any()
     dx, dA, dB = run_backward(K, d, dt, x, A, B, g, tp, part_ad, r, spec, v)
     gx, ga, gb = oracle.add_lora_backward(g, xdrop, A, B, tp, part_ad, dt)
     gx = oracle.dropout_rows(gx, rp, seed, offset, dt)
@@ -233,3 +253,71 @@ def test_backward_dropout_gaussian(K, oracle, gpu_device, dt):
     for a in range(NA):
         close(dA[a], ga[a], atol=ATOL * max(1.0, float(np.abs(ga[a]).max())))
         close(dB[a], gb[a], atol=ATOL * max(1.0, float(np.abs(gb[a]).max())))
+
+
+def test_mixed_lora_linear_layer_with_dropout(K, oracle, gpu_device):
+    """MixedLoraLinear(fused=True) with nn.Dropout adapters: the layer hands the kernels a
+    descriptor (seed = torch's seed, offset drawn from torch's generator) instead of
+    dropping x itself; forward and gradients equal the oracle's on the dropped x."""
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.mixed_lora import MixedLoraContext, MixedLoraLinear, NamedLoraLayer
+    from loquetier_amd.segments import build_segments
+    dt, tdt = "bf16", torch.bfloat16
+    d = gpu_device
+    h_in, h_out, r, NA = 256, 384, 16, 4
+    rng = np.random.default_rng(41)
+    W = oracle.round_to(rng.standard_normal((h_out, h_in)) / 16, dt)
+    A = [oracle.round_to(rng.standard_normal((r, h_in)) / 16, dt) for _ in range(NA)]
+    B = [oracle.round_to(rng.standard_normal((h_out, r)) / 4, dt) for _ in range(NA)]
+    # train (1x24) on adapter 1, train (1x16) on adapter 3, prefill 9 on 3 (merges with the
+    # partition before it into one segment), decode on 2, 2, 1
+    req_ids, req_len = [1, 3, 3, 2, 2, 1], [24, 16, 9, 1, 1, 1]
+    T = sum(req_len)
+    xs = oracle.round_to(rng.standard_normal((T, h_in)), dt)
+    drops = [torch.nn.Identity(), torch.nn.Dropout(0.5), torch.nn.Dropout(0.9), torch.nn.Dropout(0.25)]
+    base = torch.nn.Linear(h_in, h_out, bias=False, device=d, dtype=tdt)
+    base.weight.data.copy_(dev_t(W, dt, d))
+    base.weight.requires_grad_(False)
+    adapters = [NamedLoraLayer(f"a{i}", dev_t(A[i], dt, d), dev_t(B[i], dt, d), drops[i], 1.0) for i in range(NA)]
+    ctx = MixedLoraContext()
+    layer = MixedLoraLinear(ctx, base, adapters, r, tdt, is_scaled=True, fused=True)
+    layer.set_trainable([1, 3])
+    lora_ids, lora_len, segment = build_segments(req_ids, req_len, d)
+    assert lora_ids == [1, 3, 2, 1]
+    blen = BatchLenInfo([(1, 24), (1, 16)], [9], 3, [], d)
+    ctx.update(blen=blen, lora_ids=lora_ids, lora_len=lora_len, segment=segment, train_idx=[1, 3])
+    torch.manual_seed(777)
+    offset = int(torch.randint(0, 2 ** 62, (1,)).item())  # what the layer will draw after the same seeding
+    torch.manual_seed(777)
+    xd = dev_t(xs, dt, d).requires_grad_(True)
+    out = layer(xd)
+    # rows 0..23 drop with 0.5, rows 24..39 with 0.25, the prefill rows of adapter 3 and the decode
+    # rows (adapter 2 has p = 0.9 but never trains here) are not dropped
+    rp = np.zeros(T, np.float32)
+    rp[:24], rp[24:40] = 0.5, 0.25
+    xdrop = oracle.dropout_rows(xs, rp, 777, offset, dt)
+    seg = segment.cpu().numpy()
+    base_np = oracle.round_to(xs.astype(np.float64) @ W.T.astype(np.float64), dt)
+    want, _ = oracle.lora_fused(base_np, xdrop, [A[i] for i in lora_ids], [B[i] for i in lora_ids], seg,
+                                None, 1.0, dt)
+    close(to_np(out), want, atol=2e-2)
+    plain, _ = oracle.lora_fused(base_np, xs, [A[i] for i in lora_ids], [B[i] for i in lora_ids], seg,
+                                 None, 1.0, dt)
+    assert np.abs(to_np(out)[:40] - plain[:40]).max() > 0.1   # the mask was applied
+    close(to_np(out)[40:], plain[40:], atol=2e-2)              # and only to the training rows
+    g = oracle.round_to(rng.standard_normal((T, h_out)), dt)
+    out.backward(dev_t(g, dt, d))
+    tp = [0, 24, 40]
+    gx, ga, gb = oracle.add_lora_backward(g[:40], xdrop[:40], [A[1], A[3]], [B[1], B[3]], tp, [0, 1], "fp32")
+    gx = oracle.dropout_rows(gx, rp[:40], 777, offset, "fp32")
+    for k, idx in enumerate((1, 3)):
+        pa = layer.get_parameter(f"lora-{idx}-A").grad
+        pb = layer.get_parameter(f"lora-{idx}-B").grad
+        close(to_np(pa), ga[k], rtol=2e-2, atol=2e-2 * float(np.abs(ga[k]).max()))
+        close(to_np(pb), gb[k], rtol=2e-2, atol=2e-2 * float(np.abs(gb[k]).max()))
+    want_dx = g.astype(np.float64) @ W.astype(np.float64)
+    want_dx[:40] += gx
+    close(to_np(xd.grad), want_dx, rtol=2e-2, atol=5e-2)
+    # a second call draws a new offset: another mask
+    out2 = layer(dev_t(xs, dt, d))
+    assert not torch.equal(out2[:40], out.detach()[:40]) and torch.equal(out2[40:], out.detach()[40:])
