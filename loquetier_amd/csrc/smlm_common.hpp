@@ -70,7 +70,14 @@ template <int DT>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return Num<DT>::bits(lo) | (Num<DT>::bits(hi) << 16);
 }
-// gfx950 rounds a pair of floats to bf16 (nearest even) in one instruction
+// gfx950 rounds a pair of floats to fp16 or bf16 (nearest even) in one instruction
+template <>
+__device__ __forceinline__ uint32_t pack2<SMLM_DTYPE_F16>(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+}
 template <>
 __device__ __forceinline__ uint32_t pack2<SMLM_DTYPE_BF16>(float lo, float hi) {
   typedef float f32x2_t __attribute__((ext_vector_type(2)));
