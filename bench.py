@@ -194,6 +194,9 @@ def main():
     ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
     ap.add_argument("--eager", action="store_true",
                     help="launch the steps one by one instead of replaying a graph (for counter runs)")
+    ap.add_argument("--padded-ranks", action="store_true",
+                    help="workloads with adapters below the padded rank: do not pass the true ranks "
+                         "(the kernels then read the zero padding, as the reference's do)")
     ap.add_argument("--dropout", type=float, default=0.0,
                     help="dropout probability of the training adapters (workloads with a backward): the "
                          "kernels regenerate the mask in the forward and the backward; default 0 = off")
@@ -275,6 +278,12 @@ def main():
         part_indptr = torch.tensor(w["seg"][:P + 1], dtype=torch.int32, device=dev)
         part_ad = torch.tensor([train.index(a) for a in w["ids"][:P]], dtype=torch.int32, device=dev)
         part_scale = torch.full((P,), 2.0, device=dev)
+    # adapters below the padded rank (cfg5): the kernels are told the true ranks and skip the padding
+    rank_f = rank_b = None
+    if ranks and not args.padded_ranks:
+        rank_f = torch.tensor([ranks[a % 4] for a in range(NA)], dtype=torch.int32, device=dev)
+        if P:
+            rank_b = torch.tensor([ranks[a % 4] for a in train], dtype=torch.int32, device=dev)
     drop_f = drop_b = None
     if P and args.dropout > 0:
         seg_p = torch.zeros(S, device=dev)
@@ -291,7 +300,8 @@ def main():
         pr = st["proj"]
         K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
                                   [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
-                                  v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f)
+                                  v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f,
+                                  adapter_rank=rank_f)
 
     def step(st, build_plan=True):
         if build_plan:
@@ -302,7 +312,7 @@ def main():
             for i, d in enumerate(st["proj"]):
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
                                      d["ta_tab"], d["tb_tab"], bplan, r, part_scale,
-                                     dropout=drop_b[i] if drop_b else None)
+                                     dropout=drop_b[i] if drop_b else None, adapter_rank=rank_b)
 
     # eager once on the capture stream (sizes its workspace outside any capture)
     cap_stream = torch.cuda.Stream()
@@ -445,7 +455,8 @@ def main():
                    "projections": [f"{n}:{a}->{b}" for n, a, b in w["proj"]],
                    "buffer_sets_rotated": R, "step_includes": "plan build + fused forward per projection"
                    + (" + backward" if P else ""), "graph_replay": not args.eager,
-                   "dropout": args.dropout if P else 0.0},
+                   "dropout": args.dropout if P else 0.0,
+                   "true_ranks_passed": bool(ranks and not args.padded_ranks)},
         "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
         "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),

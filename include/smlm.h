@@ -220,18 +220,36 @@ typedef struct smlm_dropout {
   void* mask_bits;
 } smlm_dropout;
 
-/* smlm_lora_fwd_multi with dropout of x (NULL descriptor: identical to it). */
-SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void* const* x,
-                                         void* const* v_out, const void* const* const* a_ptrs,
-                                         const void* const* const* b_ptrs, int n_weights,
-                                         const int* h_in, const int* h_out, const void* plan,
-                                         void* workspace, size_t workspace_bytes, int T, int S, int r,
-                                         int dtype, float beta, const float* seg_scale, int stages,
-                                         const smlm_dropout* dropout, void* stream);
+/*
+ * Options of the _ex entry points; a NULL pointer or a zeroed struct changes nothing.
+ *   dropout      : see smlm_dropout above.
+ *   adapter_rank : device int32, indexed like the weight tables (by adapter id for
+ *                  SMLM_KEY_I32 plans, by segment otherwise): the true rank of each
+ *                  adapter.  The reference keeps adapters of different ranks zero-padded
+ *                  to one rank r (MixedLoraModel._prepare_weight,
+ *                  src/loquetier_src/models/mixed_lora.py:501-521); with the true ranks
+ *                  the kernels do not read the padding (rows of A, columns of B and of v
+ *                  at or past the rank rounded up to 8) and treat it as the zeros it
+ *                  holds, so results equal the padded computation bit for bit.
+ */
+typedef struct smlm_lora_opts {
+  const smlm_dropout* dropout;
+  const int32_t* adapter_rank;
+} smlm_lora_opts;
+
+/* smlm_lora_fwd_multi with options. */
+SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* const* x,
+                                    void* const* v_out, const void* const* const* a_ptrs,
+                                    const void* const* const* b_ptrs, int n_weights,
+                                    const int* h_in, const int* h_out, const void* plan,
+                                    void* workspace, size_t workspace_bytes, int T, int S, int r,
+                                    int dtype, float beta, const float* seg_scale, int stages,
+                                    const smlm_lora_opts* opts, void* stream);
 
 /*
- * smlm_lora_bwd for a forward that ran with dropout (NULL descriptor: identical
- * to smlm_lora_bwd).  seg_p is indexed by the backward plan's partitions and the
+ * smlm_lora_bwd with options (NULL: identical to smlm_lora_bwd).  adapter_rank is
+ * indexed by the training adapters 0..NA-1.  For a forward that ran with dropout:
+ * seg_p is indexed by the backward plan's partitions and the
  * partitions of one adapter must carry the same probability; (seed, offset) are
  * the pair the forward of this projection used (offset + i for projection i of a
  * multi-projection call); rows >= n_rows.  x is the caller's x before dropout: v
@@ -239,13 +257,12 @@ SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void*
  * the gradient with respect to x before its dropout (the mask and factor applied
  * once more, as autograd's dropout backward does after add_lora.backward).
  */
-SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* db_ptrs,
-                                   const void* dy, const void* x, const void* v,
-                                   const void* const* a_ptrs, const void* const* b_ptrs,
-                                   const void* plan, void* workspace, size_t workspace_bytes,
-                                   int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
-                                   const float* part_scale, const smlm_dropout* dropout,
-                                   void* stream);
+SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_ptrs,
+                              const void* dy, const void* x, const void* v,
+                              const void* const* a_ptrs, const void* const* b_ptrs,
+                              const void* plan, void* workspace, size_t workspace_bytes,
+                              int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
+                              const float* part_scale, const smlm_lora_opts* opts, void* stream);
 
 /*
  * RMSNorm forward.  Replaces dispatch_rms_norm / rms_norm<T>

@@ -28,7 +28,12 @@ class Dropout(C.Structure):
                 ("mask_bits", C.c_void_p)]
 
 
-_pdrop = C.POINTER(Dropout)
+class LoraOpts(C.Structure):
+    """struct smlm_lora_opts of include/smlm.h."""
+    _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p)]
+
+
+_popts = C.POINTER(LoraOpts)
 
 # name -> (restype, argtypes); must list every symbol include/smlm.h declares
 SIGNATURES = {
@@ -47,13 +52,13 @@ SIGNATURES = {
     "smlm_lora_fwd_multi_workspace_size": (_i, [_i, _i, _pi, _i, _psz]),
     "smlm_lora_fwd_multi": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _i, _pi, _pi, _vp, _vp, _sz, _i, _i, _i,
                                  _i, _f, _vp, _i, _vp]),
-    "smlm_lora_fwd_multi_dropout": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _i, _pi, _pi, _vp, _vp, _sz, _i, _i,
-                                         _i, _i, _f, _vp, _i, _pdrop, _vp]),
+    "smlm_lora_fwd_multi_ex": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _i, _pi, _pi, _vp, _vp, _sz, _i, _i,
+                                         _i, _i, _f, _vp, _i, _popts, _vp]),
     "smlm_lora_bwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _i, _psz]),
     "smlm_lora_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
                            _i, _vp, _vp]),
-    "smlm_lora_bwd_dropout": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i,
-                                   _i, _i, _vp, _pdrop, _vp]),
+    "smlm_lora_bwd_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i,
+                                   _i, _i, _vp, _popts, _vp]),
     "smlm_rms_norm_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "smlm_rms_norm_bwd_workspace_size": (_i, [_i, _i, _psz]),
     "smlm_rms_norm_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),

@@ -325,12 +325,13 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
                const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false,
-               const DropArgs* drop = nullptr) {
+               const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr) {
   if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
   ShrinkArgs a{};
   if (drop) a.drop = *drop;
   a.w_kn = w_kn ? 1 : 0;
   a.plan = tile_args(pv);
+  a.plan.w_rank = w_rank;  // the output columns are the rank
   a.seg_scale = seg_scale;
   a.beta = beta;
   a.T = T;
@@ -596,22 +597,23 @@ SMLM_API int smlm_lora_fwd_multi(int n_proj, void* const* y, const void* const* 
                                  const int* h_out, const void* plan, void* workspace,
                                  size_t workspace_bytes, int T, int S, int r, int dtype, float beta,
                                  const float* seg_scale, int stages, void* stream) {
-  return smlm_lora_fwd_multi_dropout(n_proj, y, x, v_out, a_ptrs, b_ptrs, n_weights, h_in, h_out, plan,
-                                     workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale, stages,
-                                     nullptr, stream);
+  return smlm_lora_fwd_multi_ex(n_proj, y, x, v_out, a_ptrs, b_ptrs, n_weights, h_in, h_out, plan,
+                                workspace, workspace_bytes, T, S, r, dtype, beta, seg_scale, stages,
+                                nullptr, stream);
 }
 
-SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void* const* x,
-                                         void* const* v_out, const void* const* const* a_ptrs,
-                                         const void* const* const* b_ptrs, int n_weights,
-                                         const int* h_in, const int* h_out, const void* plan,
-                                         void* workspace, size_t workspace_bytes, int T, int S, int r,
-                                         int dtype, float beta, const float* seg_scale, int stages,
-                                         const smlm_dropout* dropout, void* stream) {
+SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* const* x,
+                                    void* const* v_out, const void* const* const* a_ptrs,
+                                    const void* const* const* b_ptrs, int n_weights,
+                                    const int* h_in, const int* h_out, const void* plan,
+                                    void* workspace, size_t workspace_bytes, int T, int S, int r,
+                                    int dtype, float beta, const float* seg_scale, int stages,
+                                    const smlm_lora_opts* opts, void* stream) {
   int rc = check_common(T, S, dtype);
   if (rc) return rc;
   DropArgs drop;
-  if ((rc = drop_args(dropout, &drop))) return rc;
+  if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
+  const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
     return SMLM_ERR_ARG;
   if (stages < 1 || stages > (SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND)) return SMLM_ERR_ARG;
@@ -660,13 +662,14 @@ SMLM_API int smlm_lora_fwd_multi_dropout(int n_proj, void* const* y, const void*
   }
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                    0.0f, nullptr, st, !expand_folds, false, &drop);
+                    0.0f, nullptr, st, !expand_folds, false, &drop, w_rank);
     if (rc) return rc;
   }
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;
 
   ExpandArgs ea{};
   ea.plan = tile_args(pv);
+  ea.plan.w_rank = w_rank;
   ea.seg_scale = seg_scale;
   ea.beta = beta;
   ea.T = T; ea.nt_max = pv.nt_max;
@@ -715,22 +718,21 @@ SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs,
                            const void* const* b_ptrs, const void* plan, void* workspace,
                            size_t workspace_bytes, int n_rows, int P, int NA, int h_in, int h_out,
                            int r, int dtype, const float* part_scale, void* stream) {
-  return smlm_lora_bwd_dropout(dx, da_ptrs, db_ptrs, dy, x, v, a_ptrs, b_ptrs, plan, workspace,
-                               workspace_bytes, n_rows, P, NA, h_in, h_out, r, dtype, part_scale, nullptr,
-                               stream);
+  return smlm_lora_bwd_ex(dx, da_ptrs, db_ptrs, dy, x, v, a_ptrs, b_ptrs, plan, workspace,
+                          workspace_bytes, n_rows, P, NA, h_in, h_out, r, dtype, part_scale, nullptr, stream);
 }
 
-SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* db_ptrs,
-                                   const void* dy, const void* x, const void* v,
-                                   const void* const* a_ptrs, const void* const* b_ptrs,
-                                   const void* plan, void* workspace, size_t workspace_bytes,
-                                   int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
-                                   const float* part_scale, const smlm_dropout* dropout,
-                                   void* stream) {
+SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_ptrs,
+                              const void* dy, const void* x, const void* v,
+                              const void* const* a_ptrs, const void* const* b_ptrs,
+                              const void* plan, void* workspace, size_t workspace_bytes,
+                              int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
+                              const float* part_scale, const smlm_lora_opts* opts, void* stream) {
   int rc = check_common(n_rows, P, dtype);
   if (rc) return rc;
   DropArgs drop;
-  if ((rc = drop_args(dropout, &drop))) return rc;
+  if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
+  const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   if (NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
   if ((h_in & 7) || (h_out & 7) || (r & 7)) return SMLM_ERR_ALIGN;
   if (r > 64) return SMLM_ERR_LIMIT;
@@ -788,7 +790,7 @@ SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* 
     DropArgs vdrop = drop;
     vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
-                         0.0f, nullptr, st, true, false, &vdrop)))  // v of the dropped x, as the forward made it
+                         0.0f, nullptr, st, true, false, &vdrop, w_rank)))  // v of the dropped x, as the forward made it
       return rc;
     vv = reinterpret_cast<const uint16_t*>(v16);
   }
@@ -797,12 +799,13 @@ SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* 
   const void* const* btp = in_place ? b_ptrs : bt_ptrs;
   const int b_ld = in_place ? r : h_out;
   if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
-                       0.0f, nullptr, st, true, in_place)))
+                       0.0f, nullptr, st, true, in_place, nullptr, w_rank)))
     return rc;
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
   ExpandArgs ea{};
   ea.plan = tile_args(pv);
+  ea.plan.w_rank = w_rank;
   ea.seg_scale = part_scale;
   ea.pt_a = pt_a;
   ea.pt_b = pt_b;
@@ -838,6 +841,7 @@ SMLM_API int smlm_lora_bwd_dropout(void* dx, void* const* da_ptrs, void* const* 
   wa.h_in = h_in; wa.h_out = h_out; wa.r = r;
   wa.chunks_a = ceil_div(h_in, kWgCols);
   wa.grp_seg = pv.grp_seg;
+  wa.w_rank = w_rank;
   wa.drop = drop;  // dA against the dropped x
   dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA);
   const int nbj = ceil_div(r, 16);

@@ -82,6 +82,7 @@ struct WgradArgs {
   void* const* db_ptrs;  // [NA] -> [h_out, r]
   long pitch;
   int h_in, h_out, r, chunks_a;  // chunks_a = ceil(h_in/64): blockIdx.x below it works on dA
+  const int32_t* w_rank;   // optional [NA]: true rank of each adapter (rows of dV / v past it are zero padding)
   const int32_t* grp_seg;  // DROP kernels: first segment of every group (its adapter's dropout probability)
   DropArgs drop;           // DROP kernels: dA is taken against the dropped x, regenerated while x is staged
 };
@@ -146,6 +147,11 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       break;
     }
   }
+  int rlim = a.r;
+  if (a.w_rank) {
+    const int tr = (uload(a.w_rank, ad) + 7) & ~7;
+    rlim = tr < a.r ? tr : a.r;
+  }
   constexpr int kStepTiles = kWgSlots / kTileRows;
   const int n_steps = (t_end - t_beg + kStepTiles - 1) / kStepTiles;
 
@@ -197,7 +203,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       for (int jb = 0; jb < NBJ; ++jb) {
         const int j = 16 * jb + c;
         const int tile = tile0 + 2 * ks + (g >> 1);
-        const bool ok = step < n_steps && tile < t_end && j < a.r;
+        const bool ok = step < n_steps && tile < t_end && j < rlim;
         pf[jb][ks] = ldg16_or(PT + (long)j * a.pitch + (long)tile0 * kTileRows + 32 * ks + 8 * g, ok, zeros);
       }
   };

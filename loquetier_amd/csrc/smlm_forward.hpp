@@ -37,7 +37,18 @@ struct TileArgs {
   const int32_t* tile_rseg;
   const int32_t* tile_wid;
   const int32_t* blk;        // (first tile << 3) | tile count, per tile block
+  const int32_t* w_rank;     // optional, indexed like the weight tables: true rank of each adapter
 };
+
+// Adapters of different ranks live zero-padded to one rank (the reference pads every adapter
+// of a layer to the layer's maximum, src/loquetier_src/models/mixed_lora.py:501-521).  With the
+// true ranks at hand the padding is not read: loads at or past the rank (rounded up to the
+// 8-element load width) are predicated off and read zeros, which is what the padding holds.
+__device__ __forceinline__ int rank_limit(const TileArgs& p, int wid, int d) {
+  if (!p.w_rank) return d;
+  const int r = (uload(p.w_rank, wid) + 7) & ~7;
+  return r < d ? r : d;
+}
 
 // Items [first, last) of this workgroup, visited with stride `step`.  The grid
 // size is a multiple of kNumXcd.
@@ -212,6 +223,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+    const int nlim = rank_limit(a.plan, wid, P.d_out);  // weight rows at or past it are zero padding
     DropRow dr{};
     DropArgs dp{};
     if (DROP) dp = drop_proj(a.drop, pj), dr = drop_row(dp, row, a.plan.tile_rseg, slot);
@@ -237,7 +249,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const int n = n0 + 16 * nb + c;
-          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out
+          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < nlim
 #ifdef SMLM_TUNING
                                                              && !(a.dbg & 1)
 #endif
@@ -350,6 +362,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
     const int slot = (t0 + (active ? wave : 0)) * kTileRows + c;
     const int row = active ? a.plan.tile_row[slot] : -1;
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+    const int nlim = rank_limit(a.plan, wid, P.d_out);  // weight rows at or past it are zero padding
     const int kbeg = kz * kFwdWaves * P.k_per_wave;
     const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
     const uint16_t* xrow = P.x + (long)(row < 0 ? 0 : row) * P.d_in;
@@ -375,11 +388,11 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
         if (WKN) {
           const int kl = idx / (kRowsW / 8), n8 = (idx % (kRowsW / 8)) * 8;
           st[j] = ldg16_or(W + (long)(kb + kl) * P.ldw + n0 + n8,
-                           idx < kPieces && n0 + n8 < P.d_out && kb + kl < kend, zeros);
+                           idx < kPieces && n0 + n8 < nlim && kb + kl < kend, zeros);
         } else {
           const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
           st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
-                           idx < kPieces && n0 + nl < P.d_out && kb + k8 < kend
+                           idx < kPieces && n0 + nl < nlim && kb + k8 < kend
 #ifdef SMLM_TUNING
                                && !(a.dbg & 1)
 #endif
@@ -703,6 +716,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     const int wid = uload(a.plan.tile_wid, tile);
     if (wid < 0) continue;  // past the last tile (direct mode)
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+    const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
     const int rseg = a.seg_scale ? a.plan.tile_rseg[slot] : -1;  // -1 on empty slots too
@@ -739,17 +753,17 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 #pragma unroll KSU
     for (int ks = 0; ks < nks; ++ks) {
       const int kk = 32 * ks + 8 * g;
-      const bool kin = kk < P.d_in;
+      const bool kin = kk < P.d_in, kreal = kk < klim;
       u32x4 wf[NQ][2];
 #pragma unroll
       for (int q = 0; q < NQ; ++q)
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           const int n = ncol0 + 32 * q + 4 * p + mrow;
-          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < P.d_out, zeros);
+          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kreal && n < P.d_out, zeros);
         }
       u32x4 vf;
-      const bool vok = kin && row >= 0;
+      const bool vok = kreal && row >= 0;
       if (VFOLD) {  // fold (and round) the shrink's fp32 partial sums as its fold launch would
         const float* zf = reinterpret_cast<const float*>(zeros);
         f32x4 part[kMaxVsplit][2];
@@ -805,7 +819,9 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
     const int packed = uload(a.plan.blk, tb);
     const int t0 = packed >> 3, cnt = packed & 7;
     if (cnt == 0) continue;  // past the last block (direct mode); uniform over the workgroup
-    const uint16_t* W = uload_ptr(P.w_ptrs, uload(a.plan.tile_wid, t0));
+    const int wid = uload(a.plan.tile_wid, t0);
+    const uint16_t* W = uload_ptr(P.w_ptrs, wid);
+    const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
     const bool active = wave < cnt;
     const int tslot = (t0 + (active ? wave : 0)) * kTileRows;
     const int slot = tslot + c;
@@ -836,11 +852,11 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
       if (WKN) {
         const int kl = idx / (4 * NQ), n8 = (idx % (4 * NQ)) * 8;
         stage[j] = ldg16_or(W + (long)kl * P.ldw + ncol0 + n8,
-                            idx < kPieces && ncol0 + n8 < P.d_out && kl < P.d_in, zeros);
+                            idx < kPieces && ncol0 + n8 < P.d_out && kl < klim, zeros);
       } else {
         const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
         stage[j] = ldg16_or(W + (long)(ncol0 + nl) * P.ldw + k8,
-                            idx < kPieces && ncol0 + nl < P.d_out && k8 < P.d_in
+                            idx < kPieces && ncol0 + nl < P.d_out && k8 < klim
 #ifdef SMLM_TUNING
                                 && !(a.dbg & 1)
 #endif
@@ -858,7 +874,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_block_kernel(ExpandArgs a)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int kk = 32 * ks + 8 * g;
-      vf[ks] = ldg16_or(P.v + (long)row * P.d_in + kk, kk < P.d_in && row >= 0, zeros);
+      vf[ks] = ldg16_or(P.v + (long)row * P.d_in + kk, kk < klim && row >= 0, zeros);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) L.scale[j] = (sseg[j] >= 0 && L.srow[j] >= 0) ? a.seg_scale[sseg[j]] : 1.0f;

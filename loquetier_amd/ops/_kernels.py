@@ -238,25 +238,48 @@ class DropoutSpec:
         return _lib.Dropout(self.seg_p.data_ptr(), self.rows, self.seed, self.offset, _ptr(self.mask_bits))
 
 
+def _opts(plan: SegmentPlan, dropout: Optional["DropoutSpec"], widths, adapter_rank: Optional[torch.Tensor],
+          n_weights: int):
+    """struct smlm_lora_opts for a call (None when there is nothing to say).  The returned
+    object keeps the dropout struct alive."""
+    if dropout is None and adapter_rank is None:
+        return None
+    if adapter_rank is not None:
+        _check_input(adapter_rank, "adapter_rank")
+        if adapter_rank.dtype != torch.int32 or adapter_rank.dim() != 1 or adapter_rank.size(0) < n_weights:
+            raise RuntimeError("adapter_rank must be a 1D int32 tensor with one entry per weight table entry")
+    opts = _lib.LoraOpts()
+    if dropout is not None:
+        opts._drop = dropout.struct(plan, widths)
+        opts.dropout = C.pointer(opts._drop)
+    opts.adapter_rank = _ptr(adapter_rank)
+    return opts
+
+
 def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_ptrs: torch.Tensor,
                       plan: SegmentPlan, rank: int, seg_scale: Optional[torch.Tensor] = None,
                       beta: float = 0.0, v_out: Optional[torch.Tensor] = None,
-                      dropout: Optional[DropoutSpec] = None) -> None:
+                      dropout: Optional[DropoutSpec] = None,
+                      adapter_rank: Optional[torch.Tensor] = None) -> None:
     """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call (two launches).
     a_ptrs / b_ptrs are indexed by adapter id when the plan was built from int32
     adapter ids, by segment otherwise."""
     smlm_lora_forward_multi([y], [x], [a_ptrs], [b_ptrs], plan, rank, seg_scale=seg_scale, beta=beta,
-                            v_out=None if v_out is None else [v_out], dropout=dropout)
+                            v_out=None if v_out is None else [v_out], dropout=dropout,
+                            adapter_rank=adapter_rank)
 
 
 def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
-                            v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None) -> None:
+                            v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None,
+                            adapter_rank: Optional[torch.Tensor] = None) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
     in two launches.  Lists of equal length; entries of xs may be the same tensor.
     stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
     arguments on the same stream), 3 = both.  dropout: the training rows of x are
-    dropped inside the shrink kernel; projection i uses the stream offset + i."""
+    dropped inside the shrink kernel; projection i uses the stream offset + i.
+    adapter_rank (int32, indexed like the tables): true ranks of adapters stored
+    zero-padded to `rank`; the padding is then not read."""
     n = len(ys)
     if not (1 <= n <= 8) or len(xs) != n or len(a_ptrs) != n or len(b_ptrs) != n or \
             (v_out is not None and len(v_out) != n):
@@ -287,13 +310,14 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
         _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(n, plan.T, h_in, rank, C.byref(need)),
                    "smlm_lora_fwd_multi_workspace_size")
         ws = _workspace(dev, need.value)
-        drop = None if dropout is None else C.byref(dropout.struct(plan, [x.size(1) for x in xs]))
-        rc = _lib.load().smlm_lora_fwd_multi_dropout(
+        n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
+        opts = _opts(plan, dropout, [x.size(1) for x in xs], adapter_rank, n_weights)
+        rc = _lib.load().smlm_lora_fwd_multi_ex(
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
-            min(t.size(0) for t in list(a_ptrs) + list(b_ptrs)), h_in, h_out,
+            n_weights, h_in, h_out,
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
-            _ptr(seg_scale), int(stages), drop, _stream(dev))
+            _ptr(seg_scale), int(stages), None if opts is None else C.byref(opts), _stream(dev))
     _lib.check(rc, "smlm_lora_forward")
 
 
@@ -301,7 +325,8 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                        dy: torch.Tensor, x: torch.Tensor, v: Optional[torch.Tensor],
                        a_ptrs: torch.Tensor, b_ptrs: torch.Tensor, plan: SegmentPlan, rank: int,
                        part_scale: Optional[torch.Tensor] = None,
-                       dropout: Optional[DropoutSpec] = None) -> None:
+                       dropout: Optional[DropoutSpec] = None,
+                       adapter_rank: Optional[torch.Tensor] = None) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
     forward's stream with seg_p per partition; x is the tensor before dropout."""
@@ -328,12 +353,13 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
         ws = _workspace(dev, need)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
-        drop = None if dropout is None else C.byref(dropout.struct(plan, h_in))
-        rc = _lib.load().smlm_lora_bwd_dropout(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
+        opts = _opts(plan, dropout, h_in, adapter_rank, NA)
+        rc = _lib.load().smlm_lora_bwd_ex(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
                                                dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
                                                b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
                                                ws.numel(), n_rows, plan.S, NA, h_in, h_out, rank, code,
-                                               _ptr(part_scale), drop, _stream(dev))
+                                               _ptr(part_scale), None if opts is None else C.byref(opts),
+                                               _stream(dev))
     _lib.check(rc, "smlm_lora_backward")
 
 

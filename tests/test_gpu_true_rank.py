@@ -1,0 +1,125 @@
+"""Adapters of different true ranks stored zero-padded to one rank, as the reference keeps
+them (MixedLoraModel._prepare_weight, src/loquetier_src/models/mixed_lora.py:501-521): with
+`adapter_rank` the kernels skip the padding.  The result must equal the padded computation
+bit for bit -- and must not depend on what the padding holds, which is checked by filling it
+with NaN."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TDT = {"fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def K(gpu_device):
+    from loquetier_amd import _lib
+    from loquetier_amd.ops import _kernels
+    _lib.load()
+    return _kernels
+
+
+def ptrs(ts, dev):
+    return torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=dev)
+
+
+def padded_adapters(gen, NA, ranks, r_pad, h_in, h_out, tdt, d, poison):
+    A, B = [], []
+    for a in range(NA):
+        ra = ranks[a % len(ranks)]
+        wa = torch.zeros(r_pad, h_in)
+        wb = torch.zeros(h_out, r_pad)
+        wa[:ra] = torch.randn(ra, h_in, generator=gen) / h_in ** 0.5
+        wb[:, :ra] = torch.randn(h_out, ra, generator=gen) / ra ** 0.5
+        if poison:  # whatever lies past the rank (rounded up to 8) must never be read
+            r8 = (ra + 7) // 8 * 8
+            wa[r8:] = float("nan")
+            wb[:, r8:] = float("nan")
+        A.append(wa.to(tdt).to(d))
+        B.append(wb.to(tdt).to(d))
+    return A, B
+
+
+# name, T, seg, ids, NA, h_in, h_out, r_pad, true ranks by adapter
+CASES = [
+    ("small", 90, [0, 20, 41, 41, 60, 77, 90], [0, 1, 2, 3, 1, 2], 4, 256, 192, 64, [8, 16, 32, 64]),
+    ("decode-route", 48, list(range(49)), [i % 4 for i in range(48)], 4, 512, 256, 64, [8, 16, 32, 64]),
+    ("tile-blocks", 1500, [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 512, 320, 64, [8, 16, 32, 64]),
+    ("rank32-pad", 200, [0, 64, 200], [1, 0], 2, 1024, 128, 32, [8, 24]),
+    ("odd-rank", 70, [0, 30, 70], [0, 1], 2, 256, 64, 16, [4, 12]),      # rounded up to 8 and 16 by the kernels
+    ("long-k", 70, [0, 33, 70], [1, 0], 2, 4096, 64, 64, [16, 8]),        # k split and folded
+]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_forward_with_true_ranks_equals_padded(K, gpu_device, case, dt):
+    name, T, seg, ids, NA, h_in, h_out, r_pad, ranks = case
+    d, tdt = gpu_device, TDT[dt]
+    gen = torch.Generator().manual_seed(51)
+    A, B = padded_adapters(gen, NA, ranks, r_pad, h_in, h_out, tdt, d, poison=False)
+    gen = torch.Generator().manual_seed(51)
+    An, Bn = padded_adapters(gen, NA, ranks, r_pad, h_in, h_out, tdt, d, poison=True)
+    x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    y0 = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    plan = K.SegmentPlan(torch.tensor(seg, dtype=torch.int32, device=d),
+                         torch.tensor(ids, dtype=torch.int32, device=d), T)
+    sc = torch.full((len(ids),), 2.0, device=d)
+    rk = torch.tensor([ranks[a % len(ranks)] for a in range(NA)], dtype=torch.int32, device=d)
+
+    def run(Aw, Bw, rank_arg):
+        y, v = y0.clone(), torch.full((T, r_pad), 7.0, dtype=tdt, device=d)
+        K.smlm_lora_forward(y, x, ptrs(Aw, d), ptrs(Bw, d), plan, r_pad, seg_scale=sc, beta=1.0, v_out=v,
+                            adapter_rank=rank_arg)
+        return y, v
+
+    y_pad, v_pad = run(A, B, None)
+    y_rk, v_rk = run(A, B, rk)
+    assert torch.equal(y_pad, y_rk) and torch.equal(v_pad, v_rk)
+    y_nan, v_nan = run(An, Bn, rk)          # the padding is poisoned and never read
+    assert torch.equal(y_pad, y_nan) and torch.equal(v_pad, v_nan)
+    assert not torch.isnan(y_nan).any()
+
+
+BWD_CASES = [
+    ("two-parts", [0, 35, 90], [0, 1], 2, 192, 320, 64, [8, 32]),
+    ("shared", [0, 40, 70, 100], [1, 0, 1], 2, 128, 256, 32, [16, 8]),
+    ("in-place", [0, 500, 520, 1300], [2, 0, 2], 3, 256, 192, 64, [8, 16, 64]),
+    ("many-rows", [0, 1100, 2300], [0, 1], 2, 320, 128, 64, [32, 16]),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("with_v", [False, True])
+@pytest.mark.parametrize("case", BWD_CASES, ids=[c[0] for c in BWD_CASES])
+def test_backward_with_true_ranks_equals_padded(K, gpu_device, case, dt, with_v):
+    name, tp, part_ad, NA, h_in, h_out, r_pad, ranks = case
+    d, tdt = gpu_device, TDT[dt]
+    n_rows = tp[-1]
+    gen = torch.Generator().manual_seed(52)
+    A, B = padded_adapters(gen, NA, ranks, r_pad, h_in, h_out, tdt, d, poison=False)
+    gen = torch.Generator().manual_seed(52)
+    An, Bn = padded_adapters(gen, NA, ranks, r_pad, h_in, h_out, tdt, d, poison=True)
+    x = torch.randn(n_rows, h_in, generator=gen).to(tdt).to(d)
+    g = torch.randn(n_rows, h_out, generator=gen).to(tdt).to(d)
+    plan = K.SegmentPlan(torch.tensor(tp, dtype=torch.int32, device=d),
+                         torch.tensor(part_ad, dtype=torch.int32, device=d), n_rows)
+    rk = torch.tensor([ranks[a % len(ranks)] for a in range(NA)], dtype=torch.int32, device=d)
+    v = None
+    if with_v:
+        v = torch.zeros(n_rows, r_pad, dtype=tdt, device=d)
+        K.smlm_lora_forward(torch.zeros(n_rows, h_out, dtype=tdt, device=d), x, ptrs(A, d), ptrs(B, d), plan,
+                            r_pad, v_out=v)
+
+    def run(Aw, Bw, rank_arg):
+        dA, dB = [torch.full_like(a, 5.0) for a in Aw], [torch.full_like(b, 5.0) for b in Bw]
+        dx = torch.empty(n_rows, h_in, dtype=tdt, device=d)
+        K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), g, x, v, ptrs(Aw, d), ptrs(Bw, d), plan, r_pad,
+                             adapter_rank=rank_arg)
+        return [dx] + dA + dB
+
+    pad, rkd, nan = run(A, B, None), run(A, B, rk), run(An, Bn, rk)
+    for a, b, c in zip(pad, rkd, nan):
+        assert torch.equal(a, b)
+        assert torch.equal(a, c)     # gradients of the padding are zeros either way, and no NaN leaks in

@@ -177,13 +177,14 @@ def test_dropout_entry_points_validate_like_their_plain_forms(lib):
     p = (ctypes.addressof(buf) + 255) // 256 * 256  # fake "device" address; never dereferenced
     big = 1 << 30
     VP, CI = ctypes.c_void_p * 1, ctypes.c_int * 1
-    drop = lib.Dropout(p, -1, 1, 2)
-    fwd = lambda dr, **k: L.smlm_lora_fwd_multi_dropout(
+    drop = lib.Dropout(p, -1, 1, 2, None)
+    opts = lib.LoraOpts(ctypes.pointer(drop), None)
+    fwd = lambda dr, **k: L.smlm_lora_fwd_multi_ex(
         1, VP(p), VP(p), None, VP(p), VP(p), 2, CI(64), CI(64), p, p, big, k.get("T", 16), 2, k.get("r", 16),
         k.get("dtype", 0), 0.0, None, 3, dr, None)
-    assert fwd(ctypes.byref(drop)) == -1            # negative row count
+    assert fwd(ctypes.byref(opts)) == -1            # negative row count
     assert fwd(None, r=12) == -3 and fwd(None, dtype=2) == -2 and fwd(None, T=0) == 0
-    bwd = lambda dr, **k: L.smlm_lora_bwd_dropout(p, p, p, p, p, None, p, p, p, p, k.get("ws", big), 16, 1, 1, 64,
+    bwd = lambda dr, **k: L.smlm_lora_bwd_ex(p, p, p, p, p, None, p, p, p, p, k.get("ws", big), 16, 1, 1, 64,
                                                   64, k.get("r", 8), 1, None, dr, None)
-    assert bwd(ctypes.byref(drop)) == -1
+    assert bwd(ctypes.byref(opts)) == -1
     assert bwd(None, r=128) == -6 and bwd(None, ws=16) == -4
