@@ -81,7 +81,7 @@ def close(got, want, rtol=RTOL, atol=ATOL):
 # ---------------------------------------------------------------- forward ---
 FWD_CASES = [
     # name, T, seg, ids, NA, h_in, h_out, r
-    ("survey-small", 13, [0, 5, 5, 9, 13], [2, 0, 2, 1], 3, 64, 96, 8),
+    ("tiny-with-empty-segment", 13, [0, 5, 5, 9, 13], [2, 0, 2, 1], 3, 64, 96, 8),
     ("one-segment", 16, [0, 16], [0], 1, 128, 128, 16),
     ("ragged", 77, [0, 1, 18, 18, 50, 51, 52, 77], [3, 1, 2, 1, 0, 3, 1], 4, 256, 320, 32),
     ("uncovered-rows", 40, [3, 10, 31], [1, 0], 2, 64, 64, 16),
