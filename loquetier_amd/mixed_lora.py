@@ -68,8 +68,15 @@ class MixedLoraContext:
         return self._train_idx
 
     def seg_adapter(self, device: torch.device) -> torch.Tensor:
+        """Adapter id of every segment as a device tensor.  `lora_ids` may already be one (int32,
+        e.g. from segments.build_segments_device, whose arrays keep the request count as capacity
+        and describe empty segments past the real ones): it is then used as it is, and the fused
+        path never brings the ids to the host."""
         if self._seg_adapter is None or self._seg_adapter.device != device:
-            self._seg_adapter = torch.tensor(self._lora_ids, dtype=torch.int32, device=device)
+            if isinstance(self._lora_ids, torch.Tensor):
+                self._seg_adapter = self._lora_ids.to(device=device, dtype=torch.int32)
+            else:
+                self._seg_adapter = torch.tensor(self._lora_ids, dtype=torch.int32, device=device)
         return self._seg_adapter
 
     def plan(self, device: torch.device, T: int) -> kernel.SegmentPlan:

@@ -103,3 +103,35 @@ def test_forward_from_device_built_segments(K, oracle, gpu_device, dt):
     assert torch.equal(y_host, y_dev)
     assert torch.equal(y_dev[int(o_seg[-1]):], y0[int(o_seg[-1]):])  # rows past the last request untouched
     assert not torch.equal(y_dev[:33], y0[:33])
+
+
+def test_layer_from_device_built_segments(K, oracle, gpu_device):
+    """MixedLoraLinear (fused) driven by the device segment builder's padded arrays gives the
+    bits it gives with the host loop's segments."""
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.mixed_lora import MixedLoraContext, MixedLoraLinear, NamedLoraLayer
+    from loquetier_amd.segments import build_segments, build_segments_device
+    d, tdt = gpu_device, torch.float16
+    h_in, h_out, r, NA = 128, 192, 16, 3
+    g = torch.Generator().manual_seed(13)
+    req_ids, req_len = [1, 1, 0, 2, 2, 2, 1], [9, 1, 30, 1, 1, 1, 1]
+    T = sum(req_len)
+    base = torch.nn.Linear(h_in, h_out, bias=False, device=d, dtype=tdt)
+    adapters = [NamedLoraLayer(f"a{i}", (torch.randn(r, h_in, generator=g) / 8).to(tdt).to(d),
+                               (torch.randn(h_out, r, generator=g) / 4).to(tdt).to(d), torch.nn.Identity(), 2.0)
+                for i in range(NA)]
+    x = torch.randn(T, h_in, generator=g).to(tdt).to(d)
+    blen = BatchLenInfo([], [40], 4, [], d)
+    outs = []
+    for on_device in (False, True):
+        ctx = MixedLoraContext()
+        layer = MixedLoraLinear(ctx, base, adapters, r, tdt, is_scaled=False, fused=True)
+        if on_device:
+            ids, lens, segment, _ = build_segments_device(torch.tensor(req_ids, dtype=torch.int32, device=d),
+                                                          torch.tensor(req_len, dtype=torch.int32, device=d))
+        else:
+            ids, lens, segment = build_segments(req_ids, req_len, d)
+        ctx.update(blen=blen, lora_ids=ids, lora_len=lens, segment=segment, train_idx=[])
+        with torch.no_grad():
+            outs.append(layer(x))
+    assert torch.equal(outs[0], outs[1])
