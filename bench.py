@@ -308,7 +308,9 @@ def main():
             st["plan"] = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
         fwd(st)
         if P:
-            bplan = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
+            if build_plan or "bplan" not in st:
+                st["bplan"] = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
+            bplan = st["bplan"]
             for i, d in enumerate(st["proj"]):
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
                                      d["ta_tab"], d["tb_tab"], bplan, r, part_scale,

@@ -542,7 +542,7 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(ReduceArgs a) {
     f32x4 sum = part[0];
 #pragma unroll
     for (int z = 1; z < kMaxKsplit; ++z) sum += part[z];
-    if (row >= first && row < first + count) store4<DT>(P.out + (long)row * a.d_out + n, sum, 1.0f, a.beta);
+    if (in_batch && row >= first && row < first + count) store4<DT>(P.out + (long)row * a.d_out + n, sum, 1.0f, a.beta);
   }
 }
 
