@@ -1,11 +1,13 @@
-// Dropout of the training rows of x, regenerated wherever x (or dX) passes through registers.
+// Dropout of the training rows of x, applied where x (or dX) passes through registers.
 //
 // The reference drops x before the LoRA term, one nn.Dropout(p) per adapter
 // (src/loquetier_src/models/mixed_lora.py:185-192): a dropped copy of every training partition
 // plus a torch.cat of the whole batch, and autograd's mask multiply on the way back.  Here no
-// dropped copy and no mask are stored: the mask is a pure function of (seed, offset, row,
-// column), so the shrink kernels apply it to the x fragments they load, the weight-gradient
-// kernel to the x fragments it loads, and the dX kernel to the values it stores.
+// dropped copy of x exists.  The mask is a pure function of (seed, offset, row, column): the
+// shrink kernels generate it for the x fragments they load and leave its keep bits behind (one
+// byte per eight columns, 1/16 of x's bytes); the backward applies those bits -- or the same bits
+// made again by drop_bits_kernel -- to the x rows the weight-gradient kernel stages and to the
+// dX values the expand kernel stores.
 //
 // Mask: the eight 16-bit pieces of philox4x32_10(counter = (row, col / 8, offset), key = seed)
 // decide elements col .. col + 7 of a row; an element is dropped when its piece is below
