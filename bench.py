@@ -34,9 +34,11 @@ METRIC = "SMLM tokens/s + HBM GB/s (% of 8 TB/s), Llama-2-7B shapes, 1 GPU"
 
 def workload(name: str):
     """Shapes and routing of BASELINE.json's configs 2-5 (seeds = config number)."""
-    if name == "cfg2":
-        ids = np.random.default_rng(2).integers(0, 32, 256).tolist()
-        return dict(name="cfg2: 256 single-token segments over 32 adapters, r=16, q/k/v/o 4096->4096, "
+    if name in ("cfg2", "cfg2mod"):
+        # adapters drawn uniformly (the headline workload) or dealt round-robin, i % 32 (the variant)
+        ids = np.random.default_rng(2).integers(0, 32, 256).tolist() if name == "cfg2" else [i % 32 for i in range(256)]
+        return dict(name=f"{name}: 256 single-token segments over 32 adapters"
+                         f"{'' if name == 'cfg2' else ' dealt round-robin'}, r=16, q/k/v/o 4096->4096, "
                          "fp16, forward", dtype="fp16", r=16, NA=32, seg=list(range(257)), ids=ids,
                     proj=[("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096)],
                     n_train_parts=0)
@@ -234,7 +236,7 @@ def main():
     R = 1 if args.no_rotate else max(2, math.ceil(640e6 / footprint))
     R = min(R, 16)
 
-    gen = torch.Generator(device="cpu").manual_seed(int(args.config[-1]))
+    gen = torch.Generator(device="cpu").manual_seed(int("".join(ch for ch in args.config if ch.isdigit())))
     seg_t = torch.tensor(w["seg"], dtype=torch.int32, device=dev)
     ids_t = torch.tensor(w["ids"], dtype=torch.int32, device=dev)
     scale_t = torch.full((S,), 2.0, device=dev)
