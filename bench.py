@@ -420,6 +420,22 @@ def main():
                     frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
                     us_per_launch=round(expand_us, 3), algorithmic_bytes=expand_bytes)
 
+    # ---- what a plain streaming kernel reaches at this launch size: torch's in-place add_ (one
+    # read and one write per byte, nothing else) over tensors sized so that one launch moves the
+    # expand launch's algorithmic bytes, rotating over enough of them to stay out of the
+    # Infinity Cache.  HBM-bound kernels on this part climb with the bytes per launch, so this, not
+    # the 8 TB/s peak, is what the launch above can be held against.
+    n_el = max(1, expand_bytes // 4)                      # fp16 elements: 2 bytes read + 2 written each
+    n_ref = 1 if args.no_rotate else max(2, min(64, math.ceil(640e6 / (2 * n_el))))
+    ref_bufs = [torch.zeros(n_el, dtype=torch.float16, device=dev) for _ in range(n_ref)]
+    ref_reps = max(2, 48 // n_ref)
+    g_ref = capture(lambda: [b.add_(1.0) for _ in range(ref_reps) for b in ref_bufs])
+    timed([(g_ref, 2)])
+    ref_us = timed([(g_ref, 10)]) * 1e3 / (10 * ref_reps * n_ref)
+    streaming = dict(kernel="torch in-place add_ (elementwise read-modify-write)", bytes=int(n_el * 4),
+                     us_per_launch=round(ref_us, 3), gbps=round(n_el * 4 / (ref_us * 1e-6) / 1e9, 1))
+    del ref_bufs, g_ref
+
     # ---- CPU baseline: per-segment torch matmuls on the host cores (bounded sample)
     cpu = None
     if not args.no_cpu_baseline:
@@ -466,6 +482,7 @@ def main():
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
         "ms_per_step_plan_reused": round(reuse_ms, 5),
         "roofline": roofline,
+        "streaming_reference": streaming,
         "kernels": {"shrink_us": round(shrink_us, 3), "shrink_bytes": shrink_bytes,
                     "shrink_gbps": round(shrink_bytes / (shrink_us * 1e-6) / 1e9, 1),
                     "expand_us": round(expand_us, 3), "expand_bytes": expand_bytes,
