@@ -72,6 +72,27 @@ def workload(name: str):
     raise SystemExit(f"unknown config {name}")
 
 
+def adapter_sorted(w):
+    """The same requests handed over grouped by adapter (training part and serving part each on
+    its own): what a scheduler that batches by adapter would pass.  Neighbouring segments of one
+    adapter merge, as the run-length segment builder merges them, so the rows of an adapter are
+    one contiguous run instead of many short ones."""
+    seg, ids, P = w["seg"], w["ids"], w["n_train_parts"]
+    lens = [seg[i + 1] - seg[i] for i in range(len(ids))]
+
+    def group(lo, hi):
+        out = {}
+        for i in range(lo, hi):
+            out[ids[i]] = out.get(ids[i], 0) + lens[i]
+        return sorted(out.items())
+    train, serve = group(0, P), group(P, len(ids))
+    new_ids = [a for a, _ in train + serve]
+    new_seg = np.concatenate([[0], np.cumsum([n for _, n in train + serve])]).tolist()
+    w = dict(w, seg=new_seg, ids=new_ids, n_train_parts=len(train))
+    w["name"] += ", requests grouped by adapter"
+    return w
+
+
 def algorithmic_bytes(w, h_in, h_out, accumulate=True):
     """Forward bytes of one projection: x and y once (y read too when accumulating),
     A and B of each distinct active adapter once, v written and read once at I/O width."""
@@ -196,6 +217,8 @@ def main():
     ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
     ap.add_argument("--eager", action="store_true",
                     help="launch the steps one by one instead of replaying a graph (for counter runs)")
+    ap.add_argument("--sorted", action="store_true",
+                    help="hand the same requests over grouped by adapter (a scheduler that batches by adapter)")
     ap.add_argument("--padded-ranks", action="store_true",
                     help="workloads with adapters below the padded rank: do not pass the true ranks "
                          "(the kernels then read the zero padding, as the reference's do)")
@@ -223,6 +246,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = workload(args.config)
+    if args.sorted:
+        w = adapter_sorted(w)
     tdt = torch.float16 if w["dtype"] == "fp16" else torch.bfloat16
     T, S, r, NA = w["seg"][-1], len(w["ids"]), w["r"], w["NA"]
     P = w["n_train_parts"]
