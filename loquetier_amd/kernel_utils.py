@@ -101,7 +101,8 @@ def _unique_adapters(weight_list: Sequence[torch.Tensor]):
 
 def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Optional[torch.Tensor],
                   weight_list: Sequence[torch.Tensor], tp: Sequence[int], lora_rank: int,
-                  part_scale: Optional[torch.Tensor] = None, dropout=None):
+                  part_scale: Optional[torch.Tensor] = None, dropout=None,
+                  adapter_rank: Optional[torch.Tensor] = None):
     """Shared backward: returns (grad_x [T, h_in], [grad per weight occurrence]).
 
     Partitions that train the same adapter contribute to one summed gradient,
@@ -130,7 +131,7 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
         kernel.smlm_lora_backward(
             grad_x, _ptr_table(da, dev), _ptr_table(db, dev), g, x_train, v_train,
             _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
-            plan, lora_rank, part_scale, dropout=dropout)
+            plan, lora_rank, part_scale, dropout=dropout, adapter_rank=adapter_rank)
     else:
         for t in da + db:
             t.zero_()

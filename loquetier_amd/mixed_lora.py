@@ -92,6 +92,9 @@ class NamedLoraLayer:
     wb: torch.Tensor  # [h_out, rank]
     dropout: Union[nn.Dropout, nn.Identity]
     scaling: Optional[float] = None
+    # Rank of the adapter before prepare_weight padded it to the layer's rank (None: the layer's
+    # rank).  Not in the reference's record; with it the fused kernels skip the zero padding.
+    true_rank: Optional[int] = None
 
 
 def prepare_weight(weight: torch.Tensor, rank: int, dtype: torch.dtype, device, rank_dim: int = 0,
@@ -114,8 +117,11 @@ class fused_add_lora(Function):
     """result <- result + scale_seg * (x A_seg^T) B_seg^T, in place, one call.
 
     Arguments: (result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-    train_len, train_partition, dropout, *weights); the tables hold one address
-    per adapter and the plan is keyed by adapter id.  `dropout` (a
+    train_len, train_partition, dropout, adapter_rank, *weights); the tables hold
+    one address per adapter and the plan is keyed by adapter id.  `adapter_rank`
+    (None, or a pair of int32 device tensors: the true rank of every adapter, and
+    of the training adapters in order of first appearance among the partitions)
+    tells the kernels which adapters are stored zero-padded.  `dropout` (a
     kernel.DropoutSpec or None) drops the training rows of x inside the kernels,
     in place of the reference's nn.Dropout calls and torch.cat before the op
     (src/loquetier_src/models/mixed_lora.py:185-192); x is the tensor before
@@ -125,8 +131,9 @@ class fused_add_lora(Function):
 
     @staticmethod
     def forward(ctx: FunctionCtx, result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-                train_len, train_partition, dropout, *weights):
+                train_len, train_partition, dropout, adapter_rank, *weights):
         need_v = len(weights) > 0 and train_len > 0
+        adapter_rank, train_rank = adapter_rank if adapter_rank is not None else (None, None)
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
         if dropout is not None and need_v and dropout.mask_bits is None:
             # the backward reads the forward's keep bits (1/16 of x's bytes) instead of making them again
@@ -134,7 +141,7 @@ class fused_add_lora(Function):
                                device=x.device)
             dropout = kernel.DropoutSpec(dropout.seg_p, dropout.rows, dropout.seed, dropout.offset, bits)
         kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
-                                 beta=1.0, v_out=v, dropout=dropout)
+                                 beta=1.0, v_out=v, dropout=dropout, adapter_rank=adapter_rank)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
@@ -144,6 +151,7 @@ class fused_add_lora(Function):
         # kept as a device gather so nothing is read back to the host
         ctx.part_scale = None
         ctx.part_drop = None
+        ctx.train_rank = train_rank if need_v else None
         if need_v and (seg_scale is not None or dropout is not None):
             starts = torch.tensor([int(t) for t in train_partition][: ctx.n_parts],
                                   dtype=torch.int32, device=x.device)
@@ -159,12 +167,13 @@ class fused_add_lora(Function):
 
     @staticmethod
     def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
-        n_fixed = 10
+        n_fixed = 11
         if not ctx.has_v:
             return (grad_output, None) + (None,) * (n_fixed - 2) + (None,) * (2 * ctx.n_parts)
         x, v, *weight_list = ctx.saved_tensors
         grad_x, grads = lora_backward(grad_output, x, v, weight_list, ctx.tp, ctx.rank,
-                                      part_scale=ctx.part_scale, dropout=ctx.part_drop)
+                                      part_scale=ctx.part_scale, dropout=ctx.part_drop,
+                                      adapter_rank=ctx.train_rank)
         return (grad_output, grad_x) + (None,) * (n_fixed - 2) + tuple(grads)
 
 
@@ -195,6 +204,23 @@ class MixedLoraLinear(nn.Module):
         if not self.is_scaled:
             self.scaling = torch.tensor([a.scaling for a in adapters], dtype=self.dtype,
                                         device=self.device)
+        ranks = [rank if a.true_rank is None else min(int(a.true_rank), rank) for a in adapters]
+        self.adapter_rank = (torch.tensor(ranks, dtype=torch.int32, device=self.device)
+                             if any(q < rank for q in ranks) else None)
+        self._train_rank_key, self._train_rank = None, None
+
+    def _rank_args(self, train_idx):
+        """(ranks of all adapters, ranks of the training adapters in order of first appearance),
+        or None when every adapter has the layer's rank."""
+        if self.adapter_rank is None:
+            return None
+        order = list(dict.fromkeys(int(i) for i in train_idx))
+        key = tuple(order)
+        if self._train_rank_key != key:
+            self._train_rank_key = key
+            self._train_rank = (self.adapter_rank[torch.tensor(order, dtype=torch.long, device=self.device)]
+                                if order else None)
+        return self.adapter_rank, self._train_rank
 
     def add_adapter(self, adapter: NamedLoraLayer):
         """New adapter must have the rank of the existing ones."""
@@ -248,7 +274,7 @@ class MixedLoraLinear(nn.Module):
                 x = x.contiguous()
             result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale,
                                           ctx.plan(self.device, x.size(0)), self.rank, blen.tlen,
-                                          blen.train_partition, drop_spec, *weights)
+                                          blen.train_partition, drop_spec, self._rank_args(train_idx), *weights)
             return result.to(torch_result_dtype)
 
         segment = ctx.segment.to(self.device)

@@ -123,3 +123,40 @@ def test_backward_with_true_ranks_equals_padded(K, gpu_device, case, dt, with_v)
     for a, b, c in zip(pad, rkd, nan):
         assert torch.equal(a, b)
         assert torch.equal(a, c)     # gradients of the padding are zeros either way, and no NaN leaks in
+
+
+def test_layer_with_true_ranks_equals_padded_layer(K, gpu_device):
+    """MixedLoraLinear: adapters that carry their true rank give the bits (output and
+    gradients) of the same adapters treated as full-rank."""
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.mixed_lora import MixedLoraContext, MixedLoraLinear, NamedLoraLayer, prepare_weight
+    from loquetier_amd.segments import build_segments
+    d, tdt = gpu_device, torch.bfloat16
+    h_in, h_out, r_pad, ranks = 256, 320, 32, [8, 32, 16]
+    gen = torch.Generator().manual_seed(71)
+    raw = [((torch.randn(q, h_in, generator=gen) / 16), (torch.randn(h_out, q, generator=gen) / 4)) for q in ranks]
+    req_ids, req_len = [2, 0, 0, 1, 1, 2], [40, 24, 5, 1, 1, 1]   # train on adapters 2 and 0
+    T = sum(req_len)
+    x0 = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    g = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    base = torch.nn.Linear(h_in, h_out, bias=False, device=d, dtype=tdt)
+    base.weight.requires_grad_(False)
+    results = []
+    for with_rank in (False, True):
+        adapters = [NamedLoraLayer(f"a{i}", prepare_weight(wa, r_pad, tdt, d, rank_dim=0),
+                                   prepare_weight(wb, r_pad, tdt, d, rank_dim=1), torch.nn.Identity(), 2.0,
+                                   true_rank=ranks[i] if with_rank else None) for i, (wa, wb) in enumerate(raw)]
+        ctx = MixedLoraContext()
+        layer = MixedLoraLinear(ctx, base, adapters, r_pad, tdt, is_scaled=False, fused=True)
+        assert (layer.adapter_rank is not None) == with_rank
+        layer.set_trainable([2, 0])
+        lora_ids, lora_len, segment = build_segments(req_ids, req_len, d)
+        ctx.update(blen=BatchLenInfo([(1, 40), (1, 24)], [5], 3, [], d), lora_ids=lora_ids, lora_len=lora_len,
+                   segment=segment, train_idx=[2, 0])
+        x = x0.clone().requires_grad_(True)
+        out = layer(x)
+        out.backward(g)
+        results.append([out.detach(), x.grad] + [layer.get_parameter(f"lora-{i}-{m}").grad for i in (2, 0) for m in "AB"])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    assert not (results[1][2][16:] != 0).any()  # dA of adapter 2 (true rank 16): the padding rows get zero gradient
