@@ -86,6 +86,8 @@ FWD_CASES = [
     ("ragged", 77, [0, 1, 18, 18, 50, 51, 52, 77], [3, 1, 2, 1, 0, 3, 1], 4, 256, 320, 32),
     ("uncovered-rows", 40, [3, 10, 31], [1, 0], 2, 64, 64, 16),
     ("uncovered-rows-long-k", 75, [5, 22, 22, 60], [1, 0, 1], 2, 4096, 64, 16),  # k split and folded
+    # more segments than the one-workgroup plan takes, first rows uncovered, k split and folded row by row
+    ("many-segments-offset", 1600, list(range(7, 1508)), [i % 5 for i in range(1500)], 5, 2048, 64, 16),
     ("rank64", 45, [0, 20, 45], [0, 1], 2, 512, 256, 64),
     ("rank24", 33, [0, 33], [0], 1, 96, 136, 24),
     ("decode", 64, list(range(65)), [i % 5 for i in range(64)], 5, 512, 512, 16),
