@@ -187,7 +187,8 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const bool ok = row[u] >= 0 && col_ok;
-      val[u] = ldg16_or(Q + (long)row[u] * h + n0 + lcol, ok, zeros);
+      // x and dY are read here for the last time in the backward: non-temporal
+      val[u] = ldg16_or_nt(Q + (long)row[u] * h + n0 + lcol, ok, zeros);
       if (DROP) {  // rows at or past drop.rows keep everything: their byte is never applied
         const bool dropped = ok && row[u] < a.drop.rows;
         keep[u] = *(const SMLM_GLOBAL uint8_t*)(dropped ? a.drop.bits + (long)row[u] * a.drop.bits_pitch + ((n0 + lcol) >> 3)

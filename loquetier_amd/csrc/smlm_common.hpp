@@ -115,6 +115,17 @@ __device__ __forceinline__ u32x4 ldg16_if(const uint16_t* p, bool ok, const uint
 __device__ __forceinline__ u32x4 ldg16_or(const uint16_t* p, bool ok, const uint16_t* zeros) {
   return ldg16(ok ? p : zeros);
 }
+// the same for data that is read once (activations, gradients): marked non-temporal so that it
+// does not push the weights, which other workgroups read again, out of the caches
+__device__ __forceinline__ u32x4 ldg16_or_nt(const uint16_t* p, bool ok, const uint16_t* zeros) {
+  return __builtin_nontemporal_load((const SMLM_GLOBAL u32x4*)(ok ? p : zeros));
+}
+__device__ __forceinline__ u32x4 ldg16_nt(const uint16_t* p) {
+  return __builtin_nontemporal_load((const SMLM_GLOBAL u32x4*)(p));
+}
+__device__ __forceinline__ void stg16_nt(uint16_t* p, u32x4 v) {
+  __builtin_nontemporal_store(v, (SMLM_GLOBAL u32x4*)(p));
+}
 constexpr int kHdrZeros = 12;  // header words 12..15 are always zero
 
 // Transposing LDS read of gfx950: within each 16 lanes, lane i names a "row" of
