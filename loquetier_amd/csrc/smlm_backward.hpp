@@ -337,7 +337,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int j = 16 * jb + orow + 8 * i, n = n0 + ocol;
-        if (j < a.r && n < h) stg16(out + (long)j * h + n, o[i]);
+        if (j < a.r && n < h) stg16_nt(out + (long)j * h + n, o[i]);
       }
     }
   } else {
@@ -355,7 +355,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int n = n0 + 16 * nb + orow + 8 * i;
-        if (ocol < a.r && n < h) stg16(out + (long)n * a.r + ocol, o[i]);
+        if (ocol < a.r && n < h) stg16_nt(out + (long)n * a.r + ocol, o[i]);
       }
     }
   }
