@@ -66,9 +66,10 @@ struct RmsFwdArgs {
 // reduced, scaled and stored.  (Measured: one turn per workgroup is fastest for
 // the forward, four for the backward, whose per-workgroup dw partials cost
 // traffic of their own.)
-// STREAM (batches of 1024 rows and more): the output is written non-temporally, as it is far
-// larger than the caches; x is always read so (its next reader is the backward, much later).
-template <int DT, int WPR, bool ONE_TURN, bool STREAM>
+// x is read and the output written non-temporally: both are touched once per launch (the next
+// reader of x is the backward, much later; a reader of the output that follows at once still
+// finds it in the caches when it fits them).
+template <int DT, int WPR, bool ONE_TURN>
 __global__ __launch_bounds__(256) void rms_fwd_kernel(RmsFwdArgs a) {
   __shared__ float part[2][4];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(256) void rms_fwd_kernel(RmsFwdArgs a) {
       u32x4 o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) o[e] = pack2<DT>(f[2 * e] * rms * g[2 * e], f[2 * e + 1] * rms * g[2 * e + 1]);
-      if (STREAM) stg16_nt(orow + col, o); else stg16(orow + col, o);
+      stg16_nt(orow + col, o);
     }
 #pragma unroll
     for (int i = 0; i < kRmsChunks; ++i) xv[i] = xn[i];
@@ -157,7 +158,7 @@ struct RmsBwdArgs {
 // A workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ... (WPR == 4: one
 // row at a time, a quarter of the columns per wave; WPR == 1: four rows at a
 // time, one per wave) and keeps its share of dw in registers.
-template <int DT, int WPR, bool STREAM>
+template <int DT, int WPR>
 __global__ __launch_bounds__(256) void rms_bwd_kernel(RmsBwdArgs a) {
   __shared__ float part[2][4];
   __shared__ __attribute__((aligned(16))) float dwred[WPR == 1 ? 4 * (kRmsWaveCols / 2) : 4];
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(256) void rms_bwd_kernel(RmsBwdArgs a) {
       for (int e = 0; e < 4; ++e)
         o[e] = pack2<DT>((gf[2 * e] * wf[2 * e] - xf[2 * e] * coef) * rms,
                          (gf[2 * e + 1] * wf[2 * e + 1] - xf[2 * e + 1] * coef) * rms);
-      if (STREAM) stg16_nt(a.dx + off + col, o); else stg16(a.dx + off + col, o);
+      stg16_nt(a.dx + off + col, o);
 #pragma unroll
       for (int e = 0; e < 8; ++e) dw[i][e] += xf[e] * rms * gf[e];
     }

@@ -429,23 +429,6 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
   return L;
 }
 
-template <bool STREAM>
-int launch_rms_fwd(bool f16, bool one_wave, bool one_turn, dim3 grid, hipStream_t st, const RmsFwdArgs& a) {
-  const dim3 bl(256);
-  if (one_wave) {
-    if (one_turn)
-      return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, true, STREAM>, grid, bl, st, a)
-                 : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 1, true, STREAM>, grid, bl, st, a);
-    return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, false, STREAM>, grid, bl, st, a)
-               : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 1, false, STREAM>, grid, bl, st, a);
-  }
-  if (one_turn)
-    return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 4, true, STREAM>, grid, bl, st, a)
-               : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 4, true, STREAM>, grid, bl, st, a);
-  return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 4, false, STREAM>, grid, bl, st, a)
-             : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 4, false, STREAM>, grid, bl, st, a);
-}
-
 }  // namespace
 
 extern "C" {
@@ -905,9 +888,19 @@ SMLM_API int smlm_rms_norm_fwd(void* out, float* rms, const void* x, const void*
   const dim3 grid((unsigned)nb);
   const int rows_per_step = cols <= kRmsWaveCols ? 4 : 1;
   const bool one_turn = (long)nb * rows_per_step >= rows;  // every workgroup sees one row group
-  const bool stream_out = tiles_per_wave(rows) > 1;  // 1024 rows and more
-  return stream_out ? launch_rms_fwd<true>(f16, cols <= kRmsWaveCols, one_turn, grid, st, a)
-                    : launch_rms_fwd<false>(f16, cols <= kRmsWaveCols, one_turn, grid, st, a);
+  const dim3 bl(256);
+  if (cols <= kRmsWaveCols) {
+    if (one_turn)
+      return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, true>, grid, bl, st, a)
+                 : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 1, true>, grid, bl, st, a);
+    return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, false>, grid, bl, st, a)
+               : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 1, false>, grid, bl, st, a);
+  }
+  if (one_turn)
+    return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 4, true>, grid, bl, st, a)
+               : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 4, true>, grid, bl, st, a);
+  return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 4, false>, grid, bl, st, a)
+             : launch(rms_fwd_kernel<SMLM_DTYPE_BF16, 4, false>, grid, bl, st, a);
 }
 
 SMLM_API int smlm_rms_norm_bwd_workspace_size(int rows, int cols, size_t* bytes) {
@@ -936,23 +929,13 @@ SMLM_API int smlm_rms_norm_bwd(void* dx, void* dw, const void* g, const void* x,
                      reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const uint16_t*>(x),
                      reinterpret_cast<const uint16_t*>(w), rms, rows, cols};
   const dim3 grid((unsigned)nb);
-  const bool stream_out = tiles_per_wave(rows) > 1;  // 1024 rows and more
   const dim3 bl(256);
-  if (cols <= kRmsWaveCols) {
-    if (stream_out)
-      rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 1, true>, grid, bl, st, a)
-               : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 1, true>, grid, bl, st, a);
-    else
-      rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 1, false>, grid, bl, st, a)
-               : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 1, false>, grid, bl, st, a);
-  } else {
-    if (stream_out)
-      rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 4, true>, grid, bl, st, a)
-               : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 4, true>, grid, bl, st, a);
-    else
-      rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 4, false>, grid, bl, st, a)
-               : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 4, false>, grid, bl, st, a);
-  }
+  if (cols <= kRmsWaveCols)
+    rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 1>, grid, bl, st, a)
+             : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 1>, grid, bl, st, a);
+  else
+    rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 4>, grid, bl, st, a)
+             : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 4>, grid, bl, st, a);
   if (rc) return rc;
   const RmsFoldArgs fa{reinterpret_cast<uint16_t*>(dw), reinterpret_cast<const float*>(workspace), nb, cols};
   const dim3 fgrid((unsigned)ceil_div(cols, 64));

@@ -634,25 +634,24 @@ __device__ __forceinline__ void load_keep_bits(LineLane& L, const DropArgs& d, i
     }
 }
 
-// STREAM (the tile-block kernels, batches of 1024 rows and more): y is read and written once
-// and is far larger than the caches, so its accesses are marked non-temporal; left to the
-// default policy its lines crowd out the weights and leave dirty lines behind that the next
-// launch has to wait for (measured: 4-12 % of a step).  Small batches keep the default policy:
-// their y is likely to be in a cache already and to be read again from there.
-template <int NQ, bool STREAM = false>
+// y is read and written once per launch, so its accesses are marked non-temporal: left to the
+// default policy its lines crowd the weights out of L2 and leave dirty lines behind that the next
+// launch has to wait for (measured: 4-12 % of a step on the large batches, 3.5 % on the decode
+// step).  A reader that follows at once is not slowed down as long as the data fits the caches
+// (measured with a writer / reader pair: 2 and 8 MB read back equally fast, 32 MB 9 % slower).
+template <int NQ>
 __device__ __forceinline__ void load_y_lines(u32x4 (&yold)[NQ / 2][2], const LineLane& L, int ncol0, int d_out,
                                              bool read_y, const uint16_t* zeros) {
 #pragma unroll
   for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int h = 0; h < NQ / 2; ++h)
-      yold[h][j] = STREAM ? ldg16_or_nt(L.yrow[j] + 64 * h, read_y && L.srow[j] >= 0 && ncol0 + 64 * h + L.ocol < d_out, zeros)
-                          : ldg16_or(L.yrow[j] + 64 * h, read_y && L.srow[j] >= 0 && ncol0 + 64 * h + L.ocol < d_out, zeros);
+      yold[h][j] = ldg16_or_nt(L.yrow[j] + 64 * h, read_y && L.srow[j] >= 0 && ncol0 + 64 * h + L.ocol < d_out, zeros);
 }
 
 // DROP: what is stored is the gradient with respect to x before its dropout: the value as it
 // would be stored otherwise, times the row's factor where the element was kept, zero elsewhere
-template <int DT, int NQ, bool DROP = false, bool STREAM = false>
+template <int DT, int NQ, bool DROP = false>
 __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ][2], const u32x4 (&yold)[NQ / 2][2],
                                               const LineLane& L, int c, int g, int ncol0, int d_out, float beta) {
 #pragma unroll
@@ -692,7 +691,7 @@ __device__ __forceinline__ void store_y_lines(float* stg, const f32x4 (&acc)[NQ]
         o[3] = pack2<DT>(sc * hi4[j][2], sc * hi4[j][3]);
       }
       if (DROP) o = drop8_bits<DT>(o, L.drop[j], L.keep[h][j]);
-      if (STREAM) stg16_nt(L.yrow[j] + 64 * h, o); else stg16(L.yrow[j] + 64 * h, o);
+      stg16_nt(L.yrow[j] + 64 * h, o);
     }
   }
 }
@@ -877,7 +876,7 @@ void expand_block_kernel(ExpandArgs a) {
     if (a.dbg & 2) read_y = false;
 #endif
     u32x4 yold[NQ / 2][2];
-    load_y_lines<NQ, true>(yold, L, ncol0, P.d_out, read_y, zeros);
+    load_y_lines<NQ>(yold, L, ncol0, P.d_out, read_y, zeros);
     if (DROP) load_keep_bits<NQ>(L, a.drop, ncol0, P.d_out, zeros);
     u32x4 vf[KS];
 #pragma unroll
@@ -929,7 +928,7 @@ void expand_block_kernel(ExpandArgs a) {
           acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
         }
 
-    store_y_lines<DT, NQ, DROP, true>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
+    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
   }
 }
 
