@@ -243,7 +243,9 @@ int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipS
     if (block)  // launch_expand admits only [k][n] weights here
       return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, true, true>, grid, bl, st, a)
                      : launch(expand_block_kernel<DT, 4, 2, DIRECT, true, true>, grid, bl, st, a);
-    if (KS == 0) return SMLM_ERR_LIMIT;  // the backward stops at rank 64
+    if (KS == 0)  // ranks above 64: the general loop over k
+      return nq == 4 ? launch(expand_wave_kernel<DT, 4, 0, false, DIRECT, false, true>, grid, bl, st, a)
+                     : launch(expand_wave_kernel<DT, 2, 0, false, DIRECT, false, true>, grid, bl, st, a);
     if (nq == 4)
       return KS == 1 ? launch(expand_wave_kernel<DT, 4, 1, false, DIRECT, false, true>, grid, bl, st, a)
                      : launch(expand_wave_kernel<DT, 4, 2, false, DIRECT, false, true>, grid, bl, st, a);
@@ -735,7 +737,6 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   if (NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
   if ((h_in & 7) || (h_out & 7) || (r & 7)) return SMLM_ERR_ALIGN;
-  if (r > 64) return SMLM_ERR_LIMIT;
   if (NA == 0 || n_rows == 0 || P == 0) return SMLM_ERR_ARG;
   if (!da_ptrs || !db_ptrs || !a_ptrs || !b_ptrs || !workspace) return SMLM_ERR_ARG;
   if (!dx || !dy || !x || !plan) return SMLM_ERR_ARG;
@@ -763,7 +764,8 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The
   // tile-block kernels (1024 rows and more) read the weights as they lie in memory; smaller
   // batches work on transposed copies At [h_in, r], Bt [r, h_out] made here.
-  const bool in_place = tiles_per_wave(n_rows) > 1;
+  // (ranks above 64 take the one-tile expand kernel's general k loop, which reads [n][k] weights)
+  const bool in_place = tiles_per_wave(n_rows) > 1 && r <= 64;
   if (!in_place) {
     TransposeArgs ta{};
     ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
@@ -843,8 +845,9 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   wa.grp_seg = pv.grp_seg;
   wa.w_rank = w_rank;
   wa.drop = drop;  // dA against the dropped x
-  dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA);
-  const int nbj = ceil_div(r, 16);
+  // ranks above 64 are covered 64 at a time along the grid's z axis
+  dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA, ceil_div(r, 64));
+  const int nbj = r > 64 ? 4 : ceil_div(r, 16);
   // four waves splitting the rows of an adapter pay off when adapters have many rows each
   const bool split = n_rows / NA >= 256;
   return dtype == SMLM_DTYPE_F16 ? launch_wgrad<SMLM_DTYPE_F16>(nbj, split, grid, st, wa)

@@ -99,8 +99,8 @@ __device__ __forceinline__ int wg_lds_row(int s) {
   return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1);
 }
 
-// grid: (ceil(h_in/64) + ceil(h_out/64), NA), block 64*NW.  A workgroup owns 64
-// columns of one adapter's dA or dB and walks all of that adapter's tiles, 64
+// grid: (ceil(h_in/64) + ceil(h_out/64), NA, ceil(r/64)), block 64*NW.  A workgroup owns 64
+// columns (and up to 64 ranks) of one adapter's dA or dB and walks all of that adapter's tiles, 64
 // gathered rows (four tiles, two MFMA k steps) per wave and loop step.  With
 // NW = 4 (adapters with many rows each) the waves take steps round-robin and
 // their accumulators are summed through LDS in wave order; with NW = 1 (many
@@ -122,6 +122,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
 
   const int ad = blockIdx.y;
+  const int j0 = 64 * blockIdx.z;  // first rank of this workgroup (ranks above 64: 64 per z)
   constexpr bool is_a = IS_A;
   const int n0 = (is_a ? blockIdx.x : blockIdx.x - a.chunks_a) * kWgCols;
   const int h = is_a ? a.h_in : a.h_out;
@@ -202,7 +203,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
       for (int jb = 0; jb < NBJ; ++jb) {
-        const int j = 16 * jb + c;
+        const int j = j0 + 16 * jb + c;
         const int tile = tile0 + 2 * ks + (g >> 1);
         const bool ok = step < n_steps && tile < t_end && j < rlim;
         pf[jb][ks] = ldg16_or(PT + (long)j * a.pitch + (long)tile0 * kTileRows + 32 * ks + 8 * g, ok, zeros);
@@ -336,7 +337,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       wave_sync();
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const int j = 16 * jb + orow + 8 * i, n = n0 + ocol;
+        const int j = j0 + 16 * jb + orow + 8 * i, n = n0 + ocol;
         if (j < a.r && n < h) stg16_nt(out + (long)j * h + n, o[i]);
       }
     }
@@ -355,7 +356,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int n = n0 + 16 * nb + orow + 8 * i;
-        if (ocol < a.r && n < h) stg16_nt(out + (long)n * a.r + ocol, o[i]);
+        if (j0 + ocol < a.r && n < h) stg16_nt(out + (long)n * a.r + j0 + ocol, o[i]);
       }
     }
   }

@@ -155,6 +155,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   __shared__ int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];  // by sorted position
   __shared__ int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
   __shared__ int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
+  __shared__ int32_t gpos[kPlanSmallSegs + 1];  // group -> sorted position of its first segment, [NG] = S
   __shared__ uint64_t wave_tot[17];
   __shared__ int bad_key, wide_key;
   const PlanView pv = args.pv;
@@ -217,8 +218,6 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
   __syncthreads();
 
   // gathered-row position of every sorted segment, group heads
-  int32_t* gpos = len0;  // group -> sorted position of its first segment (len0 is read before the scan
-                         // below, gpos written after it)
   constexpr uint64_t kRowMask = 0xffffffffull;  // rows in the low half, group heads in the high half
   int seg = 0, len = 0;
   uint64_t gk = 0;

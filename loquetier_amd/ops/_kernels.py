@@ -17,22 +17,55 @@ from .. import _lib
 
 _DTYPE_CODE = {torch.float16: _lib.SMLM_DTYPE_F16, torch.bfloat16: _lib.SMLM_DTYPE_BF16}
 
-# (device index, stream handle) -> uint8 workspace tensor, grown on demand.
-# Calls on one stream are ordered, so they can share one buffer.
-_WORKSPACES: Dict[Tuple[int, int], torch.Tensor] = {}
+class Workspace:
+    """Scratch memory for the kernels (k-split partial sums, the rounded v, transposed weights).
+
+    The C ABI allocates nothing: every call is handed a buffer at least as large as its
+    `*_workspace_size` query says.  A Workspace owns such a buffer.  It only ever grows, a
+    buffer that was handed out is never freed while the Workspace lives (a captured HIP graph
+    keeps the raw address of the buffer it was captured with), and it refuses to grow while
+    its stream is being captured: size it first, with `reserve` or with one eager pass.
+    Calls that share a Workspace must be ordered on one stream."""
+
+    def __init__(self, device: torch.device, nbytes: int = 0):
+        self.device = torch.device(device)
+        self._buf: Optional[torch.Tensor] = None
+        self._retired = []
+        if nbytes:
+            self.reserve(nbytes)
+
+    def reserve(self, nbytes: int) -> torch.Tensor:
+        if self._buf is None or self._buf.numel() < nbytes:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(
+                    f"the workspace must grow to {nbytes} bytes during a graph capture: reserve it "
+                    "before capturing (Workspace.reserve, or one eager pass of the same calls)")
+            if self._buf is not None:
+                self._retired.append(self._buf)
+            self._buf = torch.empty(max(nbytes, 1 << 20) * 3 // 2, dtype=torch.uint8, device=self.device)
+        return self._buf
+
+
+# default workspaces, one per (device index, stream handle): calls on one stream are ordered,
+# so they can share one buffer.  Callers that want to own the memory pass `workspace=`.
+_WORKSPACES: Dict[Tuple[int, int], Workspace] = {}
 
 
 def _stream(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def _workspace(dev: torch.device, nbytes: int, tag: int = 0) -> torch.Tensor:
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream(dev), tag)
-    buf = _WORKSPACES.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20) * 3 // 2, dtype=torch.uint8, device=dev)
-        _WORKSPACES[key] = buf
-    return buf
+def _workspace(dev: torch.device, nbytes: int, own: Optional[Workspace] = None) -> torch.Tensor:
+    if own is not None:
+        buf = own.reserve(nbytes)
+        if buf.device != dev:
+            raise RuntimeError(f"workspace lives on {buf.device}, the tensors on {dev}")
+        return buf
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream(dev))
+    ws = _WORKSPACES.get(key)
+    if ws is None:
+        ws = _WORKSPACES[key] = Workspace(dev)
+    return ws.reserve(nbytes)
 
 
 def _check_input(t: torch.Tensor, name: str) -> None:
@@ -172,7 +205,7 @@ def _check_scale(seg_scale: Optional[torch.Tensor], plan: SegmentPlan) -> None:
 
 def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, plan: SegmentPlan,
                       is_row_major: bool = False, seg_scale: Optional[torch.Tensor] = None,
-                      beta: float = 0.0) -> None:
+                      beta: float = 0.0, workspace: Optional[Workspace] = None) -> None:
     """Grouped GEMM over a prebuilt plan: y[seg] = beta*y[seg] + scale*x[seg] @ W_seg.
     w_ptrs is indexed by adapter id when the plan was built from int32 adapter ids,
     by segment otherwise."""
@@ -190,7 +223,7 @@ def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, pl
     dev = x.device
     with torch.cuda.device(dev):
         need = _lib.size_query("smlm_gemm_planned_workspace_size", T, d_in, d_out)
-        ws = _workspace(dev, need)
+        ws = _workspace(dev, need, workspace)
         rc = _lib.load().smlm_gemm_planned(y.data_ptr(), x.data_ptr(), w_ptrs.data_ptr(), w_ptrs.size(0),
                                            plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), T, plan.S,
                                            d_in, d_out, w_ld, int(bool(is_row_major)), code,
@@ -260,19 +293,21 @@ def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_
                       plan: SegmentPlan, rank: int, seg_scale: Optional[torch.Tensor] = None,
                       beta: float = 0.0, v_out: Optional[torch.Tensor] = None,
                       dropout: Optional[DropoutSpec] = None,
-                      adapter_rank: Optional[torch.Tensor] = None) -> None:
+                      adapter_rank: Optional[torch.Tensor] = None,
+                      workspace: Optional[Workspace] = None) -> None:
     """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call (two launches).
     a_ptrs / b_ptrs are indexed by adapter id when the plan was built from int32
     adapter ids, by segment otherwise."""
     smlm_lora_forward_multi([y], [x], [a_ptrs], [b_ptrs], plan, rank, seg_scale=seg_scale, beta=beta,
                             v_out=None if v_out is None else [v_out], dropout=dropout,
-                            adapter_rank=adapter_rank)
+                            adapter_rank=adapter_rank, workspace=workspace)
 
 
 def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
                             v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None,
-                            adapter_rank: Optional[torch.Tensor] = None) -> None:
+                            adapter_rank: Optional[torch.Tensor] = None,
+                            workspace: Optional[Workspace] = None) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
     in two launches.  Lists of equal length; entries of xs may be the same tensor.
     stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
@@ -309,7 +344,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
         need = C.c_size_t(0)
         _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(n, plan.T, h_in, rank, C.byref(need)),
                    "smlm_lora_fwd_multi_workspace_size")
-        ws = _workspace(dev, need.value)
+        ws = _workspace(dev, need.value, workspace)
         n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
         opts = _opts(plan, dropout, [x.size(1) for x in xs], adapter_rank, n_weights)
         rc = _lib.load().smlm_lora_fwd_multi_ex(
@@ -326,7 +361,8 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                        a_ptrs: torch.Tensor, b_ptrs: torch.Tensor, plan: SegmentPlan, rank: int,
                        part_scale: Optional[torch.Tensor] = None,
                        dropout: Optional[DropoutSpec] = None,
-                       adapter_rank: Optional[torch.Tensor] = None) -> None:
+                       adapter_rank: Optional[torch.Tensor] = None,
+                       workspace: Optional[Workspace] = None) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
     forward's stream with seg_p per partition; x is the tensor before dropout."""
@@ -350,7 +386,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     dev = dy.device
     with torch.cuda.device(dev):
         need = _lib.size_query("smlm_lora_bwd_workspace_size", n_rows, plan.S, NA, h_in, h_out, rank)
-        ws = _workspace(dev, need)
+        ws = _workspace(dev, need, workspace)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
         opts = _opts(plan, dropout, h_in, adapter_rank, NA)

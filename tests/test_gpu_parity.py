@@ -90,6 +90,8 @@ FWD_CASES = [
     ("many-segments-offset", 1600, list(range(7, 1508)), [i % 5 for i in range(1500)], 5, 2048, 64, 16),
     ("rank64", 45, [0, 20, 45], [0, 1], 2, 512, 256, 64),
     ("rank24", 33, [0, 33], [0], 1, 96, 136, 24),
+    ("rank128", 45, [0, 20, 45], [0, 1], 2, 512, 256, 128),   # ranks above 64: general k loop in the expand
+    ("rank72", 33, [0, 33], [0], 1, 96, 136, 72),
     ("decode", 64, list(range(65)), [i % 5 for i in range(64)], 5, 512, 512, 16),
 ]
 
@@ -406,6 +408,32 @@ def test_forward_dyadic_bit_exact_decode_route(K, oracle, gpu_device, shape, dt)
     _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
 
 
+@pytest.mark.parametrize("keyed", [True, False], ids=["distinct-ids", "no-key"])
+def test_one_launch_plan_with_as_many_groups_as_segments(K, oracle, gpu_device, keyed):
+    """The largest batch the one-workgroup plan takes (1024 segments) with every segment a group
+    of its own -- 1024 distinct adapters, or a plan without keys: the group tables then have
+    their last entry at index 1024."""
+    T = S = 1024
+    NA, h_in, h_out, r, dt = 1024, 64, 64, 8, "bf16"
+    rng = np.random.default_rng(53)
+    seg = list(range(T + 1))
+    ids = rng.permutation(NA).tolist()
+    x, A, B = make_case(oracle, 205, T, seg, ids, NA, h_in, h_out, r, dt, dy=True)
+    base = dyadic(rng, (T, h_out), 16, 8)
+    d = gpu_device
+    if keyed:
+        _fwd_exact(K, oracle, d, dt, x, A, B, seg, ids, r, base)
+        return
+    xd, yd = dev_t(x, dt, d), dev_t(base, dt, d)
+    Ad, Bd = [dev_t(a, dt, d) for a in A], [dev_t(b, dt, d) for b in B]
+    plan = K.SegmentPlan(torch.tensor(seg, dtype=torch.int32, device=d), None, T)
+    assert plan.header()[1] == S
+    K.smlm_lora_forward(yd, xd, ptrs([Ad[i] for i in ids], d), ptrs([Bd[i] for i in ids], d), plan, r,
+                        seg_scale=torch.full((S,), 2.0, device=d), beta=1.0)
+    yo, _ = oracle.lora_fused(base, x, [A[i] for i in ids], [B[i] for i in ids], seg, [2.0] * S, 1.0, dt)
+    assert np.array_equal(to_np(yd), yo)
+
+
 def test_forward_beyond_the_direct_grid(K, oracle, gpu_device):
     """More than 65535 tile units: the launches fall back to the persistent walk over the
     plan's exact tile count (and the plan to its two-launch route).  Bit-exact on dyadic
@@ -503,6 +531,11 @@ BWD_CASES = [
     ("empty-part", [0, 17, 17, 50], [0, 1, 2], 3, 0, 256, 128, 32),
     ("rank64", [0, 33, 90], [0, 1], 2, 4, 192, 320, 64),
     ("long", [0, 300, 700], [1, 0], 2, 20, 512, 384, 16),
+    # ranks above 64 (PEFT ranks 128 / 256 are ordinary): general k loop in the dX expand, the weight
+    # gradient covers the rank 64 at a time
+    ("rank128", [0, 33, 90], [0, 1], 2, 4, 192, 320, 128),
+    ("rank72", [0, 50], [0], 1, 0, 128, 136, 72),
+    ("rank256-blocks", [0, 600, 1100], [1, 0], 2, 3, 256, 192, 256),
     # few rows and long k: the sixteen-wave shrink (k split in two, folded by a launch) for v and dV
     ("long-k", [0, 30, 75], [1, 0], 2, 4, 4096, 2048, 16),
 ]

@@ -79,8 +79,8 @@ def test_argument_validation_codes(lib):
     assert L.smlm_plan_build(p, big, p, p, 9, 16, 2, None) == -1      # unknown key kind
     assert L.smlm_plan_build(p, 64, p, None, 0, 16, 2, None) == -4
     assert L.smlm_lora_fwd(p, p, None, p, p, 2, p, p, big, 16, 2, 64, 64, 12, 0, 0.0, None, None) == -3
-    assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, big, 16, 1, 1, 64, 64, 128, 1,
-                           None, None) == -6        # rank above the backward kernels' limit
+    assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, big, 16, 1, 1, 64, 64, 12, 1,
+                           None, None) == -3        # rank not a multiple of 8
     assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, 16, 16, 1, 1, 64, 64, 8, 1,
                            None, None) == -4
 
@@ -187,4 +187,4 @@ def test_dropout_entry_points_validate_like_their_plain_forms(lib):
     bwd = lambda dr, **k: L.smlm_lora_bwd_ex(p, p, p, p, p, None, p, p, p, p, k.get("ws", big), 16, 1, 1, 64,
                                                   64, k.get("r", 8), 1, None, dr, None)
     assert bwd(ctypes.byref(opts)) == -1
-    assert bwd(None, r=128) == -6 and bwd(None, ws=16) == -4
+    assert bwd(None, r=12) == -3 and bwd(None, ws=16) == -4
