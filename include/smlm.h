@@ -57,6 +57,7 @@ extern "C" {
 #define SMLM_ERR_WORKSPACE (-4) /* workspace or plan buffer too small         */
 #define SMLM_ERR_LAUNCH (-5)    /* the HIP runtime refused a kernel launch    */
 #define SMLM_ERR_LIMIT (-6)     /* size beyond what the kernels index         */
+#define SMLM_ERR_SCRATCH (-7)   /* the call needs more scratch than the library's static array holds */
 
 SMLM_API int smlm_abi_version(void);
 SMLM_API const char* smlm_strerror(int code);
@@ -106,6 +107,30 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
                        void* workspace, size_t workspace_bytes, int T, int S, int d_in, int d_out,
                        int w_ld, int w_row_major, int dtype, float beta, const float* seg_scale,
                        void* stream);
+
+/*
+ * smlm_gemm for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference (whose caller allocates `tmp` with torch,
+ * src/loquetier_src/kernel_utils.py:113-116).  Same arguments as smlm_gemm
+ * without the workspace, same kernels, same results bit for bit; the plan and the
+ * k-split partial sums live in an array of SMLM_STATIC_SCRATCH_BYTES that is part
+ * of the library's code object (every GPU the library runs on holds its own copy
+ * until the process ends).  Returns SMLM_ERR_SCRATCH when
+ * smlm_gemm_workspace_size(T, S, d_in, d_out) exceeds that size.  Calls neither
+ * hipMalloc nor hipFree nor any allocating routine.  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress) and should be made outside a
+ * capture.  All calls on one GPU share the array: calls that overlap on one GPU
+ * (different streams, or different host threads without ordering) race; calls on
+ * one stream are safe.  Nothing in the array has to start at zero -- every word a
+ * kernel reads is written earlier in the same call -- so the contents left by an
+ * earlier call never matter.
+ */
+#define SMLM_STATIC_SCRATCH_BYTES (8u << 20)
+SMLM_API int smlm_gemm_static(void* y, const void* x, const void* const* w_ptrs,
+                              const int32_t* seg_indptr, int T, int S, int d_in, int d_out, int w_ld,
+                              int w_row_major, int dtype, float beta, const float* seg_scale,
+                              void* stream);
 
 /*
  * The same grouped GEMM with a plan built beforehand by smlm_plan_build for

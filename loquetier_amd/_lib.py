@@ -15,6 +15,8 @@ LIB_PATH = os.environ.get("SMLM_HIP_LIBRARY") or os.path.join(_PKG_DIR, "lib", "
 SMLM_DTYPE_F16, SMLM_DTYPE_BF16 = 0, 1
 SMLM_KEY_NONE, SMLM_KEY_I32, SMLM_KEY_PTR = 0, 1, 2
 SMLM_ERR_DTYPE = -2
+SMLM_ERR_SCRATCH = -7
+SMLM_STATIC_SCRATCH_BYTES = 8 << 20
 SMLM_STAGE_SHRINK, SMLM_STAGE_EXPAND = 1, 2
 
 _vp, _i, _sz, _f = C.c_void_p, C.c_int, C.c_size_t, C.c_float
@@ -44,6 +46,7 @@ SIGNATURES = {
     "smlm_plan_build": (_i, [_vp, _sz, _vp, _vp, _i, _i, _i, _vp]),
     "smlm_gemm_workspace_size": (_i, [_i, _i, _i, _i, _psz]),
     "smlm_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
+    "smlm_gemm_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_gemm_planned_workspace_size": (_i, [_i, _i, _i, _psz]),
     "smlm_gemm_planned": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_lora_fwd_workspace_size": (_i, [_i, _i, _i, _i, _i, _psz]),

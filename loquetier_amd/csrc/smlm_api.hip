@@ -3,6 +3,7 @@
 // synchronisation, no state.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdlib>
 
 #include "rms_norm.hpp"
@@ -14,6 +15,9 @@
 #include "smlm_plan.hpp"
 
 using namespace smlm;
+
+// Scratch of smlm_gemm_static (file scope; see static_scratch below).
+static __device__ __align__(256) unsigned char scratch[SMLM_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -431,6 +435,24 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
   return L;
 }
 
+// Scratch of smlm_gemm_static: part of the code object, so every device the library is loaded
+// on has its own copy at its own address.  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels and copies get the looked-up device address.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> scratch_addr[kMaxDevices];
+
+// device address of `scratch` on the current device (looked up once per device), or null
+void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = scratch_addr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+    scratch_addr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+  }
+  return p;
+}
+
 }  // namespace
 
 extern "C" {
@@ -446,6 +468,7 @@ SMLM_API const char* smlm_strerror(int code) {
     case SMLM_ERR_WORKSPACE: return "workspace too small";
     case SMLM_ERR_LAUNCH: return "kernel launch failed";
     case SMLM_ERR_LIMIT: return "size beyond the supported range";
+    case SMLM_ERR_SCRATCH: return "the call needs more scratch than the library's static array holds";
     default: return "unknown error";
   }
 }
@@ -565,6 +588,23 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
   return smlm_gemm_planned(y, x, w_ptrs, S, workspace, reinterpret_cast<char*>(workspace) + plan_bytes,
                            workspace_bytes - plan_bytes, T, S, d_in, d_out, w_ld, w_row_major, dtype,
                            beta, seg_scale, stream);
+}
+
+SMLM_API int smlm_gemm_static(void* y, const void* x, const void* const* w_ptrs,
+                              const int32_t* seg_indptr, int T, int S, int d_in, int d_out, int w_ld,
+                              int w_row_major, int dtype, float beta, const float* seg_scale,
+                              void* stream) {
+  int rc = check_common(T, S, dtype);
+  if (rc) return rc;
+  if (d_in <= 0 || d_out <= 0) return SMLM_ERR_ARG;
+  size_t need = 0;
+  if ((rc = smlm_gemm_workspace_size(T, S, d_in, d_out, &need))) return rc;
+  if (need > SMLM_STATIC_SCRATCH_BYTES) return SMLM_ERR_SCRATCH;
+  // an empty batch launches nothing (smlm_gemm validates the rest and returns): no device needed
+  void* ws = (T == 0 || S == 0) ? nullptr : static_scratch();
+  if (!ws && T != 0 && S != 0) return SMLM_ERR_LAUNCH;
+  return smlm_gemm(y, x, w_ptrs, seg_indptr, ws, SMLM_STATIC_SCRATCH_BYTES, T, S, d_in, d_out, w_ld,
+                   w_row_major, dtype, beta, seg_scale, stream);
 }
 
 SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_in, int r,

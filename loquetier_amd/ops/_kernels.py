@@ -139,6 +139,37 @@ def smlm_forward_cutlass(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, 
     _lib.check(rc, "smlm_forward_cutlass")
 
 
+def smlm_forward_cutlass_static(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, s: torch.Tensor,
+                                is_row_major: bool, beta: float = 0.0,
+                                seg_scale: Optional[torch.Tensor] = None) -> None:
+    """smlm_forward_cutlass without `tmp` and without any allocation (smlm_gemm_static): the
+    scratch is an array inside the library, SMLM_STATIC_SCRATCH_BYTES per GPU, shared by all
+    calls on that GPU -- keep them on one stream.  Raises when the batch needs more."""
+    for t, n in ((y, "y"), (x, "x"), (w_ptr, "w_ptr"), (s, "s")):
+        _check_input(t, n)
+    _check_dim(2, y, "y")
+    _check_dim(2, x, "x")
+    _check_dim(1, w_ptr, "w_ptr")
+    _check_dim(1, s, "s")
+    num_problems = s.size(0) - 1
+    if w_ptr.dtype != torch.int64 or s.dtype != torch.int32:
+        raise RuntimeError("w_ptr must be int64 and s must be int32")
+    if w_ptr.size(0) != num_problems or y.size(0) != x.size(0) or y.dtype != x.dtype:
+        raise RuntimeError("inconsistent shapes: w_ptr [S], s [S+1], x [T,d_in], y [T,d_out]")
+    if seg_scale is not None and (seg_scale.dtype != torch.float32 or seg_scale.numel() != num_problems
+                                  or not seg_scale.is_cuda):
+        raise RuntimeError("seg_scale must be a device float32 tensor with one entry per segment")
+    code = _dtype_code(x)
+    d_in, d_out = x.size(1), y.size(1)
+    dev = x.device
+    with torch.cuda.device(dev):
+        rc = _lib.load().smlm_gemm_static(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s.data_ptr(),
+                                          x.size(0), num_problems, d_in, d_out,
+                                          d_out if is_row_major else d_in, int(bool(is_row_major)), code,
+                                          float(beta), _ptr(seg_scale), _stream(dev))
+    _lib.check(rc, "smlm_forward_cutlass_static")
+
+
 class SegmentPlan:
     """Tile plan of one flat batch: built once from (segment, adapter ids) and
     shared by every LoRA linear of the step (the reference rebuilds its

@@ -81,6 +81,15 @@ def test_argument_validation_codes(lib):
     assert L.smlm_lora_fwd(p, p, None, p, p, 2, p, p, big, 16, 2, 64, 64, 12, 0, 0.0, None, None) == -3
     assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, big, 16, 1, 1, 64, 64, 12, 1,
                            None, None) == -3        # rank not a multiple of 8
+    # the entry point that carries its own scratch refuses batches beyond it before touching the device
+    st = lambda T, d_in, d_out, dtype=0: L.smlm_gemm_static(p, p, p, p, T, 2, d_in, d_out, d_in, 0, dtype,
+                                                             0.0, None, None)
+    assert st(1 << 20, 4096, 64) == lib.SMLM_ERR_SCRATCH
+    assert "scratch" in lib.strerror(lib.SMLM_ERR_SCRATCH)
+    assert st(16, 64, 8, dtype=2) == -2
+    assert st(0, 64, 8) == 0                         # empty batch
+    need = lib.size_query("smlm_gemm_workspace_size", 4224, 132, 4096, 16)
+    assert need <= lib.SMLM_STATIC_SCRATCH_BYTES     # the fine-tune + serve batch fits
     assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, 16, 16, 1, 1, 64, 64, 8, 1,
                            None, None) == -4
 
