@@ -89,6 +89,9 @@ ORACLE_API void oracle_round(float* a, size_t n, int dtype) {
 static void dense(float* c, int ldc, const float* a, long a_rs, long a_cs,
                   const float* b, long b_rs, long b_cs, int m, int n, int k,
                   int dtype, int acc64) {
+  /* output elements are independent: large products are shared out over the host cores; each
+   * element is still one dot product in index order, so the result does not depend on it */
+#pragma omp parallel for collapse(2) schedule(static) if ((double)m * n * k > 4e6)
   for (int i = 0; i < m; ++i)
     for (int j = 0; j < n; ++j) {
       float r;

@@ -768,15 +768,18 @@ def _config5_segments():
     return np.concatenate([[0], np.cumsum(lens)]).tolist()
 
 
-def test_full_config5_heterogeneous_ranks(K, oracle, gpu_device):
+@pytest.mark.parametrize("shape", [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096)],
+                         ids=["q", "k_v", "gate_up", "down"])
+def test_full_config5_heterogeneous_ranks(K, oracle, gpu_device, shape):
     """64 adapters, true ranks cycling {8,16,32,64} zero-padded to 64 (the
     reference's realisation, mixed_lora.py:501-521), geometric segment lengths
-    totalling 8192 rows, k/v projection 4096 -> 1024, bf16; backward on the
-    first quarter of the segments."""
+    totalling 8192 rows, every projection shape of the Llama-3-8B layer (q 4096 -> 4096, k/v 4096 ->
+    1024, gate/up 4096 -> 14336, down 14336 -> 4096), bf16; backward on the first quarter of the
+    segments.  Bit for bit on exactly representable inputs."""
     seg = _config5_segments()
     S = len(seg) - 1
     ids = [i % 64 for i in range(S)]
-    h_in, h_out = 4096, 1024
+    h_in, h_out = shape
     rng = np.random.default_rng(55)
     x = dyadic(rng, (8192, h_in), 16, 8)
     base = dyadic(rng, (8192, h_out), 16, 8)
@@ -791,6 +794,42 @@ def test_full_config5_heterogeneous_ranks(K, oracle, gpu_device):
     n_rows = seg[P]
     g = dyadic(rng, (n_rows, h_out), 16, 8)
     _bwd_exact(K, oracle, gpu_device, "bf16", x[:n_rows], A, B, g, seg[:P + 1], ids[:P], 64)
+
+
+def test_full_config2_four_projections_one_call(K, oracle, gpu_device):
+    """The decode step as the benchmark issues it: q, k, v, o (4096 -> 4096, own weights and
+    inputs each) of 256 single-token segments over 32 adapters in ONE smlm_lora_forward_multi
+    call, every projection against the oracle: bit for bit on exactly representable inputs, and
+    to rtol 1e-2 / atol 1e-3 of the fp32 host reference on Gaussian ones (fp16)."""
+    d, dt = gpu_device, "fp16"
+    T, r, NA, n_proj = 256, 16, 32, 4
+    ids = np.random.default_rng(2).integers(0, NA, T).tolist()
+    seg = list(range(T + 1))
+    s = torch.tensor(seg, dtype=torch.int32, device=d)
+    plan = K.SegmentPlan(s, torch.tensor(ids, dtype=torch.int32, device=d), T)
+    sc = torch.full((T,), 2.0, device=d)
+    for exact in (True, False):
+        cases = []
+        for p in range(n_proj):
+            if exact:
+                x, A, B, base = _dyadic_full(20 + p, T, 4096, 4096, r, NA)
+            else:
+                x, A, B = make_case(oracle, 30 + p, T, seg, ids, NA, 4096, 4096, r, dt)
+                base = oracle.round_to(np.random.default_rng(40 + p).standard_normal((T, 4096)), dt)
+            cases.append((x, A, B, base))
+        dev = [dict(x=dev_t(x, dt, d), A=[dev_t(a, dt, d) for a in A], B=[dev_t(b, dt, d) for b in B],
+                    y=dev_t(base, dt, d)) for x, A, B, base in cases]
+        vs = [torch.zeros(T, r, dtype=TDT[dt], device=d) for _ in range(n_proj)]
+        K.smlm_lora_forward_multi([c["y"] for c in dev], [c["x"] for c in dev], [ptrs(c["A"], d) for c in dev],
+                                  [ptrs(c["B"], d) for c in dev], plan, r, seg_scale=sc, beta=1.0, v_out=vs)
+        for p, (x, A, B, base) in enumerate(cases):
+            yo, vo = oracle.lora_fused(base, x, [A[i] for i in ids], [B[i] for i in ids], seg, [2.0] * T, 1.0, dt)
+            if exact:
+                assert np.array_equal(to_np(vs[p]), vo), f"v of projection {p}"
+                assert np.array_equal(to_np(dev[p]["y"]), yo), f"y of projection {p}"
+            else:
+                close(to_np(vs[p]), vo)
+                close(to_np(dev[p]["y"]), yo)
 
 
 @pytest.mark.parametrize("cfg", ["decode_fp16", "train_bf16"])

@@ -339,3 +339,41 @@ def test_oracle_matches_golden_fixture(oracle, dt):
     np.testing.assert_allclose(gx, z[f"{dt}_dx"], **tol)
     np.testing.assert_allclose(np.stack(ga), z[f"{dt}_dA"], **tol)
     np.testing.assert_allclose(np.stack(gb), z[f"{dt}_dB"], **tol)
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+def test_reference_tail_rounding_points_against_torch_16bit_ops(oracle, dt):
+    """oracle_mixed_lora_linear in 16 bits, bit for bit against torch's CPU fp16 / bf16 tensor ops
+    applied as the reference applies them (src/loquetier_src/models/mixed_lora.py:214-217):
+    lora_res (a 16-bit tensor) * scaling[lora_ids] repeated per row (a 16-bit tensor, so the
+    scale itself is rounded) -> rounded; result + lora_res -> rounded.  The scales are not
+    representable in 16 bits and the values are random, so a rounding that is skipped, moved
+    behind the add, or taken with the unrounded scale changes bits."""
+    import torch
+    tdt = torch.float16 if dt == "fp16" else torch.bfloat16
+    rng = np.random.default_rng(77)
+    T, h_in, h_out, r = 37, 64, 96, 8
+    seg, ids = [0, 5, 5, 20, 37], [1, 0, 2, 1]
+    x, A, B = _rand_case(rng, T, seg, ids, 3, h_in, h_out, r)
+    x = oracle.round_to(x, dt)
+    A = [oracle.round_to(a, dt) for a in A]
+    B = [oracle.round_to(b, dt) for b in B]
+    base = oracle.round_to(rng.standard_normal((T, h_out)), dt)
+    sc = [0.3, 1.7, 0.123, 2.9]   # none exact in fp16 or bf16
+    wa, wb = [A[i] for i in ids], [B[i] for i in ids]
+    got = oracle.mixed_lora_linear(base, x, wa, wb, seg, sc, dt)
+    # the LoRA term as the kernel hands it back: a 16-bit tensor (pinned by the GEMM tests above)
+    lora, _ = oracle.add_lora_forward(x, wa, wb, seg, h_out, dt)
+    lora_t = torch.from_numpy(lora).to(tdt)
+    scaling = torch.tensor(sc, dtype=tdt)                       # mixed_lora.py:163-166
+    lens = torch.tensor([seg[i + 1] - seg[i] for i in range(len(ids))])
+    lora_t = lora_t * torch.repeat_interleave(scaling, lens).unsqueeze(-1)   # :214-216
+    result = torch.from_numpy(base).to(tdt) + lora_t                          # :217
+    assert np.array_equal(got, result.float().numpy())
+    # and the roundings matter on this input: one rounding at the end gives other bits
+    fused, _ = oracle.lora_fused(base, x, wa, wb, seg, sc, 1.0, dt)
+    assert not np.array_equal(got, fused)
+    # without a scale only the add is rounded
+    got1 = oracle.mixed_lora_linear(base, x, wa, wb, seg, None, dt)
+    want1 = torch.from_numpy(base).to(tdt) + torch.from_numpy(lora).to(tdt)
+    assert np.array_equal(got1, want1.float().numpy())
