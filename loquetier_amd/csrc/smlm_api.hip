@@ -82,10 +82,7 @@ struct ShrinkCfg {
   int NB, U, MT, NW, ksplit, k_per_wave, zblocks;
 };
 
-#ifndef SMLM_DECODE_SPLIT
-#define SMLM_DECODE_SPLIT 2
-#endif
-constexpr int kDecodeSplit = SMLM_DECODE_SPLIT;  // k halves of the sixteen-wave shrink
+constexpr int kDecodeSplit = 2;  // k halves of the sixteen-wave shrink
 constexpr int kMaxExpandFold = kMaxVsplit;  // most partials the expand kernel folds itself
 
 // waves per shrink workgroup, one choice for all projections of a launch: small
@@ -194,9 +191,6 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
                   ShrinkArgs& a) {
   const int MT = row_major ? 1 : c.MT;
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 1);
-#ifdef SMLM_TUNING
-  a.dbg = tune("SMLM_TUNE_SDBG", 0);
-#endif
   const int units = tile_units_max(a.T, S, groups, MT);
   const long items = (long)units * a.items.row_start[a.items.nproj];
   a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
@@ -279,9 +273,6 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   if (block) nq = 4;
   const int chunk = block ? 32 * nq : kFwdWaves * 32 * nq;  // columns per workgroup
   a.items.nproj = nproj;
-#ifdef SMLM_TUNING
-  a.dbg = tune("SMLM_TUNE_DBG", 0);
-#endif
   a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 0);
   a.items.row_start[0] = 0;
   for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);

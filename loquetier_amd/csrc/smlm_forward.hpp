@@ -194,9 +194,6 @@ struct ShrinkArgs {
   ItemSpace items;            // chunk rows of projection p: ksplit*zblocks
   int w_kn;                   // tile-block kernel only: weights are stored [k][n]
   DropArgs drop;              // DROP kernels: dropout of the training rows of x
-#ifdef SMLM_TUNING
-  int dbg;                    // experiments: 1 = no weight loads, 2 = no x loads, 4 = no partial/output store
-#endif
 };
 
 // Shrink for single tiles (batches below 1024 rows).  Work item -> (projection, k
@@ -241,19 +238,11 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
       for (int u = 0; u < U; ++u) {
         const int kk = k + 32 * u + 8 * g;
         const bool kin = kk < kend;
-        xf[u] = ldg16_or(P.x + (long)row * P.d_in + kk, kin && row >= 0
-#ifdef SMLM_TUNING
-                                                            && !(a.dbg & 2)
-#endif
-                         , zeros);
+        xf[u] = ldg16_or(P.x + (long)row * P.d_in + kk, kin && row >= 0, zeros);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const int n = n0 + 16 * nb + c;
-          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < nlim
-#ifdef SMLM_TUNING
-                                                             && !(a.dbg & 1)
-#endif
-                                        , zeros);
+          wf[nb][u] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kin && n < nlim, zeros);
         }
       }
     };
@@ -310,9 +299,6 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         for (int w = 1; w < NW; ++w) sum += part[w];
         const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
         if (n >= P.d_out) continue;
-#ifdef SMLM_TUNING
-        if ((a.dbg & 4) && sum[0] != 12345.f) continue;
-#endif
         if (as_partial)
           *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + row) * P.d_out + n) = sum;
         else
@@ -374,11 +360,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int kk = kb + 32 * u + 8 * g;
-        xf[u] = ldg16_or(xrow + kk, row >= 0 && kk < kend
-#ifdef SMLM_TUNING
-                                        && !(a.dbg & 2)
-#endif
-                         , zeros);
+        xf[u] = ldg16_or(xrow + kk, row >= 0 && kk < kend, zeros);
       }
     };
     auto load_w = [&](int kb, u32x4 (&st)[kPer]) {
@@ -392,11 +374,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
         } else {
           const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
           st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
-                           idx < kPieces && n0 + nl < nlim && kb + k8 < kend
-#ifdef SMLM_TUNING
-                               && !(a.dbg & 1)
-#endif
-                           , zeros);
+                           idx < kPieces && n0 + nl < nlim && kb + k8 < kend, zeros);
         }
       }
     };
@@ -460,9 +438,6 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
       for (int nb = 0; nb < NB; ++nb) {
         const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
         if (n >= P.d_out) continue;
-#ifdef SMLM_TUNING
-        if ((a.dbg & 4) && acc[nb][0] != 12345.f) continue;
-#endif
         if (as_partial)
           *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.T + row) * P.d_out + n) = acc[nb];
         else
@@ -571,9 +546,6 @@ struct ExpandArgs {
   ItemSpace items;           // chunk rows of projection p: its column chunks
   int w_kn;                  // tile-block kernel only: weights are stored [k][n]
   DropArgs drop;             // DROP kernels (the backward's dX): the mask and factor applied to the stored values
-#ifdef SMLM_TUNING
-  int dbg;                   // experiments: 1 = no weights / multiply, 2 = no read of y
-#endif
 };
 
 // by-products one wave per tile writes while it holds the token fragment: the
@@ -864,17 +836,10 @@ void expand_block_kernel(ExpandArgs a) {
       } else {
         const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
         stage[j] = ldg16_or(W + (long)(ncol0 + nl) * P.ldw + k8,
-                            idx < kPieces && ncol0 + nl < P.d_out && k8 < klim
-#ifdef SMLM_TUNING
-                                && !(a.dbg & 1)
-#endif
-                            , zeros);
+                            idx < kPieces && ncol0 + nl < P.d_out && k8 < klim, zeros);
       }
     }
-    bool read_y = a.beta != 0.0f;
-#ifdef SMLM_TUNING
-    if (a.dbg & 2) read_y = false;
-#endif
+    const bool read_y = a.beta != 0.0f;
     u32x4 yold[NQ / 2][2];
     load_y_lines<NQ>(yold, L, ncol0, P.d_out, read_y, zeros);
     if (DROP) load_keep_bits<NQ>(L, a.drop, ncol0, P.d_out, zeros);

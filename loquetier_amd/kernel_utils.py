@@ -102,13 +102,18 @@ def _unique_adapters(weight_list: Sequence[torch.Tensor]):
 def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Optional[torch.Tensor],
                   weight_list: Sequence[torch.Tensor], tp: Sequence[int], lora_rank: int,
                   part_scale: Optional[torch.Tensor] = None, dropout=None,
-                  adapter_rank: Optional[torch.Tensor] = None):
+                  adapter_rank: Optional[torch.Tensor] = None, step=None):
     """Shared backward: returns (grad_x [T, h_in], [grad per weight occurrence]).
 
     Partitions that train the same adapter contribute to one summed gradient,
     returned for the first occurrence of that adapter; later occurrences get
     None (autograd adds per-occurrence gradients, so the total is the same as
-    the reference's, src/loquetier_src/models/mixed_lora.py:201-204)."""
+    the reference's, src/loquetier_src/models/mixed_lora.py:201-204).
+
+    `step` (mixed_lora.LayerStep or None): the backward's plan, the partitions'
+    adapters, the weights' pointer tables and the layout of one buffer for all the
+    gradients, prepared outside the layer loop; without it they are built here
+    (five small host-to-device copies and a plan launch per call)."""
     dev, dt = grad_output.device, grad_output.dtype
     T = grad_output.size(0)
     h_in = x_train.size(1)
@@ -120,21 +125,39 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
         grad_x[tl:].zero_()
     if tp[0] > 0:
         grad_x[: tp[0]].zero_()
-    pairs, part_adapter = _unique_adapters(weight_list[: 2 * n_parts])
-    da = [torch.empty_like(wa) for wa, _ in pairs]
-    db = [torch.empty_like(wb) for _, wb in pairs]
-    if tl > 0:
-        g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
-        part_indptr = torch.tensor(tp, dtype=torch.int32, device=dev)
-        part_ad = torch.tensor(part_adapter, dtype=torch.int32, device=dev)
-        plan = kernel.SegmentPlan(part_indptr, part_ad, tl)
-        kernel.smlm_lora_backward(
-            grad_x, _ptr_table(da, dev), _ptr_table(db, dev), g, x_train, v_train,
-            _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
-            plan, lora_rank, part_scale, dropout=dropout, adapter_rank=adapter_rank)
+    prepared = step is not None and step.bwd_plan is not None and step.grad_offsets is not None
+    if prepared:
+        part_adapter = step.part_adapter
+        shapes, numel = step.grad_shapes
+        buf = torch.empty(numel, dtype=dt, device=dev)          # all dA, then all dB, in one allocation
+        mats = [buf[o: o + shape[0] * shape[1]].view(shape) for o, shape in shapes]
+        NA = len(mats) // 2
+        da, db = mats[:NA], mats[NA:]
+        tabs = step.grad_offsets + buf.data_ptr()               # device arithmetic, no copy from the host
+        if tl > 0:
+            g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
+            kernel.smlm_lora_backward(grad_x, tabs[:NA], tabs[NA:], g, x_train, v_train, step.a_tab, step.b_tab,
+                                      step.bwd_plan, lora_rank, part_scale, dropout=dropout,
+                                      adapter_rank=adapter_rank, workspace=step.workspace)
+        else:
+            buf.zero_()
     else:
-        for t in da + db:
-            t.zero_()
+        pairs, part_adapter = _unique_adapters(weight_list[: 2 * n_parts])
+        da = [torch.empty_like(wa) for wa, _ in pairs]
+        db = [torch.empty_like(wb) for _, wb in pairs]
+        if tl > 0:
+            g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
+            part_indptr = torch.tensor(tp, dtype=torch.int32, device=dev)
+            part_ad = torch.tensor(part_adapter, dtype=torch.int32, device=dev)
+            plan = kernel.SegmentPlan(part_indptr, part_ad, tl)
+            kernel.smlm_lora_backward(
+                grad_x, _ptr_table(da, dev), _ptr_table(db, dev), g, x_train, v_train,
+                _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
+                plan, lora_rank, part_scale, dropout=dropout, adapter_rank=adapter_rank,
+                workspace=None if step is None else step.workspace)
+        else:
+            for t in da + db:
+                t.zero_()
     grads: List[Optional[torch.Tensor]] = []
     seen = set()
     for ad in part_adapter:
@@ -162,10 +185,17 @@ class add_lora(Function):
     def forward(ctx: FunctionCtx, y_shape, x, wa_ptr, wb_ptr, s, lora_rank, train_len,
                 train_partition, *args):
         y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
-        plan = kernel.SegmentPlan(s, wa_ptr, x.size(0))
         need_v = len(args) > 0 and train_len > 0
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
-        kernel.smlm_lora_forward(y, x, wa_ptr, wb_ptr, plan, lora_rank, v_out=v)
+        # The reference looks up wa_ptr[i] and wb_ptr[i] per problem, so two segments may share A and
+        # differ in B.  A plan groups segments by ONE key and reads the weights of a group's first
+        # segment: the shrink stage runs over a plan keyed by the A addresses, the expand stage over
+        # one keyed by the B addresses (v lies between them by row, whatever the grouping).
+        plan_a = kernel.SegmentPlan(s, wa_ptr, x.size(0))
+        plan_b = kernel.SegmentPlan(s, wb_ptr, x.size(0))
+        v_arg = None if v is None else [v]  # both stages: where the shrink leaves v is where the expand finds it
+        kernel.smlm_lora_forward_multi([y], [x], [wa_ptr], [wb_ptr], plan_a, lora_rank, stages=1, v_out=v_arg)
+        kernel.smlm_lora_forward_multi([y], [x], [wa_ptr], [wb_ptr], plan_b, lora_rank, stages=2, v_out=v_arg)
         # what the reference's setup_context keeps (kernel_utils.py:122-126), plus v
         ctx.tp = train_partition
         ctx.rank = lora_rank

@@ -24,8 +24,12 @@ from .ops import _kernels as kernel
 
 class MixedLoraContext:
     """Per-step routing record shared by every LoRA linear of a model
-    (reference: mixed_lora.py:24-64).  `update` also builds the tile plan and
-    the device copy of the adapter ids once, for all layers of the step."""
+    (reference: mixed_lora.py:24-64).  Everything that depends only on the step's
+    routing is built here ONCE per `update` and shared by all layers: the device
+    copy of the adapter ids, the tile plan of the forward, the partition plan of
+    the backward, the partition -> segment map.  The context also owns the scratch
+    memory the kernels use, so that no layer allocates or copies anything from the
+    host inside the layer loop."""
 
     def __init__(self):
         self._blen = None
@@ -35,6 +39,9 @@ class MixedLoraContext:
         self._train_idx: List[int] = []
         self._plan: Optional[kernel.SegmentPlan] = None
         self._seg_adapter: Optional[torch.Tensor] = None
+        self._step: dict = {}          # per-step memo, dropped by update()
+        self._workspaces: dict = {}    # device -> kernel.Workspace, kept across steps
+        self._dropout_calls = 0        # host-side counter: every dropout call gets its own mask stream
 
     def update(self, blen: Optional[BatchLenInfo] = None, lora_ids: Optional[List[int]] = None,
                lora_len: Optional[torch.Tensor] = None, segment: Optional[torch.Tensor] = None,
@@ -46,6 +53,7 @@ class MixedLoraContext:
         self._train_idx = list(train_idx)
         self._plan = None
         self._seg_adapter = None
+        self._step = {}
 
     @property
     def blen(self) -> Optional[BatchLenInfo]:
@@ -67,6 +75,26 @@ class MixedLoraContext:
     def train_idx(self) -> List[int]:
         return self._train_idx
 
+    def memo(self, key, build):
+        """Value built once per step (per `update`) and shared by every layer that asks for `key`."""
+        if key not in self._step:
+            self._step[key] = build()
+        return self._step[key]
+
+    def workspace(self, device: torch.device) -> "kernel.Workspace":
+        """Scratch memory of the kernels, owned by the context (grow-only; size it with one eager
+        step before capturing a graph)."""
+        ws = self._workspaces.get(device)
+        if ws is None:
+            ws = self._workspaces[device] = kernel.Workspace(device)
+        return ws
+
+    def next_dropout_offset(self) -> int:
+        """Offset of the next dropout mask stream: a host-side counter, so drawing it waits for nothing
+        (eight projections' worth of offsets apart)."""
+        self._dropout_calls += 1
+        return self._dropout_calls * 8
+
     def seg_adapter(self, device: torch.device) -> torch.Tensor:
         """Adapter id of every segment as a device tensor.  `lora_ids` may already be one (int32,
         e.g. from segments.build_segments_device, whose arrays keep the request count as capacity
@@ -79,10 +107,44 @@ class MixedLoraContext:
                 self._seg_adapter = torch.tensor(self._lora_ids, dtype=torch.int32, device=device)
         return self._seg_adapter
 
+    def seg_adapter_long(self, device: torch.device) -> torch.Tensor:
+        return self.memo(("seg_adapter_long", device), lambda: self.seg_adapter(device).long())
+
     def plan(self, device: torch.device, T: int) -> kernel.SegmentPlan:
         if self._plan is None or self._plan.T != T or self._plan.buf.device != device:
             self._plan = kernel.SegmentPlan(self._segment.to(device), self.seg_adapter(device), T)
         return self._plan
+
+    def train_order(self) -> List[int]:
+        """Training adapters in order of first appearance among the train partitions: the backward
+        numbers them 0..NA-1 in this order."""
+        return list(dict.fromkeys(int(i) for i in self._train_idx))
+
+    def backward_tables(self, device: torch.device):
+        """(partition plan, partition -> training adapter list) of the step's backward: a function
+        of the train partitions and their adapters only, so one serves every layer."""
+        def build():
+            tp = [int(t) for t in self._blen.train_partition]
+            n_parts = min(len(self._train_idx), len(tp) - 1)
+            tp = tp[: n_parts + 1]
+            order = self.train_order()
+            part_adapter = [order.index(int(i)) for i in self._train_idx[:n_parts]]
+            if n_parts == 0 or tp[-1] == 0:
+                return None, part_adapter
+            plan = kernel.SegmentPlan(torch.tensor(tp, dtype=torch.int32, device=device),
+                                      torch.tensor(part_adapter, dtype=torch.int32, device=device), tp[-1])
+            return plan, part_adapter
+        return self.memo(("backward", device), build)
+
+    def part_segments(self, device: torch.device, plan: kernel.SegmentPlan) -> torch.Tensor:
+        """Segment that starts every train partition (int64 device indices): the partition's scale
+        and dropout probability are those of that segment."""
+        def build():
+            n_parts = min(len(self._train_idx), len(self._blen.train_partition) - 1)
+            starts = torch.tensor([int(t) for t in self._blen.train_partition][:n_parts],
+                                  dtype=torch.int32, device=device)
+            return (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, max(plan.S - 1, 0))
+        return self.memo(("part_segments", device), build)
 
 
 @dataclass
@@ -117,21 +179,23 @@ class fused_add_lora(Function):
     """result <- result + scale_seg * (x A_seg^T) B_seg^T, in place, one call.
 
     Arguments: (result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-    train_len, train_partition, dropout, adapter_rank, *weights); the tables hold
-    one address per adapter and the plan is keyed by adapter id.  `adapter_rank`
+    train_len, train_partition, dropout, adapter_rank, step, *weights); the tables
+    hold one address per adapter and the plan is keyed by adapter id.  `adapter_rank`
     (None, or a pair of int32 device tensors: the true rank of every adapter, and
     of the training adapters in order of first appearance among the partitions)
     tells the kernels which adapters are stored zero-padded.  `dropout` (a
     kernel.DropoutSpec or None) drops the training rows of x inside the kernels,
     in place of the reference's nn.Dropout calls and torch.cat before the op
     (src/loquetier_src/models/mixed_lora.py:185-192); x is the tensor before
-    dropout.  Returns `result`.
+    dropout.  `step` (None, or a LayerStep) carries what the step's context and the
+    layer have prepared once: scratch memory, the backward's plan and pointer tables.
+    Returns `result`.
     Gradients: result -> passed through, x -> dX on train rows (zero elsewhere),
     each trainable weight -> its summed gradient (None when not training)."""
 
     @staticmethod
     def forward(ctx: FunctionCtx, result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-                train_len, train_partition, dropout, adapter_rank, *weights):
+                train_len, train_partition, dropout, adapter_rank, step, *weights):
         need_v = len(weights) > 0 and train_len > 0
         adapter_rank, train_rank = adapter_rank if adapter_rank is not None else (None, None)
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
@@ -141,21 +205,26 @@ class fused_add_lora(Function):
                                device=x.device)
             dropout = kernel.DropoutSpec(dropout.seg_p, dropout.rows, dropout.seed, dropout.offset, bits)
         kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
-                                 beta=1.0, v_out=v, dropout=dropout, adapter_rank=adapter_rank)
+                                 beta=1.0, v_out=v, dropout=dropout, adapter_rank=adapter_rank,
+                                 workspace=None if step is None else step.workspace)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
         ctx.has_v = v is not None
         ctx.n_parts = len(weights) // 2
+        ctx.step = step
         # scale of each train partition = scale of the segment that starts it;
         # kept as a device gather so nothing is read back to the host
         ctx.part_scale = None
         ctx.part_drop = None
         ctx.train_rank = train_rank if need_v else None
         if need_v and (seg_scale is not None or dropout is not None):
-            starts = torch.tensor([int(t) for t in train_partition][: ctx.n_parts],
-                                  dtype=torch.int32, device=x.device)
-            seg_of = (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, plan.S - 1)
+            if step is not None:
+                seg_of = step.part_segments
+            else:
+                starts = torch.tensor([int(t) for t in train_partition][: ctx.n_parts],
+                                      dtype=torch.int32, device=x.device)
+                seg_of = (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, plan.S - 1)
             if seg_scale is not None:
                 ctx.part_scale = seg_scale[seg_of].contiguous()
             if dropout is not None:  # the same stream, probabilities by train partition
@@ -167,14 +236,28 @@ class fused_add_lora(Function):
 
     @staticmethod
     def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
-        n_fixed = 11
+        n_fixed = 12
         if not ctx.has_v:
             return (grad_output, None) + (None,) * (n_fixed - 2) + (None,) * (2 * ctx.n_parts)
         x, v, *weight_list = ctx.saved_tensors
         grad_x, grads = lora_backward(grad_output, x, v, weight_list, ctx.tp, ctx.rank,
                                       part_scale=ctx.part_scale, dropout=ctx.part_drop,
-                                      adapter_rank=ctx.train_rank)
+                                      adapter_rank=ctx.train_rank, step=ctx.step)
         return (grad_output, grad_x) + (None,) * (n_fixed - 2) + tuple(grads)
+
+
+@dataclass
+class LayerStep:
+    """What one layer call hands to the operator besides tensors: prepared once per step by the
+    context (shared by all layers) or once per adapter set by the layer, never inside the call."""
+    workspace: Any                      # kernel.Workspace owned by the context
+    part_segments: Optional[torch.Tensor] = None   # segment that starts every train partition
+    bwd_plan: Optional[Any] = None      # kernel.SegmentPlan over the train partitions
+    part_adapter: Optional[List[int]] = None       # training-adapter index of every partition
+    a_tab: Optional[torch.Tensor] = None           # addresses of the training adapters' A / B, in order
+    b_tab: Optional[torch.Tensor] = None
+    grad_offsets: Optional[torch.Tensor] = None    # byte offsets of dA_0.., dB_0.. inside one gradient buffer
+    grad_shapes: Optional[list] = None             # [(offset in elements, shape)] in the same order
 
 
 class MixedLoraLinear(nn.Module):
@@ -208,6 +291,42 @@ class MixedLoraLinear(nn.Module):
         self.adapter_rank = (torch.tensor(ranks, dtype=torch.int32, device=self.device)
                              if any(q < rank for q in ranks) else None)
         self._train_rank_key, self._train_rank = None, None
+        self._scaling_f32 = None if self.is_scaled else self.scaling.float()
+        self._scaling_key = None if self.is_scaled else tuple(float(a.scaling) for a in adapters)
+        self._train_tabs: dict = {}   # training-adapter order -> pointer tables and gradient layout
+        self._drop_probs: dict = {}   # adapter dropout probabilities -> device tensor
+
+    def _train_tables(self, order):
+        """Pointer tables of the training adapters' weights and the layout of one buffer holding all
+        their gradients; built once per set of training adapters (addresses of the weights are
+        stable: the parameters share the adapters' storage)."""
+        key = tuple(order)
+        tabs = self._train_tabs.get(key)
+        if tabs is None:
+            idx = torch.tensor(list(order), dtype=torch.long, device=self.device)
+            shapes, offsets, off = [], [], 0
+            for group in ("wa", "wb"):
+                for i in order:
+                    w = getattr(self.adapters[i], group)
+                    shapes.append((off, tuple(w.shape)))
+                    offsets.append(off * w.element_size())
+                    off += (w.numel() + 7) // 8 * 8   # every matrix 16-byte aligned
+            tabs = dict(a_tab=self.wa_ptrs[idx].contiguous(), b_tab=self.wb_ptrs[idx].contiguous(),
+                        grad_offsets=torch.tensor(offsets, dtype=torch.int64, device=self.device),
+                        grad_shapes=shapes, grad_numel=off)
+            self._train_tabs[key] = tabs
+        return tabs
+
+    def _seg_dropout(self, ctx, train_idx):
+        """Dropout probability of every segment (device float32) or None when no training adapter drops."""
+        probs = tuple(float(a.dropout.p) if isinstance(a.dropout, nn.Dropout) and a.dropout.training else 0.0
+                      for a in self.adapters)
+        if not any(probs[idx] > 0.0 for idx in train_idx):
+            return None
+        table = self._drop_probs.get(probs)
+        if table is None:
+            table = self._drop_probs[probs] = torch.tensor(probs, dtype=torch.float32, device=self.device)
+        return ctx.memo(("seg_p", probs, self.device), lambda: table[ctx.seg_adapter_long(self.device)])
 
     def _rank_args(self, train_idx):
         """(ranks of all adapters, ranks of the training adapters in order of first appearance),
@@ -249,15 +368,12 @@ class MixedLoraLinear(nn.Module):
         drop_spec = None
         if blen.tlen > 0 and self.fused:
             # the kernels drop the training rows themselves: no dropped copy, no torch.cat
-            probs = [float(a.dropout.p) if isinstance(a.dropout, nn.Dropout) and a.dropout.training else 0.0
-                     for a in self.adapters]
-            if any(probs[idx] > 0.0 for idx in train_idx):
-                seg_p = torch.tensor(probs, dtype=torch.float32, device=self.device)[
-                    ctx.seg_adapter(self.device).long()]
-                # the stream: torch's seed, and an offset drawn from torch's generator so that every
-                # call (layer, step) gets its own mask and torch.manual_seed makes runs repeatable
-                offset = int(torch.randint(0, 2 ** 62, (1,)).item())
-                drop_spec = kernel.DropoutSpec(seg_p, blen.tlen, torch.initial_seed(), offset)
+            seg_p = self._seg_dropout(ctx, train_idx)
+            if seg_p is not None:
+                # the stream: torch's seed, and an offset from the context's host-side counter, so that
+                # every call (layer, step) gets its own mask, torch.manual_seed makes runs repeatable
+                # and nothing waits for the device
+                drop_spec = kernel.DropoutSpec(seg_p, blen.tlen, torch.initial_seed(), ctx.next_dropout_offset())
         elif blen.tlen > 0:
             dropped_x = []
             for idx, pi in zip(train_idx, range(len(blen.train_partition) - 1)):
@@ -267,14 +383,27 @@ class MixedLoraLinear(nn.Module):
         weights = [w for idx in train_idx for w in (self.get_parameter(f"lora-{idx}-A"),
                                                     self.get_parameter(f"lora-{idx}-B"))]
         if self.fused:
-            seg_adapter = ctx.seg_adapter(self.device)
-            seg_scale = None if self.is_scaled else self.scaling.float()[seg_adapter.long()]
+            # per-step tables come from the context (built once for all layers), per-layer ones from
+            # the layer (built once per adapter set): nothing is copied from the host in here
+            seg_scale = None
+            if not self.is_scaled:
+                # (layers whose adapters have the same scales share one gather per step)
+                seg_scale = ctx.memo(("seg_scale", self._scaling_key, self.device),
+                                     lambda: self._scaling_f32[ctx.seg_adapter_long(self.device)])
             result = result.to(self.dtype).contiguous()
             if not x.is_contiguous():
                 x = x.contiguous()
-            result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale,
-                                          ctx.plan(self.device, x.size(0)), self.rank, blen.tlen,
-                                          blen.train_partition, drop_spec, self._rank_args(train_idx), *weights)
+            plan = ctx.plan(self.device, x.size(0))
+            step = LayerStep(workspace=ctx.workspace(self.device))
+            if weights and blen.tlen > 0:
+                step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
+                step.part_segments = ctx.part_segments(self.device, plan)
+                tabs = self._train_tables(ctx.train_order())
+                step.a_tab, step.b_tab = tabs["a_tab"], tabs["b_tab"]
+                step.grad_offsets, step.grad_shapes = tabs["grad_offsets"], (tabs["grad_shapes"], tabs["grad_numel"])
+            result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale, plan, self.rank,
+                                          blen.tlen, blen.train_partition, drop_spec,
+                                          self._rank_args(train_idx), step, *weights)
             return result.to(torch_result_dtype)
 
         segment = ctx.segment.to(self.device)

@@ -864,3 +864,24 @@ def test_full_size_gaussian_tolerance(K, gpu_device, cfg):
         y_ref = v[a:b].float() @ B[ids[i]].float().t()
         assert bool(((v[a:b].float() - v_ref).abs() <= ATOL + RTOL * v_ref.abs()).all())
         assert bool(((y[a:b].float() - y_ref).abs() <= ATOL + RTOL * y_ref.abs()).all())
+
+
+def test_add_lora_segments_sharing_a_but_not_b(K, oracle, gpu_device):
+    """The reference reads wa_ptr[i] and wb_ptr[i] per problem (smlm_forward_cutlass.cuh:31-46), so
+    segments may share their A and differ in B (or the other way round): every segment must get
+    its own pair."""
+    from loquetier_amd.kernel_utils import add_lora
+    d, dt = gpu_device, "fp16"
+    T, h_in, h_out, r = 60, 256, 192, 16
+    seg = [0, 10, 25, 26, 40, 60]
+    a_of, b_of = [0, 0, 1, 0, 1], [0, 1, 1, 2, 0]      # A shared by segments 0, 1, 3; B differs
+    rng = np.random.default_rng(61)
+    x = dyadic(rng, (T, h_in), 16, 8)
+    A = [dyadic(rng, (r, h_in), 8, 64) for _ in range(2)]
+    B = [dyadic(rng, (h_out, r), 8, 8) for _ in range(3)]
+    xd = dev_t(x, dt, d)
+    Ad, Bd = [dev_t(a, dt, d) for a in A], [dev_t(b, dt, d) for b in B]
+    s = torch.tensor(seg, dtype=torch.int32, device=d)
+    y = add_lora.apply((T, h_out), xd, ptrs([Ad[i] for i in a_of], d), ptrs([Bd[i] for i in b_of], d), s, r, 0, [0])
+    yo, _ = oracle.add_lora_forward(x, [A[i] for i in a_of], [B[i] for i in b_of], seg, h_out, dt)
+    assert np.array_equal(to_np(y), yo)
