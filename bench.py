@@ -206,46 +206,171 @@ def rmsnorm_bench(args, torch, K):
         "cpu_baseline": cpu}), flush=True)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="cfg2")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
-    ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
-    ap.add_argument("--eager", action="store_true",
-                    help="launch the steps one by one instead of replaying a graph (for counter runs)")
-    ap.add_argument("--sorted", action="store_true",
-                    help="hand the same requests over grouped by adapter (a scheduler that batches by adapter)")
-    ap.add_argument("--padded-ranks", action="store_true",
-                    help="workloads with adapters below the padded rank: do not pass the true ranks "
-                         "(the kernels then read the zero padding, as the reference's do)")
-    ap.add_argument("--dropout", type=float, default=0.0,
-                    help="dropout probability of the training adapters (workloads with a backward): the "
-                         "kernels regenerate the mask in the forward and the backward; default 0 = off")
-    ap.add_argument("--calibration-copy", action="store_true",
-                    help="also run a 128 MiB device copy three times before the timed region: a kernel "
-                         "of known traffic to scale FETCH_SIZE / WRITE_SIZE readings with")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; every box has one MI355X and no collective, "
-              "sharding or rank code exists in it. Run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
-
-    import torch
-    if not torch.cuda.is_available():
-        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
-    from loquetier_amd import _lib
-    from loquetier_amd.ops import _kernels as K
-    _lib.load()  # no fallback: raises when the HIP library is missing
-    if args.config == "rmsnorm":
-        return rmsnorm_bench(args, torch, K)
-
+def model_step_bench(args, torch, K):
+    """The path as the reference drives it (src/loquetier_src/models/mixed_lora.py:173-218, 224 LoRA linears
+    per model forward): 32 layers x (q, k, v, o, gate, up, down) of Llama-2-7B through MixedLoraLinear(fused=True)
+    with ONE MixedLoraContext.update per step.  The base layers hand back preallocated outputs (their GEMMs
+    are not part of this path).  Reports, per layer call: host time of an eager step (Python + ctypes + launch),
+    GPU time of the same step replayed from a graph, for the decode batch (forward) and, eager only, for the
+    fine-tune + serve batch (forward + backward through autograd)."""
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.mixed_lora import MixedLoraContext, MixedLoraLinear, NamedLoraLayer
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    w = workload(args.config)
+    shapes = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
+              ("gate", 4096, 11008), ("up", 4096, 11008), ("down", 11008, 4096)]
+    n_layers = 32
+
+    class Base(torch.nn.Module):
+        """Stands in for the frozen base projection: returns its (preallocated) output."""
+
+        def __init__(self, out):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.empty(1, device=dev), requires_grad=False)
+            self.out = out
+
+        def forward(self, x):
+            return self.out.detach()  # a fresh tensor object over the same memory: no autograd history
+
+    def build(cfg, trainable):
+        w = workload(cfg)
+        tdt = torch.float16 if w["dtype"] == "fp16" else torch.bfloat16
+        T, r, NA = w["seg"][-1], w["r"], w["NA"]
+        gen = torch.Generator(device="cpu").manual_seed(11)
+        ctx = MixedLoraContext()
+        pool = {h: [torch.randn(T, h, generator=gen).to(dev).to(tdt) for _ in range(8)] for h in (4096, 11008)}
+        outs = {h: [torch.randn(T, h, generator=gen).to(dev).to(tdt) for _ in range(8)] for h in (4096, 11008)}
+        layers = []
+        for li in range(n_layers):
+            for pi, (_, hi, ho) in enumerate(shapes):
+                A = (torch.randn(NA, r, hi, generator=gen) * hi ** -0.5).to(dev).to(tdt)
+                B = (torch.randn(NA, ho, r, generator=gen) * r ** -0.5).to(dev).to(tdt)
+                ad = [NamedLoraLayer(f"a{a}", A[a], B[a], torch.nn.Identity(), 2.0) for a in range(NA)]
+                k = (li * len(shapes) + pi) % 8
+                layer = MixedLoraLinear(ctx, Base(outs[ho][k]), ad, r, tdt, is_scaled=False, fused=True)
+                if trainable:
+                    layer.set_trainable(trainable)
+                layers.append((layer, pool[hi][k]))
+        return w, ctx, layers, tdt
+
+    staged = {}
+
+    def update(w, ctx, trainable):
+        # what ModelGeneration.generate hands over once per step (model_generation.py:267-283); the index
+        # arrays are staged on the device once (a serving loop builds them there, smlm_segments_build)
+        P = w["n_train_parts"] if trainable else 0
+        key = (w["name"], P)
+        if key not in staged:
+            lens = [w["seg"][i + 1] - w["seg"][i] for i in range(len(w["ids"]))]
+            staged[key] = (BatchLenInfo([(1, n) for n in lens[:P]], [], sum(lens[P:]), [], dev),
+                           torch.tensor(w["ids"], dtype=torch.int32, device=dev),
+                           torch.tensor(lens, dtype=torch.int32, device=dev),
+                           torch.tensor(w["seg"], dtype=torch.int32, device=dev))
+        blen, ids_t, lens_t, seg_t = staged[key]
+        ctx.update(blen=blen, lora_ids=ids_t, lora_len=lens_t, segment=seg_t, train_idx=w["ids"][:P])
+
+    out = {"metric": "SMLM layer path: per-call time of MixedLoraLinear(fused=True), 224 calls per model step",
+           "n_gpus": 1, "data": "synthetic", "config": {"workload": "model-step: 32 layers x q,k,v,o,gate,up,down, "
+                                                                 "Llama-2-7B shapes"}}
+    # ---- decode batch, forward
+    w, ctx, layers, tdt = build("cfg2", [])
+    cap = torch.cuda.Stream()
+
+    def fwd_step():
+        update(w, ctx, [])
+        for layer, x in layers:
+            layer(x)
+    with torch.no_grad(), torch.cuda.stream(cap):
+        for _ in range(3):
+            fwd_step()
+        torch.cuda.synchronize()
+        n_eager = max(1, min(args.steps, 50))
+        t0 = time.perf_counter()
+        for _ in range(n_eager):
+            fwd_step()
+        host_us = (time.perf_counter() - t0) * 1e6 / (n_eager * len(layers))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_eager):
+            fwd_step()
+        torch.cuda.synchronize()
+        eager_us = (time.perf_counter() - t0) * 1e6 / (n_eager * len(layers))
+    g = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(g, stream=cap):
+        fwd_step()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(2):
+        g.replay()
+    a.record()
+    for _ in range(10):
+        g.replay()
+    b.record()
+    torch.cuda.synchronize()
+    graph_us = a.elapsed_time(b) * 1e3 / (10 * len(layers))
+    T = w["seg"][-1]
+    step_bytes = sum(algorithmic_bytes(w, hi, ho) for _, hi, ho in shapes) * n_layers
+    out["decode_forward"] = dict(workload=w["name"], calls_per_step=len(layers), host_us_per_call=round(host_us, 2),
+                                 eager_us_per_call=round(eager_us, 2), graph_gpu_us_per_call=round(graph_us, 2),
+                                 graph_ms_per_model_step=round(graph_us * len(layers) / 1e3, 4),
+                                 step_hbm_gbps=round(step_bytes / (graph_us * len(layers) * 1e-6) / 1e9, 1),
+                                 tokens_per_s=round(T / (graph_us * len(layers) * 1e-6), 1))
+    del layers, g
+    torch.cuda.empty_cache()
+
+    # ---- fine-tune + serve batch, forward + backward through autograd (eager)
+    w, ctx, layers, tdt = build("cfg4", [0, 1, 2, 3])
+    n_train = w["seg"][w["n_train_parts"]]
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    grads = {h: torch.randn(w["seg"][-1], h, generator=gen).to(dev).to(tdt) for h in (4096, 11008)}
+
+    def train_step():
+        update(w, ctx, [0, 1, 2, 3])
+        outs = []
+        for layer, x in layers:
+            outs.append(layer(x))  # dX is computed and handed to autograd, which has no use for it here
+        t_f = time.perf_counter()
+        for o in reversed(outs):
+            o.backward(grads[o.size(1)])
+        return t_f
+    with torch.cuda.stream(cap):
+        for _ in range(2 + max(0, min(args.steps, 50) - 5) // 4):  # (more steps on request: copy-trace runs)
+            train_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        t_f = train_step()
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        a.record(cap)
+        train_step()
+        b.record(cap)
+        torch.cuda.synchronize()
+    out["finetune_forward_backward"] = dict(
+        workload=w["name"], calls_per_step=len(layers), training_rows=n_train,
+        host_us_per_call_forward=round((t_f - t0) * 1e6 / len(layers), 2),
+        host_us_per_call_backward=round((t1 - t_f) * 1e6 / len(layers), 2),
+        eager_us_per_call_incl_gpu=round((t2 - t0) * 1e6 / len(layers), 2),
+        event_us_per_call=round(a.elapsed_time(b) * 1e3 / len(layers), 2))
+    print(json.dumps(out), flush=True)
+
+
+def load_probe():
+    """The plain streaming kernels (loquetier_amd/lib/libsmlm_probe.so); None when not built."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "loquetier_amd", "lib", "libsmlm_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path)
+    lib.smlm_probe_rmw.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p]
+    lib.smlm_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
+    return lib
+
+
+def run_workload(args, cfg, torch, K, probe, brief=False):
+    """One workload: the whole step, the two forward launches alone, the plain streaming kernels at the
+    same launch sizes and the CPU baseline.  brief: fewer side measurements and a short CPU sample (the
+    non-headline workloads of the default run)."""
+    dev = torch.device("cuda:0")
+    w = workload(cfg)
     if args.sorted:
         w = adapter_sorted(w)
     tdt = torch.float16 if w["dtype"] == "fp16" else torch.bfloat16
@@ -261,7 +386,7 @@ def main():
     R = 1 if args.no_rotate else max(2, math.ceil(640e6 / footprint))
     R = min(R, 16)
 
-    gen = torch.Generator(device="cpu").manual_seed(int("".join(ch for ch in args.config if ch.isdigit())))
+    gen = torch.Generator(device="cpu").manual_seed(int("".join(ch for ch in cfg if ch.isdigit())))
     seg_t = torch.tensor(w["seg"], dtype=torch.int32, device=dev)
     ids_t = torch.tensor(w["ids"], dtype=torch.int32, device=dev)
     scale_t = torch.full((S,), 2.0, device=dev)
@@ -409,15 +534,12 @@ def main():
     step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
 
     if args.step_only:
-        print(json.dumps({"config": args.config, "ms_per_step": round(ms_per_step, 5),
-                          "step_hbm_gbps": round(step_gbps, 1)}), flush=True)
-        return
+        return {"config": cfg, "ms_per_step": round(ms_per_step, 5), "step_hbm_gbps": round(step_gbps, 1)}
 
-    # ---- dominant kernel alone: the expand launch of the step (all projections of the batch,
-    # y += s * v B^T), launched back to back from a graph over the rotating buffer sets and timed
-    # with HIP events on its stream.  The shrink launch is timed the same way.
+    # ---- the two forward launches alone (all projections of the batch each): shrink v = x A^T and
+    # expand y += s * v B^T, launched back to back from a graph over the rotating buffer sets and timed
+    # with HIP events on the stream.
     reps = max(2, 48 // R)
-    ranks = w.get("true_ranks")
     rsum = sum((ranks[a % 4] if ranks else r) for a in set(w["ids"]))
 
     def stage_us(stages):
@@ -425,8 +547,12 @@ def main():
         timed([(g, 2)])
         return timed([(g, 10)]) * 1e3 / (10 * reps * R)  # us per launch
 
-    # the same step with the batch's plan built once and reused, as the layers of one model
-    # step reuse it (reported beside the headline value, never as it)
+    # the same step with the batch's plans built once and reused, as the layers of one model
+    # step reuse them (reported beside the headline value, never as it)
+    for st in sets[1:]:  # one plan for every buffer set: the routing is the same, as across the layers of a step
+        st["plan"] = sets[0]["plan"]
+        if P:
+            st["bplan"] = sets[0]["bplan"]
     g_reuse = capture(lambda: [step(st, build_plan=False) for st in sets])
     timed([(g_reuse, 2)])
     reuse_ms = timed([(g_reuse, max(1, args.steps // R))]) / (max(1, args.steps // R) * R)
@@ -435,31 +561,58 @@ def main():
     shrink_us = stage_us(1)
     expand_bytes = sum(T * ho * 2 * 2 + rsum * ho * 2 + T * r * 2 for _, hi, ho in w["proj"])
     shrink_bytes = sum(T * hi * 2 + rsum * hi * 2 + T * r * 2 for _, hi, ho in w["proj"])
-    traffic = None
+    traffic = {}
     tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(args.config, {}).get("expand_bytes_per_launch")
-    achieved = expand_bytes / (expand_us * 1e-6) / 1e9
-    roofline = dict(kernel="expand kernel, one launch for all projections of the step", bound="hbm",
-                    achieved=round(achieved, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
-                    us_per_launch=round(expand_us, 3), algorithmic_bytes=expand_bytes)
+        traffic = json.load(open(tpath)).get(cfg, {})
 
-    # ---- what a plain streaming kernel reaches at this launch size: torch's in-place add_ (one
-    # read and one write per byte, nothing else) over tensors sized so that one launch moves the
-    # expand launch's algorithmic bytes, rotating over enough of them to stay out of the
-    # Infinity Cache.  HBM-bound kernels on this part climb with the bytes per launch, so this, not
-    # the 8 TB/s peak, is what the launch above can be held against.
-    n_el = max(1, expand_bytes // 4)                      # fp16 elements: 2 bytes read + 2 written each
-    n_ref = 1 if args.no_rotate else max(2, min(64, math.ceil(640e6 / (2 * n_el))))
-    ref_bufs = [torch.zeros(n_el, dtype=torch.float16, device=dev) for _ in range(n_ref)]
-    ref_reps = max(2, 48 // n_ref)
-    g_ref = capture(lambda: [b.add_(1.0) for _ in range(ref_reps) for b in ref_bufs])
-    timed([(g_ref, 2)])
-    ref_us = timed([(g_ref, 10)]) * 1e3 / (10 * ref_reps * n_ref)
-    streaming = dict(kernel="torch in-place add_ (elementwise read-modify-write)", bytes=int(n_el * 4),
-                     us_per_launch=round(ref_us, 3), gbps=round(n_el * 4 / (ref_us * 1e-6) / 1e9, 1))
-    del ref_bufs, g_ref
+    def launch_line(kernel, us, nbytes, key):
+        gbps = nbytes / (us * 1e-6) / 1e9
+        return dict(kernel=kernel, bound="hbm", achieved=round(gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
+                    frac=round(gbps / HBM_PEAK_GBPS, 4), traffic=traffic.get(key), us_per_launch=round(us, 3),
+                    algorithmic_bytes=nbytes)
+    lines = [launch_line("shrink launch (v = x A^T, all projections of the step)", shrink_us, shrink_bytes,
+                         "shrink_bytes_per_launch"),
+             launch_line("expand launch (y += s v B^T, all projections of the step)", expand_us, expand_bytes,
+                         "expand_bytes_per_launch")]
+    # the forward launch furthest below the HBM peak is the one the roofline entry names
+    roofline = min(lines, key=lambda l: l["frac"])
+
+    # ---- what plain streaming kernels reach at these launch sizes (loquetier_amd/csrc/stream_probe.hip:
+    # a read-modify-write moving the expand launch's bytes, a read moving the shrink launch's), cold over
+    # rotating buffers and hot in the Infinity Cache.  HBM-bound launches on this part climb with the bytes
+    # per launch, so these, not the 8 TB/s peak, are what the launches above can be held against.
+    streaming = None
+    if probe is not None and not brief:
+        stream_h = cap_stream.cuda_stream
+
+        def probe_us(nbytes, write, cold):
+            n = max(2, min(64, math.ceil(640e6 / nbytes))) if cold else 1
+            bufs = [torch.zeros(nbytes // 4, dtype=torch.int32, device=dev) for _ in range(n)]
+            sink = torch.zeros(4, dtype=torch.int32, device=dev)
+            pr = max(2, 48 // n)
+
+            def go():
+                for _ in range(pr):
+                    for b in bufs:
+                        if write:
+                            probe.smlm_probe_rmw(b.data_ptr(), nbytes, stream_h)
+                        else:
+                            probe.smlm_probe_read(b.data_ptr(), nbytes, sink.data_ptr(), stream_h)
+            with torch.cuda.stream(cap_stream):
+                go()
+            torch.cuda.synchronize()
+            g = capture(go)
+            timed([(g, 2)])
+            return timed([(g, 10)]) * 1e3 / (10 * pr * n)
+        rmw_c, rmw_h = probe_us(expand_bytes // 2, True, True), probe_us(expand_bytes // 2, True, False)
+        rd_c, rd_h = probe_us(shrink_bytes, False, True), probe_us(shrink_bytes, False, False)
+        tb = lambda nbytes, us: round(nbytes / (us * 1e-6) / 1e9, 1)
+        streaming = dict(kernel="loquetier_amd/csrc/stream_probe.hip (16-byte non-temporal accesses, 8 in flight a thread)",
+                         rmw_bytes=expand_bytes, rmw_cold_us=round(rmw_c, 3), rmw_cold_gbps=tb(expand_bytes, rmw_c),
+                         rmw_hot_us=round(rmw_h, 3), rmw_hot_gbps=tb(expand_bytes, rmw_h),
+                         read_bytes=shrink_bytes, read_cold_us=round(rd_c, 3), read_cold_gbps=tb(shrink_bytes, rd_c),
+                         read_hot_us=round(rd_h, 3), read_hot_gbps=tb(shrink_bytes, rd_h))
 
     # ---- CPU baseline: per-segment torch matmuls on the host cores (bounded sample)
     cpu = None
@@ -479,17 +632,19 @@ def main():
                 if P:
                     ref.add_lora_backward(h["g"], h["x"][:n_train], h["A"], h["B"], seg[:P + 1], ids[:P])
 
-        cpu_step()
+        budget = 3.0 if brief else 10.0
+        if not brief:
+            cpu_step()
         n, t_begin = 0, time.perf_counter()
         while True:
             cpu_step()
             n += 1
             el = time.perf_counter() - t_begin
-            if el > 12.0 or n >= 200:
+            if el > budget or n >= 200:
                 break
         cpu = dict(value=round(T * n / el, 1), unit="tokens/s", cores=cores, kind="port",
-                   sample=f"{n} whole steps of the same workload ({el:.1f} s), per-segment torch.matmul "
-                          f"in fp32 on {w['dtype']} data (oracle/torch_segments.py)")
+                   sample=f"{n} whole step{'s' if n > 1 else ''} of the same workload ({el:.1f} s), per-segment "
+                          f"torch.matmul in fp32 on {w['dtype']} data (oracle/torch_segments.py)")
 
     out = {
         "metric": METRIC, "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1,
@@ -507,13 +662,70 @@ def main():
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
         "ms_per_step_plan_reused": round(reuse_ms, 5),
         "roofline": roofline,
+        "launches": lines,
         "streaming_reference": streaming,
-        "kernels": {"shrink_us": round(shrink_us, 3), "shrink_bytes": shrink_bytes,
-                    "shrink_gbps": round(shrink_bytes / (shrink_us * 1e-6) / 1e9, 1),
-                    "expand_us": round(expand_us, 3), "expand_bytes": expand_bytes,
-                    "expand_gbps": round(achieved, 1)},
         "cpu_baseline": cpu,
     }
+    del sets
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="all",
+                    help="all (default): the headline workload cfg2 in full, then cfg3, cfg4 and cfg5 in brief "
+                         "under 'configs'; or one of cfg2 | cfg2mod | cfg3 | cfg4 | cfg5 | rmsnorm | model-step")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
+    ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch the steps one by one instead of replaying a graph (for counter runs)")
+    ap.add_argument("--sorted", action="store_true",
+                    help="hand the same requests over grouped by adapter (a scheduler that batches by adapter)")
+    ap.add_argument("--padded-ranks", action="store_true",
+                    help="workloads with adapters below the padded rank: do not pass the true ranks "
+                         "(the kernels then read the zero padding, as the reference's do)")
+    ap.add_argument("--dropout", type=float, default=0.0,
+                    help="dropout probability of the training adapters (workloads with a backward): the "
+                         "kernels regenerate the mask in the forward and the backward; default 0 = off")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a 128 MiB device copy three times before the timed region: a kernel "
+                         "of known traffic to scale FETCH_SIZE / WRITE_SIZE readings with")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; every box has one MI355X and no collective, "
+              "sharding or rank code exists in it. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
+    from loquetier_amd import _lib
+    from loquetier_amd.ops import _kernels as K
+    _lib.load()  # no fallback: raises when the HIP library is missing
+    torch.cuda.set_device(torch.device("cuda:0"))
+    if args.config == "rmsnorm":
+        return rmsnorm_bench(args, torch, K)
+    if args.config == "model-step":
+        return model_step_bench(args, torch, K)
+    probe = load_probe()
+    if args.config != "all":
+        print(json.dumps(run_workload(args, args.config, torch, K, probe)), flush=True)
+        return
+    # the headline: BASELINE.json's configs[1]; the other GPU workloads ride along in brief
+    out = run_workload(args, "cfg2", torch, K, probe)
+    if not args.step_only:
+        out["configs"] = {}
+        for cfg in ("cfg3", "cfg4", "cfg5"):
+            o = run_workload(args, cfg, torch, K, probe, brief=True)
+            out["configs"][cfg] = {k: o[k] for k in ("value", "unit", "ms_per_step", "ms_per_step_plan_reused",
+                                                     "dtype", "step_algorithmic_bytes", "step_hbm_gbps",
+                                                     "step_frac_of_8TBps", "roofline", "launches", "cpu_baseline")}
+            out["configs"][cfg]["workload"] = o["config"]["workload"]
     print(json.dumps(out), flush=True)
 
 

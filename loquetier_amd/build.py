@@ -13,8 +13,12 @@ REPO_DIR = os.path.dirname(PKG_DIR)
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libsmlm_hip.so")
-SOURCES = ["smlm_api.hip"]
-HEADERS = ["smlm_common.hpp", "smlm_plan.hpp", "smlm_forward.hpp", "smlm_backward.hpp"]
+PROBE_PATH = os.path.join(LIB_DIR, "libsmlm_probe.so")
+# library -> its translation units (headers are found through -I csrc)
+LIBRARIES = {
+    LIB_PATH: ["smlm_api.hip"],        # the operator library (include/smlm.h)
+    PROBE_PATH: ["stream_probe.hip"],  # plain streaming kernels bench.py calibrates against
+}
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
@@ -30,11 +34,9 @@ def hipcc_path() -> str:
     return "hipcc"
 
 
-def build_library(verbose: bool = False) -> str:
-    """Compile every HIP source into loquetier_amd/lib/libsmlm_hip.so (always recompiles)."""
-    os.makedirs(LIB_DIR, exist_ok=True)
+def _compile(out: str, sources, verbose: bool) -> None:
     cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC_DIR,
-           *[os.path.join(CSRC_DIR, s) for s in SOURCES], "-o", LIB_PATH + ".tmp"]
+           *[os.path.join(CSRC_DIR, s) for s in sources], "-o", out + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -44,7 +46,15 @@ def build_library(verbose: bool = False) -> str:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     if err.strip() and verbose:
         print(err, file=sys.stderr)
-    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    os.replace(out + ".tmp", out)
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile every HIP source into loquetier_amd/lib/ (always recompiles); returns the path of
+    the operator library."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    for out, sources in LIBRARIES.items():
+        _compile(out, sources, verbose)
     return LIB_PATH
 
 

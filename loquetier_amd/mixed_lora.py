@@ -11,6 +11,7 @@ of separate tensor ops (same operator calls, same rounding points).
 """
 from __future__ import annotations
 
+from contextlib import contextmanager
 from dataclasses import dataclass
 from typing import Any, List, Optional, Sequence, Union
 
@@ -147,6 +148,23 @@ class MixedLoraContext:
         return self.memo(("part_segments", device), build)
 
 
+# Adapter whose parameters a state_dict() call saves (reference: CURRENT_TRAINER_LORA_ID and
+# set_saving_lora_id, mixed_lora.py:66-76).
+CURRENT_TRAINER_LORA_ID = 0
+
+
+@contextmanager
+def set_saving_lora_id(num: int):
+    """Within the block, state_dict() of every MixedLoraLinear saves adapter `num`."""
+    global CURRENT_TRAINER_LORA_ID
+    original_lora_id = CURRENT_TRAINER_LORA_ID
+    CURRENT_TRAINER_LORA_ID = num
+    try:
+        yield
+    finally:
+        CURRENT_TRAINER_LORA_ID = original_lora_id
+
+
 @dataclass
 class NamedLoraLayer:
     adapter_name: str
@@ -225,10 +243,12 @@ class fused_add_lora(Function):
                 starts = torch.tensor([int(t) for t in train_partition][: ctx.n_parts],
                                       dtype=torch.int32, device=x.device)
                 seg_of = (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, plan.S - 1)
+            # (gathers of one step's tensors are shared by the layers that use the same tensors)
+            gather = (lambda t: step.gather(t, seg_of)) if step is not None else (lambda t: t[seg_of].contiguous())
             if seg_scale is not None:
-                ctx.part_scale = seg_scale[seg_of].contiguous()
+                ctx.part_scale = gather(seg_scale)
             if dropout is not None:  # the same stream, probabilities by train partition
-                ctx.part_drop = kernel.DropoutSpec(dropout.seg_p[seg_of].contiguous(), train_len,
+                ctx.part_drop = kernel.DropoutSpec(gather(dropout.seg_p), train_len,
                                                    dropout.seed, dropout.offset, dropout.mask_bits)
         if need_v:
             ctx.save_for_backward(x[:train_len, ...], v[:train_len, ...], *weights)
@@ -258,6 +278,12 @@ class LayerStep:
     b_tab: Optional[torch.Tensor] = None
     grad_offsets: Optional[torch.Tensor] = None    # byte offsets of dA_0.., dB_0.. inside one gradient buffer
     grad_shapes: Optional[list] = None             # [(offset in elements, shape)] in the same order
+    memo: Any = None                               # the context's per-step memo (MixedLoraContext.memo)
+
+    def gather(self, table: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+        """table[index], computed once per step for a given pair of tensors."""
+        build = lambda: table[index].contiguous()
+        return build() if self.memo is None else self.memo(("gather", id(table), id(index)), build)
 
 
 class MixedLoraLinear(nn.Module):
@@ -394,7 +420,7 @@ class MixedLoraLinear(nn.Module):
             if not x.is_contiguous():
                 x = x.contiguous()
             plan = ctx.plan(self.device, x.size(0))
-            step = LayerStep(workspace=ctx.workspace(self.device))
+            step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo)
             if weights and blen.tlen > 0:
                 step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
                 step.part_segments = ctx.part_segments(self.device, plan)
@@ -415,3 +441,20 @@ class MixedLoraLinear(nn.Module):
                                                           ctx.lora_len).unsqueeze(-1)
         result = result + lora_res
         return result.to(torch_result_dtype)
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        """LoRA-only state dict of ONE adapter under PEFT's names: the parameters `lora-{idx}-A` /
+        `lora-{idx}-B` of the adapter selected with set_saving_lora_id are saved as
+        `lora_A.weight` / `lora_B.weight`, other adapters' parameters are left out
+        (reference: mixed_lora.py:220-234).  The base layer is a plain attribute, not a
+        submodule's parameter of this module, so its weights are saved by whoever owns it."""
+        for name, param in self._parameters.items():
+            lora_info = name.split('-')
+            if len(lora_info) != 3 or param is None:
+                continue
+            lora_id, a_b = int(lora_info[1]), lora_info[2]
+            if lora_id == CURRENT_TRAINER_LORA_ID:
+                destination[prefix + 'lora_' + a_b + '.weight'] = param if keep_vars else param.detach()
+        for name, buf in self._buffers.items():
+            if buf is not None and name not in self._non_persistent_buffers_set:
+                destination[prefix + name] = buf if keep_vars else buf.detach()

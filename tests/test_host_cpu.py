@@ -197,3 +197,34 @@ def test_dropout_entry_points_validate_like_their_plain_forms(lib):
                                                   64, k.get("r", 8), 1, None, dr, None)
     assert bwd(ctypes.byref(opts)) == -1
     assert bwd(None, r=12) == -3 and bwd(None, ws=16) == -4
+
+
+def test_layer_state_dict_saves_one_adapter_under_peft_names():
+    """MixedLoraLinear._save_to_state_dict (reference mixed_lora.py:220-234): only the adapter chosen
+    with set_saving_lora_id is saved, renamed lora-{idx}-A -> lora_A.weight."""
+    import torch
+    from loquetier_amd import mixed_lora as ml
+
+    class Base(torch.nn.Module):  # a CPU stand-in: construction and state_dict launch no kernel
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.zeros(8, 16), requires_grad=False)
+
+    adapters = [ml.NamedLoraLayer(f"a{i}", torch.full((8, 16), float(i)), torch.full((8, 8), 10.0 + i),
+                                  torch.nn.Identity(), 2.0) for i in range(3)]
+    layer = ml.MixedLoraLinear(ml.MixedLoraContext(), Base(), adapters, 8, torch.float32, is_scaled=False)
+    layer.set_trainable([0, 2])
+    assert sorted(n for n, _ in layer.named_parameters() if n.startswith("lora-")) == \
+        ["lora-0-A", "lora-0-B", "lora-2-A", "lora-2-B"]
+    sd = {k: v for k, v in layer.state_dict().items() if k.startswith("lora_")}
+    assert sorted(sd) == ["lora_A.weight", "lora_B.weight"] and float(sd["lora_A.weight"][0, 0]) == 0.0
+    with ml.set_saving_lora_id(2):
+        sd2 = {k: v for k, v in layer.state_dict(prefix="m.").items() if "lora_" in k}
+    assert sorted(sd2) == ["m.lora_A.weight", "m.lora_B.weight"]
+    assert float(sd2["m.lora_A.weight"][0, 0]) == 2.0 and float(sd2["m.lora_B.weight"][0, 0]) == 12.0
+    assert not sd2["m.lora_A.weight"].requires_grad          # detached unless keep_vars
+    assert ml.CURRENT_TRAINER_LORA_ID == 0                   # restored on exit
+    with ml.set_saving_lora_id(1):                           # adapter 1 does not train here: nothing saved
+        assert not [k for k in layer.state_dict() if k.startswith("lora_")]
+    # the parameters share the adapters' storage (mixed_lora.py:168-171): an optimizer step moves no address
+    assert layer.get_parameter("lora-2-A").data_ptr() == adapters[2].wa.data_ptr()
