@@ -779,12 +779,17 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 template <int DT, int NQ, int KS, bool DIRECT, bool WKN, bool DROP = false>
 // (five workgroups a CU instead of the four the compiler's own register budget gives: more y
 // lines in flight per CU; worth 2 % on the prefill launch and 6 % on the fine-tune one)
-__global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(DIRECT && KS == 1 ? 5 : 1)))
+__global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(DIRECT ? 5 : 1)))
 void expand_block_kernel(ExpandArgs a) {
   static_assert(NQ % 2 == 0, "the output is written 64 columns at a time");
   constexpr int kPitch = WKN ? 32 * NQ + 8 : 32 * KS + 8;  // LDS row pitch in 16-bit elements
-  __shared__ __attribute__((aligned(16))) uint16_t wlds[(WKN ? 32 * KS : 32 * NQ) * kPitch];
-  __shared__ __attribute__((aligned(16))) float olds[kFwdWaves][kTileRows * kOPitch];
+  // the staged weights and the area the accumulators change layout in share their LDS (the
+  // weights are done with when the accumulators are complete): five workgroups fit a CU at rank 64 too
+  constexpr int kWBytes = (WKN ? 32 * KS : 32 * NQ) * kPitch * 2;
+  constexpr int kOBytes = kFwdWaves * kTileRows * kOPitch * 4;
+  __shared__ __attribute__((aligned(16))) char smem[kWBytes > kOBytes ? kWBytes : kOBytes];
+  uint16_t* wlds = reinterpret_cast<uint16_t*>(smem);
+  float(*olds)[kTileRows * kOPitch] = reinterpret_cast<float(*)[kTileRows * kOPitch]>(smem);
   const int units = DIRECT ? 0 : tile_units<kBlkTiles>(a.plan, 0);
   const WorkRange wr = item_range<DIRECT>(a.items, units);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -869,11 +874,11 @@ void expand_block_kernel(ExpandArgs a) {
       if (idx < kPieces) *reinterpret_cast<u32x4*>(&wlds[r_ * kPitch + c_]) = stage[j];
     }
     __syncthreads();
-    if (!active) continue;  // whole waves only (MFMA runs with every lane); barriers are behind us
-
     f32x4 acc[NQ][2];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) acc[q][0] = acc[q][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // (waves without a tile multiply zeros: whole waves only, MFMA runs with every lane, and every
+    // wave reaches the barrier below)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -893,7 +898,8 @@ void expand_block_kernel(ExpandArgs a) {
           acc[q][p] = Num<DT>::mfma(wf, vf[ks], acc[q][p]);
         }
 
-    store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
+    __syncthreads();  // every wave has read its weights: the area is free for the accumulators
+    if (active) store_y_lines<DT, NQ, DROP>(olds[wave], acc, yold, L, c, g, ncol0, P.d_out, a.beta);
   }
 }
 
