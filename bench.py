@@ -395,6 +395,8 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         return (torch.randn(*shape, generator=gen) * std).to(dev).to(tdt)
 
     ranks = w.get("true_ranks")
+    # adapters below the launch's rank (cfg5) are stored at their own rank unless asked otherwise
+    packed = bool(ranks) and not args.padded_ranks and not args.padded_storage
     sets = []
     for _ in range(R):
         projs = []
@@ -405,21 +407,22 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                 for a in range(NA):
                     A[a, ranks[a % 4]:] = 0
                     B[a, :, ranks[a % 4]:] = 0
-            d = dict(x=randn(T, hi), y=randn(T, ho), A=A, B=B,
-                     a_tab=torch.tensor([A[a].data_ptr() for a in range(NA)], dtype=torch.int64, device=dev),
-                     b_tab=torch.tensor([B[a].data_ptr() for a in range(NA)], dtype=torch.int64, device=dev))
+            Aw, Bw = [A[a] for a in range(NA)], [B[a] for a in range(NA)]
+            if packed:  # every adapter stored at its own rank: what prepare_weight(pack=True) produces
+                Aw = [A[a, :ranks[a % 4]].contiguous() for a in range(NA)]
+                Bw = [B[a, :, :ranks[a % 4]].contiguous() for a in range(NA)]
+            d = dict(x=randn(T, hi), y=randn(T, ho), A=Aw, B=Bw,
+                     a_tab=torch.tensor([w_.data_ptr() for w_ in Aw], dtype=torch.int64, device=dev),
+                     b_tab=torch.tensor([w_.data_ptr() for w_ in Bw], dtype=torch.int64, device=dev))
             if P:
                 train = sorted(set(w["ids"][:P]))
                 d.update(g=randn(n_train, ho), dx=torch.empty(n_train, hi, dtype=tdt, device=dev),
                          v=torch.empty(T, r, dtype=tdt, device=dev),
-                         dA=torch.empty(len(train), r, hi, dtype=tdt, device=dev),
-                         dB=torch.empty(len(train), ho, r, dtype=tdt, device=dev))
-                d["ta_tab"] = torch.tensor([A[a].data_ptr() for a in train], dtype=torch.int64, device=dev)
-                d["tb_tab"] = torch.tensor([B[a].data_ptr() for a in train], dtype=torch.int64, device=dev)
-                d["da_tab"] = torch.tensor([d["dA"][i].data_ptr() for i in range(len(train))],
-                                           dtype=torch.int64, device=dev)
-                d["db_tab"] = torch.tensor([d["dB"][i].data_ptr() for i in range(len(train))],
-                                           dtype=torch.int64, device=dev)
+                         dA=[torch.empty_like(Aw[a]) for a in train], dB=[torch.empty_like(Bw[a]) for a in train])
+                d["ta_tab"] = torch.tensor([Aw[a].data_ptr() for a in train], dtype=torch.int64, device=dev)
+                d["tb_tab"] = torch.tensor([Bw[a].data_ptr() for a in train], dtype=torch.int64, device=dev)
+                d["da_tab"] = torch.tensor([t_.data_ptr() for t_ in d["dA"]], dtype=torch.int64, device=dev)
+                d["db_tab"] = torch.tensor([t_.data_ptr() for t_ in d["dB"]], dtype=torch.int64, device=dev)
             projs.append(d)
         sets.append(dict(proj=projs,
                          plan_buf=torch.empty(K.SegmentPlan.nbytes(T, S), dtype=torch.uint8, device=dev),
@@ -453,7 +456,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
                                   [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
                                   v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f,
-                                  adapter_rank=rank_f)
+                                  adapter_rank=rank_f, packed_ranks=packed)
 
     def step(st, build_plan=True):
         if build_plan:
@@ -466,7 +469,8 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
             for i, d in enumerate(st["proj"]):
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
                                      d["ta_tab"], d["tb_tab"], bplan, r, part_scale,
-                                     dropout=drop_b[i] if drop_b else None, adapter_rank=rank_b)
+                                     dropout=drop_b[i] if drop_b else None, adapter_rank=rank_b,
+                                     packed_ranks=packed)
 
     # eager once on the capture stream (sizes its workspace outside any capture)
     cap_stream = torch.cuda.Stream()
@@ -656,7 +660,8 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                    "buffer_sets_rotated": R, "step_includes": "plan build + fused forward per projection"
                    + (" + backward" if P else ""), "graph_replay": not args.eager,
                    "dropout": args.dropout if P else 0.0,
-                   "true_ranks_passed": bool(ranks and not args.padded_ranks)},
+                   "true_ranks_passed": bool(ranks and not args.padded_ranks),
+                   "adapters_stored_at_true_rank": packed},
         "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
         "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
@@ -689,6 +694,9 @@ def main():
     ap.add_argument("--padded-ranks", action="store_true",
                     help="workloads with adapters below the padded rank: do not pass the true ranks "
                          "(the kernels then read the zero padding, as the reference's do)")
+    ap.add_argument("--padded-storage", action="store_true",
+                    help="workloads with adapters below the padded rank: pass the true ranks but keep the "
+                         "adapters zero-padded in memory (default: stored at their own rank, packed)")
     ap.add_argument("--dropout", type=float, default=0.0,
                     help="dropout probability of the training adapters (workloads with a backward): the "
                          "kernels regenerate the mask in the forward and the backward; default 0 = off")

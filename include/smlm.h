@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SMLM_ABI_VERSION 1
+#define SMLM_ABI_VERSION 2
 
 #if defined(__GNUC__)
 #define SMLM_API __attribute__((visibility("default")))
@@ -256,10 +256,17 @@ typedef struct smlm_dropout {
  *                  the kernels do not read the padding (rows of A, columns of B and of v
  *                  at or past the rank rounded up to 8) and treat it as the zeros it
  *                  holds, so results equal the padded computation bit for bit.
+ *   packed_ranks : non-zero (with adapter_rank): the weights are STORED at their true rank
+ *                  rounded up to 8, A_a [r_a, h_in] and B_a [h_out, r_a] contiguous, instead of
+ *                  zero-padded to r; the backward writes dA_a / dB_a in the same shapes.  A
+ *                  rank-8 adapter beside rank-64 ones then costs 16 bytes of B per output
+ *                  column instead of a 128-byte line.  Results equal the padded computation
+ *                  bit for bit; v, dV and the workspace keep the launch's rank r.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;
   const int32_t* adapter_rank;
+  int packed_ranks;
 } smlm_lora_opts;
 
 /* smlm_lora_fwd_multi with options. */

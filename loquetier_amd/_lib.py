@@ -32,7 +32,7 @@ class Dropout(C.Structure):
 
 class LoraOpts(C.Structure):
     """struct smlm_lora_opts of include/smlm.h."""
-    _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p)]
+    _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p), ("packed_ranks", C.c_int)]
 
 
 _popts = C.POINTER(LoraOpts)

@@ -322,13 +322,14 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
                const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false,
-               const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr) {
+               const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr, int packed = 0) {
   if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
   ShrinkArgs a{};
   if (drop) a.drop = *drop;
   a.w_kn = w_kn ? 1 : 0;
   a.plan = tile_args(pv);
   a.plan.w_rank = w_rank;  // the output columns are the rank
+  a.plan.packed = packed;
   a.seg_scale = seg_scale;
   a.beta = beta;
   a.T = T;
@@ -647,6 +648,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   DropArgs drop;
   if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
+  const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
   if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
     return SMLM_ERR_ARG;
   if (stages < 1 || stages > (SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND)) return SMLM_ERR_ARG;
@@ -695,7 +697,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   }
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                    0.0f, nullptr, st, !expand_folds, false, &drop, w_rank);
+                    0.0f, nullptr, st, !expand_folds, false, &drop, w_rank, packed);
     if (rc) return rc;
   }
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;
@@ -703,6 +705,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   ExpandArgs ea{};
   ea.plan = tile_args(pv);
   ea.plan.w_rank = w_rank;
+  ea.plan.packed = packed;
   ea.seg_scale = seg_scale;
   ea.beta = beta;
   ea.T = T; ea.nt_max = pv.nt_max;
@@ -766,6 +769,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   DropArgs drop;
   if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
+  const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
   if (NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
   if ((h_in & 7) || (h_out & 7) || (r & 7)) return SMLM_ERR_ALIGN;
   if (NA == 0 || n_rows == 0 || P == 0) return SMLM_ERR_ARG;
@@ -802,6 +806,8 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
     ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
     ta.set[1] = TransposeSet{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
     ta.NA = NA;
+    ta.w_rank = w_rank;
+    ta.packed = packed;
     const int gx = ceil_div(h_in > h_out ? h_in : h_out, 64), gy = ceil_div(r, 64);
     if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
   }
@@ -832,8 +838,8 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   const void* const* btp = in_place ? b_ptrs : bt_ptrs;
   const int b_ld = in_place ? r : h_out;
   if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
-                       0.0f, nullptr, st, true, in_place, nullptr, w_rank)))
-    return rc;
+                       0.0f, nullptr, st, true, in_place, nullptr, w_rank, in_place ? packed : 0)))
+    return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
   ExpandArgs ea{};
@@ -875,6 +881,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   wa.chunks_a = ceil_div(h_in, kWgCols);
   wa.grp_seg = pv.grp_seg;
   wa.w_rank = w_rank;
+  wa.packed = packed;
   wa.drop = drop;  // dA against the dropped x
   // ranks above 64 are covered 64 at a time along the grid's z axis
   dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA, ceil_div(r, 64));

@@ -21,6 +21,8 @@ struct TransposeSet {
 struct TransposeArgs {
   TransposeSet set[2];  // A [r, h_in] -> At [h_in, r] and B [h_out, r] -> Bt [r, h_out]
   int NA;
+  const int32_t* w_rank;  // optional [NA] with packed: the sources are stored at their true rank (rounded up
+  int packed;             //   to 8), A_a [r_a, h_in], B_a [h_out, r_a]; the copies keep the full-rank strides
 };
 
 constexpr int kTrPitch = 80;  // LDS row pitch in 16-bit elements (40 banks: see kWgPitch)
@@ -33,12 +35,19 @@ constexpr int kTrPitch = 80;  // LDS row pitch in 16-bit elements (40 banks: see
 __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t t[64 * kTrPitch];
   const int which = blockIdx.z / a.NA, ad = blockIdx.z - which * a.NA;
-  const TransposeSet S = a.set[which];
+  TransposeSet S = a.set[which];
+  if (a.w_rank && a.packed) {  // the rank is A's row count and B's column count
+    const int full = which == 0 ? S.rows : S.cols;
+    const int r8 = (uload(a.w_rank, ad) + 7) & ~7;
+    const int ra = r8 < full ? r8 : full;
+    if (which == 0) S.rows = ra; else S.cols = ra;
+  }
   const int c0 = (which == 0 ? blockIdx.x : blockIdx.y) * 64;
   const int r0 = (which == 0 ? blockIdx.y : blockIdx.x) * 64;
   if (c0 >= S.cols || r0 >= S.rows) return;  // uniform over the workgroup
   const uint16_t* src = reinterpret_cast<const uint16_t*>(S.src_ptrs[ad]);
   uint16_t* dst = S.dst_base + (long)ad * S.stride;
+  const int dst_pitch = a.set[which].rows;  // the copy is [cols, rows] of the full-rank shape
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) S.dst_ptrs[ad] = dst;
   const u32x4 zero = {0u, 0u, 0u, 0u};
   // in: lane -> (row = tid / 8 (+32), 8 columns at (tid % 8) * 8)
@@ -65,7 +74,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
     const uint16_t* p0 = &t[(rb + (i >> 2)) * kTrPitch + 16 * wave + 4 * (i & 3)];
     const u32x2 q0 = lds_read_tr16(p0), q1 = lds_read_tr16(p0 + 4 * kTrPitch);
     const int oc = c0 + 16 * wave + i, orow = r0 + rb;
-    if (oc < S.cols && orow < S.rows) stg16(dst + (long)oc * S.rows + orow, u32x4{q0[0], q0[1], q1[0], q1[1]});
+    if (oc < S.cols && orow < S.rows) stg16(dst + (long)oc * dst_pitch + orow, u32x4{q0[0], q0[1], q1[0], q1[1]});
   }
 }
 
@@ -83,6 +92,7 @@ struct WgradArgs {
   long pitch;
   int h_in, h_out, r, chunks_a;  // chunks_a = ceil(h_in/64): blockIdx.x below it works on dA
   const int32_t* w_rank;   // optional [NA]: true rank of each adapter (rows of dV / v past it are zero padding)
+  int packed;              // with w_rank: dA_a [r_a, h_in] and dB_a [h_out, r_a] are stored at the true rank
   const int32_t* grp_seg;  // DROP kernels: first segment of every group (its adapter's dropout probability)
   DropArgs drop;           // DROP kernels: dA is taken against the dropped x, regenerated while x is staged
 };
@@ -338,7 +348,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int j = j0 + 16 * jb + orow + 8 * i, n = n0 + ocol;
-        if (j < a.r && n < h) stg16_nt(out + (long)j * h + n, o[i]);
+        if (j < (a.packed ? rlim : a.r) && n < h) stg16_nt(out + (long)j * h + n, o[i]);
       }
     }
   } else {
@@ -356,7 +366,8 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int n = n0 + 16 * nb + orow + 8 * i;
-        if (j0 + ocol < a.r && n < h) stg16_nt(out + (long)n * a.r + j0 + ocol, o[i]);
+        const int ldb = a.packed ? rlim : a.r;  // columns of dB as it is stored
+        if (j0 + ocol < ldb && n < h) stg16_nt(out + (long)n * ldb + j0 + ocol, o[i]);
       }
     }
   }

@@ -38,6 +38,8 @@ struct TileArgs {
   const int32_t* tile_wid;
   const int32_t* blk;        // (first tile << 3) | tile count, per tile block
   const int32_t* w_rank;     // optional, indexed like the weight tables: true rank of each adapter
+  int packed;                // with w_rank: the weights are STORED at their true rank (rounded up to 8),
+                             //   A_a [r_a, h_in], B_a [h_out, r_a], instead of zero-padded to the launch's rank
 };
 
 // Adapters of different ranks live zero-padded to one rank (the reference pads every adapter
@@ -48,6 +50,13 @@ __device__ __forceinline__ int rank_limit(const TileArgs& p, int wid, int d) {
   if (!p.w_rank) return d;
   const int r = (uload(p.w_rank, wid) + 7) & ~7;
   return r < d ? r : d;
+}
+// Leading dimension of a weight matrix whose contiguous dimension is the rank (B [h_out, r], read
+// by the expand and by the backward's dV product): the launch's rank for zero-padded storage, the
+// adapter's own (rank_limit) for packed storage -- a rank-8 adapter beside rank-64 ones then costs
+// 16 bytes a row instead of a 128-byte line.
+__device__ __forceinline__ int rank_ld(const TileArgs& p, int ld, int lim) {
+  return (p.w_rank && p.packed) ? lim : ld;
 }
 
 // Items [first, last) of this workgroup, visited with stride `step`.  The grid
@@ -349,6 +358,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
     const int row = active ? a.plan.tile_row[slot] : -1;
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int nlim = rank_limit(a.plan, wid, P.d_out);  // weight rows at or past it are zero padding
+    const int ldw = WKN ? rank_ld(a.plan, P.ldw, nlim) : P.ldw;  // [k][n] weights (B) have the rank contiguous
     const int kbeg = kz * kFwdWaves * P.k_per_wave;
     const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
     const uint16_t* xrow = P.x + (long)(row < 0 ? 0 : row) * P.d_in;
@@ -369,11 +379,11 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
         const int idx = threadIdx.x + j * kFwdThreads;
         if (WKN) {
           const int kl = idx / (kRowsW / 8), n8 = (idx % (kRowsW / 8)) * 8;
-          st[j] = ldg16_or(W + (long)(kb + kl) * P.ldw + n0 + n8,
+          st[j] = ldg16_or(W + (long)(kb + kl) * ldw + n0 + n8,
                            idx < kPieces && n0 + n8 < nlim && kb + kl < kend, zeros);
         } else {
           const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
-          st[j] = ldg16_or(W + (long)(n0 + nl) * P.ldw + kb + k8,
+          st[j] = ldg16_or(W + (long)(n0 + nl) * ldw + kb + k8,
                            idx < kPieces && n0 + nl < nlim && kb + k8 < kend, zeros);
         }
       }
@@ -694,6 +704,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     if (wid < 0) continue;  // past the last tile (direct mode)
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
+    const int ldw = ROWMAJOR ? P.ldw : rank_ld(a.plan, P.ldw, klim);
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
     const int rseg = a.seg_scale ? a.plan.tile_rseg[slot] : -1;  // -1 on empty slots too
@@ -737,7 +748,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           const int n = ncol0 + 32 * q + 4 * p + mrow;
-          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, P.ldw, kreal && n < P.d_out, zeros);
+          wf[q][p] = load_w8<ROWMAJOR>(W, n, kk, ldw, kreal && n < P.d_out, zeros);
         }
       u32x4 vf;
       const bool vok = kreal && row >= 0;
@@ -807,6 +818,7 @@ void expand_block_kernel(ExpandArgs a) {
     const int wid = uload(a.plan.tile_wid, t0);
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
+    const int ldw = WKN ? P.ldw : rank_ld(a.plan, P.ldw, klim);  // [k][n] weights (A) have whole rows per rank
     const bool active = wave < cnt;
     const int tslot = (t0 + (active ? wave : 0)) * kTileRows;
     const int slot = tslot + c;
@@ -836,11 +848,11 @@ void expand_block_kernel(ExpandArgs a) {
       const int idx = threadIdx.x + j * kFwdThreads;
       if (WKN) {
         const int kl = idx / (4 * NQ), n8 = (idx % (4 * NQ)) * 8;
-        stage[j] = ldg16_or(W + (long)kl * P.ldw + ncol0 + n8,
+        stage[j] = ldg16_or(W + (long)kl * ldw + ncol0 + n8,
                             idx < kPieces && ncol0 + n8 < P.d_out && kl < klim, zeros);
       } else {
         const int nl = idx / (4 * KS), k8 = (idx % (4 * KS)) * 8;
-        stage[j] = ldg16_or(W + (long)(ncol0 + nl) * P.ldw + k8,
+        stage[j] = ldg16_or(W + (long)(ncol0 + nl) * ldw + k8,
                             idx < kPieces && ncol0 + nl < P.d_out && k8 < klim, zeros);
       }
     }

@@ -138,7 +138,8 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
             g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
             kernel.smlm_lora_backward(grad_x, tabs[:NA], tabs[NA:], g, x_train, v_train, step.a_tab, step.b_tab,
                                       step.bwd_plan, lora_rank, part_scale, dropout=dropout,
-                                      adapter_rank=adapter_rank, workspace=step.workspace)
+                                      adapter_rank=adapter_rank, workspace=step.workspace,
+                                      packed_ranks=step.packed)
         else:
             buf.zero_()
     else:
@@ -154,7 +155,8 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
                 grad_x, _ptr_table(da, dev), _ptr_table(db, dev), g, x_train, v_train,
                 _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
                 plan, lora_rank, part_scale, dropout=dropout, adapter_rank=adapter_rank,
-                workspace=None if step is None else step.workspace)
+                workspace=None if step is None else step.workspace,
+                packed_ranks=step is not None and step.packed)
         else:
             for t in da + db:
                 t.zero_()

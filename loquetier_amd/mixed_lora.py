@@ -178,15 +178,20 @@ class NamedLoraLayer:
 
 
 def prepare_weight(weight: torch.Tensor, rank: int, dtype: torch.dtype, device, rank_dim: int = 0,
-                   scaling: Optional[float] = None) -> torch.Tensor:
+                   scaling: Optional[float] = None, pack: bool = False) -> torch.Tensor:
     """Cast, optionally pre-scale, and zero-pad a LoRA weight to the layer rank
-    (reference: MixedLoraModel._prepare_weight, mixed_lora.py:501-521)."""
+    (reference: MixedLoraModel._prepare_weight, mixed_lora.py:501-521).
+
+    pack=True pads only to the next multiple of 8 instead of the layer rank: the adapter is then
+    stored at its own rank (A [r_a, h_in], B [h_out, r_a]) and the fused kernels read it so
+    (`packed_ranks`); results are those of the padded storage, bit for bit."""
     weight = weight.detach()
-    if weight.size(rank_dim) == rank:
+    target = min(rank, (weight.size(rank_dim) + 7) // 8 * 8) if pack else rank
+    if weight.size(rank_dim) == target:
         w = weight if scaling is None else weight * scaling
         return w.to(dtype=dtype, device=device).contiguous()
     new_size = list(weight.size())
-    new_size[rank_dim] = rank
+    new_size[rank_dim] = target
     new_weight = torch.zeros(new_size, dtype=dtype, device=device)
     src = weight if scaling is None else weight * scaling
     new_weight[: weight.size(0), : weight.size(1)].copy_(src, non_blocking=True)
@@ -224,7 +229,8 @@ class fused_add_lora(Function):
             dropout = kernel.DropoutSpec(dropout.seg_p, dropout.rows, dropout.seed, dropout.offset, bits)
         kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
                                  beta=1.0, v_out=v, dropout=dropout, adapter_rank=adapter_rank,
-                                 workspace=None if step is None else step.workspace)
+                                 workspace=None if step is None else step.workspace,
+                                 packed_ranks=step is not None and step.packed)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
@@ -279,6 +285,7 @@ class LayerStep:
     grad_offsets: Optional[torch.Tensor] = None    # byte offsets of dA_0.., dB_0.. inside one gradient buffer
     grad_shapes: Optional[list] = None             # [(offset in elements, shape)] in the same order
     memo: Any = None                               # the context's per-step memo (MixedLoraContext.memo)
+    packed: bool = False                           # the adapters are stored at their true ranks
 
     def gather(self, table: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
         """table[index], computed once per step for a given pair of tensors."""
@@ -313,9 +320,20 @@ class MixedLoraLinear(nn.Module):
         if not self.is_scaled:
             self.scaling = torch.tensor([a.scaling for a in adapters], dtype=self.dtype,
                                         device=self.device)
-        ranks = [rank if a.true_rank is None else min(int(a.true_rank), rank) for a in adapters]
+        # adapters stored at their own rank (prepare_weight(pack=True)): every one must be, consistently
+        self.packed = any(a.wa.size(0) < rank or a.wb.size(1) < rank for a in adapters)
+        ranks = []
+        for a in adapters:
+            stored = a.wa.size(0)
+            q = min(int(a.true_rank), rank) if a.true_rank is not None else min(stored, rank)
+            if self.packed and not (stored == a.wb.size(1) == min(rank, (q + 7) // 8 * 8)):
+                raise RuntimeError(f"adapter {a.adapter_name}: packed storage needs A [r8, h_in] and B [h_out, r8] "
+                                   f"with r8 = true rank rounded up to 8; got {tuple(a.wa.shape)}, {tuple(a.wb.shape)}")
+            ranks.append(q)
+        if self.packed and not self.fused:
+            raise RuntimeError("adapters stored at their true rank need the fused path")
         self.adapter_rank = (torch.tensor(ranks, dtype=torch.int32, device=self.device)
-                             if any(q < rank for q in ranks) else None)
+                             if self.packed or any(q < rank for q in ranks) else None)
         self._train_rank_key, self._train_rank = None, None
         self._scaling_f32 = None if self.is_scaled else self.scaling.float()
         self._scaling_key = None if self.is_scaled else tuple(float(a.scaling) for a in adapters)
@@ -420,7 +438,7 @@ class MixedLoraLinear(nn.Module):
             if not x.is_contiguous():
                 x = x.contiguous()
             plan = ctx.plan(self.device, x.size(0))
-            step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo)
+            step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed)
             if weights and blen.tlen > 0:
                 step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
                 step.part_segments = ctx.part_segments(self.device, plan)

@@ -303,9 +303,11 @@ class DropoutSpec:
 
 
 def _opts(plan: SegmentPlan, dropout: Optional["DropoutSpec"], widths, adapter_rank: Optional[torch.Tensor],
-          n_weights: int):
+          n_weights: int, packed_ranks: bool = False):
     """struct smlm_lora_opts for a call (None when there is nothing to say).  The returned
     object keeps the dropout struct alive."""
+    if packed_ranks and adapter_rank is None:
+        raise RuntimeError("packed_ranks needs adapter_rank: the kernels must know each adapter's stored rank")
     if dropout is None and adapter_rank is None:
         return None
     if adapter_rank is not None:
@@ -317,6 +319,7 @@ def _opts(plan: SegmentPlan, dropout: Optional["DropoutSpec"], widths, adapter_r
         opts._drop = dropout.struct(plan, widths)
         opts.dropout = C.pointer(opts._drop)
     opts.adapter_rank = _ptr(adapter_rank)
+    opts.packed_ranks = int(bool(packed_ranks))
     return opts
 
 
@@ -325,27 +328,28 @@ def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_
                       beta: float = 0.0, v_out: Optional[torch.Tensor] = None,
                       dropout: Optional[DropoutSpec] = None,
                       adapter_rank: Optional[torch.Tensor] = None,
-                      workspace: Optional[Workspace] = None) -> None:
+                      workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
     """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call (two launches).
     a_ptrs / b_ptrs are indexed by adapter id when the plan was built from int32
     adapter ids, by segment otherwise."""
     smlm_lora_forward_multi([y], [x], [a_ptrs], [b_ptrs], plan, rank, seg_scale=seg_scale, beta=beta,
                             v_out=None if v_out is None else [v_out], dropout=dropout,
-                            adapter_rank=adapter_rank, workspace=workspace)
+                            adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks)
 
 
 def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
                             v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None,
                             adapter_rank: Optional[torch.Tensor] = None,
-                            workspace: Optional[Workspace] = None) -> None:
+                            workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
     in two launches.  Lists of equal length; entries of xs may be the same tensor.
     stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
     arguments on the same stream), 3 = both.  dropout: the training rows of x are
     dropped inside the shrink kernel; projection i uses the stream offset + i.
     adapter_rank (int32, indexed like the tables): true ranks of adapters stored
-    zero-padded to `rank`; the padding is then not read."""
+    zero-padded to `rank`; the padding is then not read.  packed_ranks: the adapters are stored
+    AT their true rank rounded up to 8 (A_a [r_a, h_in], B_a [h_out, r_a]) instead of padded."""
     n = len(ys)
     if not (1 <= n <= 8) or len(xs) != n or len(a_ptrs) != n or len(b_ptrs) != n or \
             (v_out is not None and len(v_out) != n):
@@ -377,7 +381,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
                    "smlm_lora_fwd_multi_workspace_size")
         ws = _workspace(dev, need.value, workspace)
         n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
-        opts = _opts(plan, dropout, [x.size(1) for x in xs], adapter_rank, n_weights)
+        opts = _opts(plan, dropout, [x.size(1) for x in xs], adapter_rank, n_weights, packed_ranks)
         rc = _lib.load().smlm_lora_fwd_multi_ex(
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
@@ -393,7 +397,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                        part_scale: Optional[torch.Tensor] = None,
                        dropout: Optional[DropoutSpec] = None,
                        adapter_rank: Optional[torch.Tensor] = None,
-                       workspace: Optional[Workspace] = None) -> None:
+                       workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
     forward's stream with seg_p per partition; x is the tensor before dropout."""
@@ -420,7 +424,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
         ws = _workspace(dev, need, workspace)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
-        opts = _opts(plan, dropout, h_in, adapter_rank, NA)
+        opts = _opts(plan, dropout, h_in, adapter_rank, NA, packed_ranks)
         rc = _lib.load().smlm_lora_bwd_ex(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
                                                dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
                                                b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),

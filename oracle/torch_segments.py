@@ -24,12 +24,13 @@ def add_lora_forward(x: torch.Tensor, wa: Sequence[torch.Tensor], wb: Sequence[t
                      seg_scale: Optional[Sequence[float]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """y[s_i:s_{i+1}] = beta*y + scale_i * round(x_i A_i^T) B_i^T; returns (y, v).
 
-    wa[i] is [r, h_in], wb[i] is [h_out, r] (per segment).  With beta = 0 and no
-    scale this is add_lora.forward (kernel_utils.py:102-120)."""
+    wa[i] is [r_i, h_in], wb[i] is [h_out, r_i] (per segment; the ranks may differ, v then has
+    the largest and zeros past a segment's own).  With beta = 0 and no scale this is
+    add_lora.forward (kernel_utils.py:102-120)."""
     T = x.shape[0]
     dt = x.dtype
     h_out = wb[0].shape[0]
-    r = wa[0].shape[0]
+    r = max(w.shape[0] for w in wa)
     if y is None:
         y = torch.zeros(T, h_out, dtype=dt)
     v = torch.zeros(T, r, dtype=dt)
@@ -39,7 +40,7 @@ def add_lora_forward(x: torch.Tensor, wa: Sequence[torch.Tensor], wb: Sequence[t
         if b <= a:
             continue
         vi = (xf[a:b] @ wa[i].float().t()).to(dt)
-        v[a:b] = vi
+        v[a:b, :vi.shape[1]] = vi
         yi = vi.float() @ wb[i].float().t()
         if seg_scale is not None:
             yi = yi * float(seg_scale[i])
