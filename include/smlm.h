@@ -303,7 +303,8 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
  *   rms[t] = 1 / sqrt(mean_j x[t,j]^2 + eps)   (float, kept for the backward)
  *   out[t,j] = x[t,j] * rms[t] * w[j]          (float arithmetic, rounded once)
  * out, x: [rows, cols] of `dtype`; w: [cols] of `dtype`; rms: float [rows].
- * cols a multiple of 8 (as in the reference) and at most 16384.
+ * cols a multiple of 8 (as in the reference).  Rows of up to 16384 columns stay in registers
+ * between the reduction and the scaling (read once); wider rows take a two-pass kernel.
  */
 SMLM_API int smlm_rms_norm_fwd(void* out, float* rms, const void* x, const void* w, int rows,
                                int cols, float eps, int dtype, void* stream);

@@ -282,6 +282,91 @@ __global__ __launch_bounds__(256) void rms_bwd_kernel(RmsBwdArgs a) {
   }
 }
 
+// ---- rows wider than kRmsMaxCols: the row no longer fits the registers of four waves.  Plain
+// two-pass kernels (the reference's own scheme, rms_norm_cutlass.cu:81-159): a workgroup per row
+// walks the columns once for the reduction and once more for the output (the second pass mostly
+// hits L2).  The backward keeps its share of dw in the float partial rows themselves, read and
+// written once per row it handles.  Correct for any width that is a multiple of 8; not tuned.
+__device__ __forceinline__ float block_sum_f32(float x, float* red4) {
+  x = wave_sum_f32(x);
+  __syncthreads();  // red4 is free again
+  if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = x;
+  __syncthreads();
+  return (red4[0] + red4[1]) + (red4[2] + red4[3]);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void rms_fwd_wide_kernel(RmsFwdArgs a) {
+  __shared__ float red4[4];
+  for (int row = blockIdx.x; row < a.rows; row += gridDim.x) {
+    const uint16_t* xr = a.x + (long)row * a.cols;
+    float ss = 0.0f;
+    for (int col = threadIdx.x * 8; col < a.cols; col += 256 * 8) {
+      float f[8];
+      unpack8<DT>(ldg16(xr + col), f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+    }
+    ss = block_sum_f32(ss, red4);
+    const float rms = 1.0f / sqrtf(ss / (float)a.cols + a.eps);
+    if (threadIdx.x == 0) a.rms[row] = rms;
+    uint16_t* orow = a.out + (long)row * a.cols;
+    for (int col = threadIdx.x * 8; col < a.cols; col += 256 * 8) {
+      float f[8], g[8];
+      unpack8<DT>(ldg16(xr + col), f);
+      unpack8<DT>(ldg16(a.w + col), g);
+      u32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = pack2<DT>(f[2 * e] * rms * g[2 * e], f[2 * e + 1] * rms * g[2 * e + 1]);
+      stg16_nt(orow + col, o);
+    }
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void rms_bwd_wide_kernel(RmsBwdArgs a) {
+  __shared__ float red4[4];
+  const float inv_n = 1.0f / (float)a.cols;
+  float* prow = a.partial + (long)blockIdx.x * a.cols;
+  bool first = true;
+  for (int row = blockIdx.x; row < a.rows; row += gridDim.x) {
+    const long off = (long)row * a.cols;
+    float dot = 0.0f;
+    for (int col = threadIdx.x * 8; col < a.cols; col += 256 * 8) {
+      float xf[8], gf[8], wf[8];
+      unpack8<DT>(ldg16(a.x + off + col), xf);
+      unpack8<DT>(ldg16(a.g + off + col), gf);
+      unpack8<DT>(ldg16(a.w + col), wf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot += gf[e] * wf[e] * xf[e];
+    }
+    dot = block_sum_f32(dot, red4);
+    const float rms = a.rms[row], coef = dot * rms * rms * inv_n;
+    for (int col = threadIdx.x * 8; col < a.cols; col += 256 * 8) {
+      float xf[8], gf[8], wf[8];
+      unpack8<DT>(ldg16(a.x + off + col), xf);
+      unpack8<DT>(ldg16(a.g + off + col), gf);
+      unpack8<DT>(ldg16(a.w + col), wf);
+      u32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o[e] = pack2<DT>((gf[2 * e] * wf[2 * e] - xf[2 * e] * coef) * rms,
+                         (gf[2 * e + 1] * wf[2 * e + 1] - xf[2 * e + 1] * coef) * rms);
+      stg16_nt(a.dx + off + col, o);
+      // this thread's columns of the workgroup's partial row: nobody else touches them
+      f32x4 p0 = {0.f, 0.f, 0.f, 0.f}, p1 = p0;
+      if (!first) p0 = ldg_f4(prow + col), p1 = ldg_f4(prow + col + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) p0[e] += xf[e] * rms * gf[e], p1[e] += xf[4 + e] * rms * gf[4 + e];
+      *(SMLM_GLOBAL f32x4*)(prow + col) = p0;
+      *(SMLM_GLOBAL f32x4*)(prow + col + 4) = p1;
+    }
+    first = false;
+  }
+  if (first)  // more workgroups than rows never happens (the host sizes the grid), but a partial row must not stay unwritten
+    for (int col = threadIdx.x * 4; col < a.cols; col += 256 * 4) *(SMLM_GLOBAL f32x4*)(prow + col) = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
 struct RmsFoldArgs {
   uint16_t* dw;          // [cols]
   const float* partial;  // [n_part, cols]

@@ -898,6 +898,10 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
 // backward walks four turns per workgroup (the next rows are fetched while the current ones are
 // worked on), so that its partial sums of dw stay small next to x and g
 static int rms_blocks(int rows, int cols, bool backward) {
+  if (cols > kRmsMaxCols) {  // wide rows: a workgroup per row; the backward's partial rows are whole rows of floats
+    const int cap = backward ? 128 : (1 << 22);
+    return rows < 1 ? 1 : (rows < cap ? rows : cap);
+  }
   const int rows_per_step = cols <= kRmsWaveCols ? 4 : 1;
   int nb = ceil_div(rows, rows_per_step * (backward ? tune("SMLM_TUNE_RMS_ROWS", 4) : 1));
   const int cap = backward ? tune("SMLM_TUNE_RMS_CAP", 512) : (1 << 22);
@@ -910,7 +914,7 @@ static int rms_check(int rows, int cols, int dtype) {
   if (rows < 0 || cols <= 0) return SMLM_ERR_ARG;
   if (dtype != SMLM_DTYPE_F16 && dtype != SMLM_DTYPE_BF16) return SMLM_ERR_DTYPE;
   if (cols & 7) return SMLM_ERR_ALIGN;
-  if (cols > kRmsMaxCols || rows > (1 << 30)) return SMLM_ERR_LIMIT;
+  if (cols > (1 << 24) || rows > (1 << 30)) return SMLM_ERR_LIMIT;
   return SMLM_OK;
 }
 
@@ -930,6 +934,9 @@ SMLM_API int smlm_rms_norm_fwd(void* out, float* rms, const void* x, const void*
   const int rows_per_step = cols <= kRmsWaveCols ? 4 : 1;
   const bool one_turn = (long)nb * rows_per_step >= rows;  // every workgroup sees one row group
   const dim3 bl(256);
+  if (cols > kRmsMaxCols)
+    return f16 ? launch(rms_fwd_wide_kernel<SMLM_DTYPE_F16>, grid, bl, st, a)
+               : launch(rms_fwd_wide_kernel<SMLM_DTYPE_BF16>, grid, bl, st, a);
   if (cols <= kRmsWaveCols) {
     if (one_turn)
       return f16 ? launch(rms_fwd_kernel<SMLM_DTYPE_F16, 1, true>, grid, bl, st, a)
@@ -971,7 +978,10 @@ SMLM_API int smlm_rms_norm_bwd(void* dx, void* dw, const void* g, const void* x,
                      reinterpret_cast<const uint16_t*>(w), rms, rows, cols};
   const dim3 grid((unsigned)nb);
   const dim3 bl(256);
-  if (cols <= kRmsWaveCols)
+  if (cols > kRmsMaxCols)
+    rc = f16 ? launch(rms_bwd_wide_kernel<SMLM_DTYPE_F16>, grid, bl, st, a)
+             : launch(rms_bwd_wide_kernel<SMLM_DTYPE_BF16>, grid, bl, st, a);
+  else if (cols <= kRmsWaveCols)
     rc = f16 ? launch(rms_bwd_kernel<SMLM_DTYPE_F16, 1>, grid, bl, st, a)
              : launch(rms_bwd_kernel<SMLM_DTYPE_BF16, 1>, grid, bl, st, a);
   else

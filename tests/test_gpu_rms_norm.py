@@ -51,7 +51,9 @@ def within_ulps(got, want, dt, n):
 
 
 SHAPES = [(1, 8), (3, 64), (4, 4096), (5, 4096), (257, 4096), (33, 1000), (7, 4104), (9, 11008),
-          (130, 14336), (2, 16384), (1024, 4096)]
+          (130, 14336), (2, 16384), (1024, 4096),
+          # wider than four waves' registers hold: the two-pass kernels
+          (3, 16392), (5, 20480), (2, 32768)]
 
 
 @pytest.mark.parametrize("dt", ["fp16", "bf16"])
@@ -84,7 +86,8 @@ def test_forward_exact(K, oracle, gpu_device, dt, rows, cols):
 
 @pytest.mark.parametrize("dt", ["fp16", "bf16"])
 @pytest.mark.parametrize("rows,cols", [(1, 8), (3, 64), (4, 4096), (5, 4096), (300, 4096), (33, 1000),
-                                        (9, 11008), (70, 14336), (2, 16384), (4096, 4096)])
+                                        (9, 11008), (70, 14336), (2, 16384), (4096, 4096),
+                                        (3, 16392), (140, 20480), (2, 32768)])  # the last three: two-pass kernels
 def test_backward_gaussian(K, oracle, gpu_device, dt, rows, cols):
     rng = np.random.default_rng(rows * 7 + cols)
     x = oracle.round_to(rng.standard_normal((rows, cols)), dt)
@@ -160,9 +163,8 @@ def test_errors_and_empty(K, gpu_device):
     with pytest.raises(RuntimeError, match="CUDA tensor"):
         K.rms_norm(o.cpu(), m, x, w, 1e-6)
     L = _lib.load()
-    big = torch.zeros(1, 16392, dtype=torch.float16, device=dev)
-    assert L.smlm_rms_norm_fwd(big.data_ptr(), m.data_ptr(), big.data_ptr(), big.data_ptr(), 1, 16392, 1e-6,
-                               0, None) == -6
+    assert L.smlm_rms_norm_fwd(x.data_ptr(), m.data_ptr(), x.data_ptr(), x.data_ptr(), 1, (1 << 24) + 8, 1e-6,
+                               0, None) == -6   # refused before any launch
     empty = torch.zeros(0, 64, dtype=torch.float16, device=dev)
     K.rms_norm(torch.empty_like(empty), torch.empty(0, 1, dtype=torch.float32, device=dev), empty,
                torch.zeros(64, dtype=torch.float16, device=dev), 1e-6)  # no rows: nothing to do

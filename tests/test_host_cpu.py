@@ -102,7 +102,7 @@ def test_rms_norm_argument_validation_codes(lib):
                                           k.get("dtype", 0), None)
     assert fwd(dtype=2) == -2
     assert fwd(cols=60) == -3          # the reference refuses columns % 8 != 0 (rms_norm_cutlass.cu:166-168)
-    assert fwd(cols=16392) == -6       # beyond four waves' worth of registers per row
+    assert fwd(cols=(1 << 24) + 8) == -6   # beyond what the kernels index
     assert fwd(out=None) == -1
     assert fwd(out=p + 2) == -3
     assert fwd(rows=0) == 0            # nothing to do, no launch
