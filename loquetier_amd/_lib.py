@@ -9,8 +9,7 @@ import ctypes as C
 import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-# SMLM_HIP_LIBRARY selects another build of the same library (e.g. one made with -DSMLM_TUNING)
-LIB_PATH = os.environ.get("SMLM_HIP_LIBRARY") or os.path.join(_PKG_DIR, "lib", "libsmlm_hip.so")
+LIB_PATH = os.path.join(_PKG_DIR, "lib", "libsmlm_hip.so")
 
 SMLM_DTYPE_F16, SMLM_DTYPE_BF16 = 0, 1
 SMLM_KEY_NONE, SMLM_KEY_I32, SMLM_KEY_PTR = 0, 1, 2

@@ -4,7 +4,6 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
-#include <cstdlib>
 
 #include "rms_norm.hpp"
 #include "segments.hpp"
@@ -40,18 +39,7 @@ int launch(void (*kernel)(A), dim3 grid, dim3 block, hipStream_t st, const A& a)
 
 // ---- launch shapes: functions of (T, d_in, d_out) only, never of the
 // segmentation, so re-segmenting a batch cannot change a bit of any row. ----
-// Tuning overrides (only in builds with -DSMLM_TUNING): SMLM_TUNE_<NAME>=value.
-inline int tune(const char* name, int dflt) {
-#ifdef SMLM_TUNING
-  const char* e = getenv(name);
-  if (e && *e) return atoi(e);
-#else
-  (void)name;
-#endif
-  return dflt;
-}
-
-inline int tiles_per_wave(int T) { return tune("SMLM_TUNE_MT", T >= 1024 ? kBlkTiles : 1); }
+inline int tiles_per_wave(int T) { return T >= 1024 ? kBlkTiles : 1; }
 
 // Upper bound of the number of work units along the tile axis.  `groups` bounds
 // the number of distinct plan keys (adapters): every group ends in at most one
@@ -72,7 +60,7 @@ constexpr int kMaxGridY = 65535;  // tile units are the y axis of a direct launc
 // persistent 1-D grid: a multiple of the XCD count, no larger than the work bound
 constexpr int kMaxGrid = 2048;
 inline dim3 work_grid(long bound) {
-  const long cap = tune("SMLM_TUNE_GRID", kMaxGrid);
+  const long cap = kMaxGrid;
   long g = bound < cap ? bound : cap;
   g = (g + kNumXcd - 1) / kNumXcd * kNumXcd;
   return dim3((unsigned)g);
@@ -91,7 +79,7 @@ int shrink_waves(int T, int nproj, const int* d_in, int d_out) {
   const int kq = 32 * (d_out > 32 ? 2 : 4);  // k per wave and load batch of the sixteen-wave kernels
   bool all_long = tiles_per_wave(T) == 1;
   for (int i = 0; i < nproj; ++i) all_long = all_long && d_in[i] >= 16 * kq;
-  return tune("SMLM_TUNE_NW", all_long ? 16 : kFwdWaves);
+  return all_long ? 16 : kFwdWaves;
 }
 
 ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
@@ -114,7 +102,6 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   const int cheap = d_in / (32 * d_out), fill = ceil_div(256, units);
   const int cap = cheap > fill ? cheap : fill;
   if (want > cap) want = cap;
-  want = tune("SMLM_TUNE_KSPLIT", want);
   int max_split = d_in / (c.NW * kq);
   if (max_split < 1) max_split = 1;
   if (max_split > kMaxKsplit) max_split = kMaxKsplit;
@@ -190,10 +177,10 @@ int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStrea
 int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int groups, hipStream_t st,
                   ShrinkArgs& a) {
   const int MT = row_major ? 1 : c.MT;
-  a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 1);
+  a.items.interleave = 1;
   const int units = tile_units_max(a.T, S, groups, MT);
   const long items = (long)units * a.items.row_start[a.items.nproj];
-  a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
+  a.items.units_max = (items <= kDirectItems && units <= kMaxGridY) ? units : 0;
   const dim3 grid = item_grid(a.items, items);
   const bool f16 = dtype == SMLM_DTYPE_F16;
   if (a.items.units_max)
@@ -212,7 +199,7 @@ int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
   }
   const int units = tile_units_max(a.T, S, groups, 1);
   const long items = (long)units * a.nproj;
-  a.units_max = items <= tune("SMLM_TUNE_DIRECT", kDirectItems) ? units : 0;
+  a.units_max = items <= kDirectItems ? units : 0;
   const dim3 grid = a.units_max ? dim3((unsigned)items) : work_grid(items);
   if (dtype == SMLM_DTYPE_F16) return launch(reduce_kernel<SMLM_DTYPE_F16>, grid, dim3(256), st, a);
   return launch(reduce_kernel<SMLM_DTYPE_BF16>, grid, dim3(256), st, a);
@@ -269,11 +256,10 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   if (a.drop.seg_p && (row_major || nproj != 1 || a.p[0].vsplit > 0 || (block && !a.w_kn))) return SMLM_ERR_ARG;
   if (row_major) nq = 2;
   if (block) nq = 4;
-  nq = tune("SMLM_TUNE_NQ", nq);
   if (block) nq = 4;
   const int chunk = block ? 32 * nq : kFwdWaves * 32 * nq;  // columns per workgroup
   a.items.nproj = nproj;
-  a.items.interleave = tune("SMLM_TUNE_INTERLEAVE", 0);
+  a.items.interleave = 0;
   a.items.row_start[0] = 0;
   for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);
   const int units = tile_units_max(a.T, S, groups, block ? kBlkTiles : 1);
@@ -281,8 +267,8 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   bool same_rows = true;
   for (int i = 1; i < nproj; ++i)
     same_rows = same_rows && (a.items.row_start[i + 1] - a.items.row_start[i] == a.items.row_start[1]);
-  a.items.flat = tune("SMLM_TUNE_FLAT", same_rows ? 0 : 1);
-  a.items.units_max = (items <= tune("SMLM_TUNE_DIRECT", kDirectItems) && units <= kMaxGridY) ? units : 0;
+  a.items.flat = same_rows ? 0 : 1;
+  a.items.units_max = (items <= kDirectItems && units <= kMaxGridY) ? units : 0;
   const dim3 grid = item_grid(a.items, items);
   const bool f16 = dtype == SMLM_DTYPE_F16;
   if (a.items.units_max)
@@ -903,8 +889,8 @@ static int rms_blocks(int rows, int cols, bool backward) {
     return rows < 1 ? 1 : (rows < cap ? rows : cap);
   }
   const int rows_per_step = cols <= kRmsWaveCols ? 4 : 1;
-  int nb = ceil_div(rows, rows_per_step * (backward ? tune("SMLM_TUNE_RMS_ROWS", 4) : 1));
-  const int cap = backward ? tune("SMLM_TUNE_RMS_CAP", 512) : (1 << 22);
+  int nb = ceil_div(rows, rows_per_step * (backward ? 4 : 1));
+  const int cap = backward ? 512 : (1 << 22);
   if (nb > cap) nb = cap;
   return nb < 1 ? 1 : nb;
 }
