@@ -34,14 +34,16 @@ METRIC = "SMLM tokens/s + HBM GB/s (% of 8 TB/s), Llama-2-7B shapes, 1 GPU"
 
 def workload(name: str):
     """Shapes and routing of BASELINE.json's configs 2-5 (seeds = config number)."""
-    if name in ("cfg2", "cfg2mod"):
-        # adapters drawn uniformly (the headline workload) or dealt round-robin, i % 32 (the variant)
-        ids = np.random.default_rng(2).integers(0, 32, 256).tolist() if name == "cfg2" else [i % 32 for i in range(256)]
+    if name in ("cfg2", "cfg2mod", "cfg2one"):
+        # adapters drawn uniformly (the headline workload) or dealt round-robin, i % 32 (the variant);
+        # cfg2one is the headline batch through ONE projection, what a single layer call of the reference issues
+        ids = [i % 32 for i in range(256)] if name == "cfg2mod" else np.random.default_rng(2).integers(0, 32, 256).tolist()
+        proj = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096)]
         return dict(name=f"{name}: 256 single-token segments over 32 adapters"
-                         f"{'' if name == 'cfg2' else ' dealt round-robin'}, r=16, q/k/v/o 4096->4096, "
+                         f"{' dealt round-robin' if name == 'cfg2mod' else ''}, r=16, "
+                         f"{'q' if name == 'cfg2one' else 'q/k/v/o'} 4096->4096, "
                          "fp16, forward", dtype="fp16", r=16, NA=32, seg=list(range(257)), ids=ids,
-                    proj=[("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096)],
-                    n_train_parts=0)
+                    proj=proj[:1] if name == "cfg2one" else proj, n_train_parts=0)
     if name == "cfg3":
         return dict(name="cfg3: 4x512 prefill + 64 decode, 16 adapters, r=32, gate/up 4096->11008, "
                          "down 11008->4096, fp16, forward", dtype="fp16", r=32, NA=16,
@@ -460,7 +462,9 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
 
     def step(st, build_plan=True):
         if build_plan:
-            st["plan"] = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"])
+            # deferred: the forward call builds the plan itself -- decode batches inside their
+            # shrink launch, the others with the plan launch first (--plan-launch: always that)
+            st["plan"] = K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"], defer=not args.plan_launch)
         fwd(st)
         if P:
             if build_plan or "bplan" not in st:
@@ -563,6 +567,20 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
 
     expand_us = stage_us(2)
     shrink_us = stage_us(1)
+    # decode batches: the shrink launch that also builds the plan (what the step's first forward launches)
+    self_planned = T < 1024 and not args.plan_launch and not P
+    if self_planned:
+        bufs = [st["plan_buf"] for st in sets]
+
+        def planning_shrink():
+            for _ in range(reps):
+                for st, buf in zip(sets, bufs):
+                    keep, st["plan"] = st["plan"], K.SegmentPlan(seg_t, ids_t, T, buf=buf, defer=True)
+                    fwd(st, 1)
+                    st["plan"] = keep
+        g = capture(planning_shrink)
+        timed([(g, 2)])
+        shrink_plan_us = timed([(g, 10)]) * 1e3 / (10 * reps * R)
     expand_bytes = sum(T * ho * 2 * 2 + rsum * ho * 2 + T * r * 2 for _, hi, ho in w["proj"])
     shrink_bytes = sum(T * hi * 2 + rsum * hi * 2 + T * r * 2 for _, hi, ho in w["proj"])
     traffic = {}
@@ -579,6 +597,9 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                          "shrink_bytes_per_launch"),
              launch_line("expand launch (y += s v B^T, all projections of the step)", expand_us, expand_bytes,
                          "expand_bytes_per_launch")]
+    if self_planned:
+        lines.append(launch_line("shrink launch that also builds the plan (the step's first forward call)",
+                                 shrink_plan_us, shrink_bytes, "shrink_self_planned_bytes_per_launch"))
     # the forward launch furthest below the HBM peak is the one the roofline entry names
     roofline = min(lines, key=lambda l: l["frac"])
 
@@ -657,7 +678,8 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         "dtype": "f16" if w["dtype"] == "fp16" else "bf16", "data": "synthetic",
         "config": {"workload": w["name"], "tokens_per_step": T, "segments": S, "adapters": NA, "rank": r,
                    "projections": [f"{n}:{a}->{b}" for n, a, b in w["proj"]],
-                   "buffer_sets_rotated": R, "step_includes": "plan build + fused forward per projection"
+                   "buffer_sets_rotated": R, "step_includes": "plan build (" + ("own launch" if args.plan_launch or T >= 1024 else "inside the shrink launch")
+                   + ") + fused forward per projection"
                    + (" + backward" if P else ""), "graph_replay": not args.eager,
                    "dropout": args.dropout if P else 0.0,
                    "true_ranks_passed": bool(ranks and not args.padded_ranks),
@@ -683,7 +705,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="all",
                     help="all (default): the headline workload cfg2 in full, then cfg3, cfg4 and cfg5 in brief "
-                         "under 'configs'; or one of cfg2 | cfg2mod | cfg3 | cfg4 | cfg5 | rmsnorm | model-step")
+                         "under 'configs'; or one of cfg2 | cfg2mod | cfg2one | cfg3 | cfg4 | cfg5 | rmsnorm | model-step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
     ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
@@ -694,6 +716,9 @@ def main():
     ap.add_argument("--padded-ranks", action="store_true",
                     help="workloads with adapters below the padded rank: do not pass the true ranks "
                          "(the kernels then read the zero padding, as the reference's do)")
+    ap.add_argument("--plan-launch", action="store_true",
+                    help="build the forward plan with its own launch before the forward call, also for decode "
+                         "batches (default: the forward call builds it, decode batches inside the shrink launch)")
     ap.add_argument("--padded-storage", action="store_true",
                     help="workloads with adapters below the padded rank: pass the true ranks but keep the "
                          "adapters zero-padded in memory (default: stored at their own rank, packed)")

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SMLM_ABI_VERSION 2
+#define SMLM_ABI_VERSION 3
 
 #if defined(__GNUC__)
 #define SMLM_API __attribute__((visibility("default")))
@@ -262,11 +262,25 @@ typedef struct smlm_dropout {
  *                  rank-8 adapter beside rank-64 ones then costs 16 bytes of B per output
  *                  column instead of a 128-byte line.  Results equal the padded computation
  *                  bit for bit; v, dV and the workspace keep the launch's rank r.
+ *   build_seg_indptr, build_seg_adapter (smlm_lora_fwd_multi_ex only; both or neither):
+ *                  `plan` is a buffer of smlm_plan_size(T, S) bytes that holds NO plan yet; the
+ *                  call builds the plan smlm_plan_build(plan, ..., build_seg_indptr,
+ *                  build_seg_adapter, SMLM_KEY_I32, T, S) would build, writes it to `plan` (valid
+ *                  for every later call on the stream) and uses it.  The reference sets its
+ *                  problems up inside every call as well (precompute_smlm_forward_args,
+ *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  For
+ *                  decode batches (T < 1024, S <= 1024, n_weights <= 1024, every h_in >= 2048,
+ *                  no dropout) this costs no launch: the shrink's workgroups derive their own
+ *                  tiles from the two arrays while one more workgroup of the same launch writes
+ *                  the plan; other batches get the plan launch first.  Adapter ids must lie in
+ *                  [0, n_weights); stages must include SMLM_STAGE_SHRINK.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;
   const int32_t* adapter_rank;
   int packed_ranks;
+  const int32_t* build_seg_indptr;
+  const int32_t* build_seg_adapter;
 } smlm_lora_opts;
 
 /* smlm_lora_fwd_multi with options. */

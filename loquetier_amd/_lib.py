@@ -31,7 +31,8 @@ class Dropout(C.Structure):
 
 class LoraOpts(C.Structure):
     """struct smlm_lora_opts of include/smlm.h."""
-    _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p), ("packed_ranks", C.c_int)]
+    _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p), ("packed_ranks", C.c_int),
+                ("build_seg_indptr", C.c_void_p), ("build_seg_adapter", C.c_void_p)]
 
 
 _popts = C.POINTER(LoraOpts)

@@ -10,6 +10,7 @@
 #include "smlm.h"
 #include "smlm_backward.hpp"
 #include "smlm_common.hpp"
+#include "smlm_decode.hpp"
 #include "smlm_forward.hpp"
 #include "smlm_plan.hpp"
 
@@ -190,6 +191,37 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
              : launch_shrink_dt<SMLM_DTYPE_BF16, false>(row_major, c.NB, MT, c.NW, grid, st, a);
 }
 
+template <int DT>
+int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
+  const dim3 block(kPlanThreads);  // U must match shrink_cfg
+  if (NB == 1) return launch(shrink_self_planned_kernel<DT, 1, 4>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_self_planned_kernel<DT, 2, 4>, grid, block, st, a);
+  return launch(shrink_self_planned_kernel<DT, 4, 2>, grid, block, st, a);
+}
+
+// batches this route takes: a decode-size batch (one-workgroup plan, sixteen-wave shrink),
+// adapter ids that index a table of at most kSelfPlanWeights entries
+bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
+  return tiles_per_wave(T) == 1 && S <= kPlanSmallSegs && nt_max <= kPlanSmallTiles && n_weights >= 1 &&
+         n_weights <= kSelfPlanWeights && tile_units_max(T, S, n_weights, 1) < kMaxGridY;
+}
+
+int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups, const PlanSortArgs& build,
+                               hipStream_t st, const ShrinkArgs& a) {
+  if (c.NW != 16 || c.MT != 1) return SMLM_ERR_ARG;
+  SelfPlanArgs sp{};
+  sp.sh = a;
+  sp.plan = build;
+  sp.n_weights = groups;
+  sp.units = tile_units_max(a.T, S, groups, 1);
+  int rows = 1;
+  for (int i = 0; i < a.items.nproj; ++i)
+    if (a.items.row_start[i + 1] - a.items.row_start[i] > rows) rows = a.items.row_start[i + 1] - a.items.row_start[i];
+  const dim3 grid((unsigned)rows, (unsigned)sp.units + 1u, (unsigned)a.items.nproj);
+  if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16>(c.NB, grid, st, sp);
+  return launch_self_planned_nb<SMLM_DTYPE_BF16>(c.NB, grid, st, sp);
+}
+
 int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
   const int row_tiles = ceil_div(a.T, kTileRows);
   if (!a.seg_scale && row_tiles <= kMaxGridY * 64) {  // no scale to look up: fold row by row
@@ -308,7 +340,8 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
                const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false,
-               const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr, int packed = 0) {
+               const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr, int packed = 0,
+               const PlanSortArgs* build = nullptr) {
   if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
   ShrinkArgs a{};
   if (drop) a.drop = *drop;
@@ -349,7 +382,10 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   // counters) was measured and dropped: the device-scope release/acquire it needs writes back
   // and invalidates a whole L2 per workgroup on this multi-XCD part and cost 5-10x the launch
   // it saves.
-  int rc = launch_shrink(dtype, row_major, c0, S, groups, st, a);
+  // `build`: the plan does not exist yet -- the sixteen-wave shrink whose workgroups find their
+  // own tile, with one more workgroup that builds the plan (the caller has checked the limits)
+  int rc = build ? launch_shrink_self_planned(dtype, c0, S, groups, *build, st, a)
+                 : launch_shrink(dtype, row_major, c0, S, groups, st, a);
   if (rc || !need_reduce || !fold) return rc;
   ra.plan = a.plan;
   ra.seg_scale = seg_scale;
@@ -635,6 +671,10 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
+  const int32_t* build_s = opts ? opts->build_seg_indptr : nullptr;
+  const int32_t* build_k = opts ? opts->build_seg_adapter : nullptr;
+  if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
+  if (build_s && !(stages & SMLM_STAGE_SHRINK)) return SMLM_ERR_ARG;  // the plan is built with the shrink
   if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
     return SMLM_ERR_ARG;
   if (stages < 1 || stages > (SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND)) return SMLM_ERR_ARG;
@@ -681,9 +721,15 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
       w += align_up((size_t)T * r * 2, 256);
     }
   }
+  // A plan still to be built (opts->build_*): decode batches build it inside the shrink launch,
+  // every other batch with the plan launch first.
+  PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, S, next_pow2(S)};
+  const bool self_planned = build_s && expand_folds && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max);
+  if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, S, st))) return rc;
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                    0.0f, nullptr, st, !expand_folds, false, &drop, w_rank, packed);
+                    0.0f, nullptr, st, !expand_folds, false, &drop, w_rank, packed,
+                    self_planned ? &build : nullptr);
     if (rc) return rc;
   }
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;

@@ -149,15 +149,30 @@ __device__ __forceinline__ int count_below(const T* keys, T key, int j0, int j1)
 // All global reads (keys, segment boundaries) are issued together up front: a
 // first-touch global load costs more than everything else in this kernel, so
 // nothing that was loaded is asked for again; the sorted arrays live in LDS.
-__global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs args) {
-  __shared__ uint64_t K[kPlanSmallSegs], K0[kPlanSmallSegs];
-  __shared__ int32_t start0[kPlanSmallSegs], len0[kPlanSmallSegs];  // by segment
-  __shared__ int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];  // by sorted position
-  __shared__ int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
-  __shared__ int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
-  __shared__ int32_t gpos[kPlanSmallSegs + 1];  // group -> sorted position of its first segment, [NG] = S
-  __shared__ uint64_t wave_tot[17];
-  __shared__ int bad_key, wide_key;
+// The workgroup's LDS of the one-launch route, as a struct so that another kernel can lend the
+// same memory to a workgroup that builds a plan (it is only ever reached by name through a
+// reference that the compiler resolves at compile time, never through a stored pointer).
+struct PlanSmallLds {
+  uint64_t K[kPlanSmallSegs], K0[kPlanSmallSegs];
+  int32_t start0[kPlanSmallSegs], len0[kPlanSmallSegs];  // by segment
+  int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];  // by sorted position
+  int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
+  int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
+  int32_t gpos[kPlanSmallSegs + 1];  // group -> sorted position of its first segment, [NG] = S
+  uint64_t wave_tot[17];
+  int bad_key, wide_key;
+};
+
+// the whole plan of a batch of at most kPlanSmallSegs segments, built by the calling workgroup
+// (kPlanThreads threads)
+__device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSmallLds& L) {
+  auto& K = L.K; auto& K0 = L.K0;
+  auto& start0 = L.start0; auto& len0 = L.len0;
+  auto& sseg = L.sseg; auto& rowpos = L.rowpos;
+  auto& grow = L.grow; auto& gtile = L.gtile; auto& gblk = L.gblk;
+  auto& gseg = L.gseg; auto& gid = L.gid; auto& gpos = L.gpos;
+  auto& wave_tot = L.wave_tot;
+  int& bad_key = L.bad_key; int& wide_key = L.wide_key;
   const PlanView pv = args.pv;
   const int S = args.S, tid = threadIdx.x;  // blockDim.x >= S
 
@@ -326,6 +341,11 @@ __global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs a
     pv.tile_rseg[slot] = rseg;
     if (c == 0) pv.tile_wid[tile] = (kind == SMLM_KEY_I32) ? gid[G] : gseg[G];
   }
+}
+
+__global__ __launch_bounds__(kPlanThreads) void plan_small_kernel(PlanSortArgs args) {
+  __shared__ PlanSmallLds lds;
+  plan_small_body(args, lds);
 }
 
 // --------------------------------------------------------------- two launches

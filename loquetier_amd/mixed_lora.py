@@ -113,7 +113,9 @@ class MixedLoraContext:
 
     def plan(self, device: torch.device, T: int) -> kernel.SegmentPlan:
         if self._plan is None or self._plan.T != T or self._plan.buf.device != device:
-            self._plan = kernel.SegmentPlan(self._segment.to(device), self.seg_adapter(device), T)
+            # deferred: the step's first fused forward builds the plan (decode batches inside its
+            # shrink launch), any other first user builds it with the plan launch
+            self._plan = kernel.SegmentPlan(self._segment.to(device), self.seg_adapter(device), T, defer=True)
         return self._plan
 
     def train_order(self) -> List[int]:

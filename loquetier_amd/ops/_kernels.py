@@ -174,10 +174,15 @@ class SegmentPlan:
     """Tile plan of one flat batch: built once from (segment, adapter ids) and
     shared by every LoRA linear of the step (the reference rebuilds its
     per-problem table inside every kernel call,
-    smlm_forward_cutlass.cuh:76-79)."""
+    smlm_forward_cutlass.cuh:76-79).
+
+    defer=True (plans keyed by int32 adapter ids): nothing is launched here; the first
+    smlm_lora_forward(_multi) call that gets the plan builds it -- for decode batches
+    inside its shrink launch, at no launch of its own -- and every other user builds it
+    with the plan launch first (ensure_built)."""
 
     def __init__(self, segment: torch.Tensor, seg_key: Optional[torch.Tensor], T: int,
-                 buf: Optional[torch.Tensor] = None):
+                 buf: Optional[torch.Tensor] = None, defer: bool = False):
         _check_input(segment, "segment")
         if segment.dtype != torch.int32 or segment.dim() != 1:
             raise RuntimeError("segment must be a 1D int32 tensor")
@@ -205,10 +210,19 @@ class SegmentPlan:
         elif buf.dtype != torch.uint8 or buf.numel() < nbytes or buf.device != dev:
             raise RuntimeError(f"plan buffer must be a uint8 tensor of >= {nbytes} bytes on {dev}")
         self.buf = buf
+        self.built = False
+        if not (defer and kind == _lib.SMLM_KEY_I32):
+            self.ensure_built()
+
+    def ensure_built(self) -> None:
+        if self.built:
+            return
+        dev = self.segment.device
         with torch.cuda.device(dev):
-            rc = _lib.load().smlm_plan_build(self.buf.data_ptr(), self.buf.numel(), segment.data_ptr(),
-                                             _ptr(seg_key), kind, self.T, self.S, _stream(dev))
+            rc = _lib.load().smlm_plan_build(self.buf.data_ptr(), self.buf.numel(), self.segment.data_ptr(),
+                                             _ptr(self.seg_key), self.kind, self.T, self.S, _stream(dev))
         _lib.check(rc, "smlm_plan_build")
+        self.built = True
 
     @staticmethod
     def nbytes(T: int, S: int) -> int:
@@ -216,6 +230,7 @@ class SegmentPlan:
 
     def header(self) -> Tuple[int, int, int, int]:
         """(n_tiles, n_groups, rows covered, key kind used) -- synchronises; for tests."""
+        self.ensure_built()
         h = self.buf[:16].view(torch.int32).cpu()
         return int(h[0]), int(h[1]), int(h[2]), int(h[3])
 
@@ -246,6 +261,7 @@ def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, pl
     _check_dim(2, x, "x")
     _check_table(w_ptrs, plan, "w_ptrs")
     _check_scale(seg_scale, plan)
+    plan.ensure_built()
     if y.dtype != x.dtype or y.size(0) != x.size(0) or x.size(0) != plan.T:
         raise RuntimeError("x [T,d_in] and y [T,d_out] must share dtype and T with the plan")
     code = _dtype_code(x)
@@ -382,6 +398,13 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
         ws = _workspace(dev, need.value, workspace)
         n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
         opts = _opts(plan, dropout, [x.size(1) for x in xs], adapter_rank, n_weights, packed_ranks)
+        if not plan.built:
+            if stages & _lib.SMLM_STAGE_SHRINK:  # a deferred plan: this call builds it
+                opts = opts or _lib.LoraOpts()
+                opts.build_seg_indptr = plan.segment.data_ptr()
+                opts.build_seg_adapter = plan.seg_key.data_ptr()
+            else:
+                plan.ensure_built()
         rc = _lib.load().smlm_lora_fwd_multi_ex(
             n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
@@ -389,6 +412,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
             _ptr(seg_scale), int(stages), None if opts is None else C.byref(opts), _stream(dev))
     _lib.check(rc, "smlm_lora_forward")
+    plan.built = True
 
 
 def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.Tensor,
@@ -407,6 +431,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     if plan.kind != _lib.SMLM_KEY_I32:
         raise RuntimeError("the backward plan must be built from int32 adapter ids")
     n_rows = plan.T
+    plan.ensure_built()
     if dy.size(0) < n_rows or x.size(0) < n_rows or dx.size(0) < n_rows:
         raise RuntimeError("dy, x and dx need at least plan.T rows")
     if dx.dtype != dy.dtype or x.dtype != dy.dtype or (v is not None and v.dtype != dy.dtype):

@@ -94,3 +94,54 @@ def test_captured_step_replays_like_eager(K, gpu_device, T_train, n_dec):
         for a, b_ in zip(outputs(static), outputs(eager)):
             assert torch.equal(a, b_), f"replay {k} differs from the eager run"
         assert not torch.isnan(static["dx"].float()).any()
+
+
+def test_captured_decode_step_builds_its_plan_on_every_replay(K, gpu_device):
+    """A decode step captured with a deferred plan: the shrink launch derives the tiles and writes the
+    plan itself, so a replay follows whatever routing the segment and adapter tensors hold by then."""
+    d, tdt = gpu_device, torch.float16
+    T, h_in, h_out, r, NA = 96, 2048, 512, 16, 7
+    gen = torch.Generator().manual_seed(62)
+    A = [(torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for _ in range(NA)]
+    B = [(torch.randn(h_out, r, generator=gen) / r ** 0.5).to(tdt).to(d) for _ in range(NA)]
+    ta, tb = ptrs(A, d), ptrs(B, d)
+    seg_t = torch.arange(T + 1, dtype=torch.int32, device=d)
+    scale = torch.full((T,), 0.5, device=d)
+
+    def buffers():
+        return dict(x=torch.empty(T, h_in, dtype=tdt, device=d), y=torch.empty(T, h_out, dtype=tdt, device=d),
+                    v=torch.empty(T, r, dtype=tdt, device=d), ids=torch.zeros(T, dtype=torch.int32, device=d),
+                    plan=torch.zeros(K.SegmentPlan.nbytes(T, T), dtype=torch.uint8, device=d))
+
+    def step(b, defer):
+        plan = K.SegmentPlan(seg_t, b["ids"], T, buf=b["plan"], defer=defer)
+        K.smlm_lora_forward(b["y"], b["x"], ta, tb, plan, r, seg_scale=scale, beta=1.0, v_out=b["v"])
+        # a second layer of the step reuses the plan the first one left
+        K.smlm_lora_forward(b["y"], b["x"], ta, tb, plan, r, seg_scale=scale, beta=1.0)
+
+    def fill(b, k):
+        gk = torch.Generator().manual_seed(200 + k)
+        b["x"].copy_(torch.randn(T, h_in, generator=gk).to(tdt))
+        b["y"].copy_(torch.randn(T, h_out, generator=gk).to(tdt))
+        b["ids"].copy_(torch.randint(0, NA, (T,), generator=gk).to(torch.int32))
+
+    static, eager = buffers(), buffers()
+    side = torch.cuda.Stream()
+    fill(static, 0)
+    with torch.cuda.stream(side):
+        step(static, True)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step(static, True)
+    for k in range(1, 5):
+        fill(static, k)
+        fill(eager, k)
+        torch.cuda.synchronize()
+        graph.replay()
+        step(eager, False)          # eager, with the plan launch
+        torch.cuda.synchronize()
+        for name in ("y", "v"):
+            assert torch.equal(static[name], eager[name]), f"replay {k}: {name} differs from the eager run"
+        # the plans' headers agree (entries past the live counts keep whatever an earlier batch left)
+        assert torch.equal(static["plan"][:64], eager["plan"][:64])

@@ -1,0 +1,135 @@
+"""A plan that the first fused forward builds itself (SegmentPlan(defer=True);
+smlm_lora_opts.build_seg_indptr / build_seg_adapter).  Decode batches build it inside the
+shrink launch: every workgroup derives its own tile from the segment table and one more
+workgroup writes the plan.  Whatever route the library takes, the call must leave the very
+plan smlm_plan_build writes (byte for byte) and the very outputs a call over a prebuilt plan
+gives (bit for bit); the outputs are also held against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TDT = {"fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def K(gpu_device):
+    from loquetier_amd import _lib
+    from loquetier_amd.ops import _kernels
+    _lib.load()
+    return _kernels
+
+
+def ptrs(ts, dev):
+    return torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=dev)
+
+
+def decode_ids(n, na, seed):
+    return np.random.default_rng(seed).integers(0, na, n).tolist()
+
+
+def ragged(seed, n_seg, max_len, na):
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(0, max_len + 1, n_seg)
+    seg = np.concatenate([[0], np.cumsum(lens)]).tolist()
+    return seg, rng.integers(0, na, n_seg).tolist()
+
+
+# name, seg, ids, NA (table entries), T (rows of x; rows past seg[-1] belong to no segment), rank, [(h_in, h_out)]
+CASES = [
+    ("decode256-qkvo", list(range(257)), decode_ids(256, 32, 2), 32, 256, 16, [(4096, 4096)] * 4),
+    ("one-projection", list(range(257)), decode_ids(256, 32, 3), 32, 256, 16, [(4096, 1024)]),
+    ("ragged-empty-uncovered",) + ragged(4, 90, 9, 12) + (12, 0, 16, [(2048, 512), (2048, 256)]),
+    ("one-adapter-many-tiles", [0, 300, 301, 640], [5, 5, 5], 8, 700, 32, [(2048, 320)]),
+    ("absent-adapters", list(range(0, 200, 2)), [(7 * i) % 600 for i in range(99)], 1024, 198, 8, [(2048, 128)]),
+    ("1024-segments", list(range(0, 1000)) + [1000] * 25, [(i * 37) % 1000 for i in range(1024)], 1000, 1000, 16,
+     [(2048, 256)]),
+    ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
+    ("short-k-falls-back", list(range(41)), decode_ids(40, 4, 8), 4, 40, 16, [(512, 256)]),   # four-wave shrink: plan launch first
+    ("tile-blocks-fall-back", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 16, [(2048, 320)]),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_deferred_plan_equals_built_plan(K, gpu_device, case, dt):
+    name, seg, ids, NA, T, r, projs = case
+    T = max(T, seg[-1])
+    d, tdt = gpu_device, TDT[dt]
+    gen = torch.Generator().manual_seed(61)
+    S = len(ids)
+    seg_t = torch.tensor(seg, dtype=torch.int32, device=d)
+    ids_t = torch.tensor(ids, dtype=torch.int32, device=d)
+    used = sorted(set(ids))
+    xs, y0, A, B = [], [], [], []
+    for h_in, h_out in projs:
+        xs.append((torch.randn(T, h_in, generator=gen)).to(tdt).to(d))
+        y0.append(torch.randn(T, h_out, generator=gen).to(tdt).to(d))
+        # only the adapters in use get weights; the other table entries hold an address that must never be read
+        wa = {a: (torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for a in used}
+        wb = {a: (torch.randn(h_out, r, generator=gen) / r ** 0.5).to(tdt).to(d) for a in used}
+        A.append(wa)
+        B.append(wb)
+    tab = lambda w: torch.tensor([w[a].data_ptr() if a in w else 16 for a in range(NA)], dtype=torch.int64, device=d)
+    a_tabs, b_tabs = [tab(w) for w in A], [tab(w) for w in B]
+    sc = (torch.rand(S, generator=gen) + 0.5).to(d)
+
+    def run(plan):
+        ys = [y.clone() for y in y0]
+        vs = [torch.full((T, r), 3.0, dtype=tdt, device=d) for _ in projs]
+        K.smlm_lora_forward_multi(ys, xs, a_tabs, b_tabs, plan, r, seg_scale=sc, beta=1.0, v_out=vs)
+        return ys, vs
+
+    nbytes = max(K.SegmentPlan.nbytes(T, S), 64)
+    fresh = lambda: torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=d)  # bytes no build writes stay as they are
+    built = K.SegmentPlan(seg_t, ids_t, T, buf=fresh())
+    ys_ref, vs_ref = run(built)
+    deferred = K.SegmentPlan(seg_t, ids_t, T, buf=fresh(), defer=True)
+    assert not deferred.built
+    ys, vs = run(deferred)
+    assert deferred.built
+    torch.cuda.synchronize()
+    assert torch.equal(deferred.buf, built.buf), "the call must leave the plan smlm_plan_build writes"
+    for i in range(len(projs)):
+        assert torch.equal(ys[i], ys_ref[i]) and torch.equal(vs[i], vs_ref[i])
+    # the plan it left serves later calls
+    ys2, vs2 = run(deferred)
+    for i in range(len(projs)):
+        assert torch.equal(ys2[i], ys_ref[i]) and torch.equal(vs2[i], vs_ref[i])
+
+    # and the outputs are the oracle's
+    from oracle import torch_segments as ref
+    for i, (h_in, h_out) in enumerate(projs[:1]):
+        wa = [A[i][a].cpu() for a in ids]
+        wb = [B[i][a].cpu() for a in ids]
+        y_o, v_o = ref.add_lora_forward(xs[i].cpu(), wa, wb, seg, y=y0[i].cpu().clone(), beta=1.0,
+                                        seg_scale=sc.cpu().tolist())
+        assert torch.allclose(vs[i].cpu().float()[:seg[-1]], v_o.float()[:seg[-1]], rtol=1e-2, atol=1e-3 if dt == "fp16" else 8e-3)
+        # y against the oracle fed with the kernel's own v (a rounding flip of v moves a whole row of y)
+        vk = vs[i].cpu().float()
+        for s_i in range(S):
+            lo, hi = seg[s_i], seg[s_i + 1]
+            if hi <= lo:
+                continue
+            want = (y0[i].cpu().float()[lo:hi] + float(sc[s_i]) * (vk[lo:hi] @ wb[s_i].float().t())).to(tdt).float()
+            assert torch.allclose(ys[i].cpu().float()[lo:hi], want, rtol=1e-2, atol=2e-2 if dt == "bf16" else 4e-3)
+    if T > seg[-1]:  # rows past the last segment are left alone
+        for i in range(len(projs)):
+            assert torch.equal(ys[i][seg[-1]:], y0[i][seg[-1]:])
+
+
+def test_deferred_plan_is_built_by_other_users_first(K, gpu_device):
+    d = gpu_device
+    seg = torch.tensor([0, 3, 9], dtype=torch.int32, device=d)
+    ids = torch.tensor([1, 0], dtype=torch.int32, device=d)
+    fresh = lambda: torch.full((max(K.SegmentPlan.nbytes(9, 2), 64),), 0xA5, dtype=torch.uint8, device=d)
+    p1 = K.SegmentPlan(seg, ids, 9, buf=fresh())
+    p2 = K.SegmentPlan(seg, ids, 9, buf=fresh(), defer=True)
+    assert not p2.built
+    assert p2.header() == p1.header() and p2.built
+    torch.cuda.synchronize()
+    assert torch.equal(p1.buf, p2.buf)
+    # pointer-keyed plans are never deferred
+    p3 = K.SegmentPlan(seg, torch.tensor([32, 16], dtype=torch.int64, device=d), 9, defer=True)
+    assert p3.built

@@ -31,7 +31,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
     for name in declared:
         assert hasattr(handle, name), f"{name} is declared in smlm.h but not exported"
     assert declared == set(lib.SIGNATURES), "ctypes binding and header disagree"
-    assert lib.load().smlm_abi_version() == 2
+    assert lib.load().smlm_abi_version() == 3
 
 
 def test_missing_library_fails_loudly(lib, monkeypatch):
@@ -92,6 +92,25 @@ def test_argument_validation_codes(lib):
     assert need <= lib.SMLM_STATIC_SCRATCH_BYTES     # the fine-tune + serve batch fits
     assert L.smlm_lora_bwd(p, p, p, p, p, None, p, p, p, p, 16, 16, 1, 1, 64, 64, 8, 1,
                            None, None) == -4
+
+
+def test_plan_on_first_use_argument_validation(lib):
+    """smlm_lora_opts.build_seg_indptr / build_seg_adapter: both or neither, and only with the shrink stage."""
+    L = lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256  # aligned fake "device" address; never dereferenced
+    VP, CI = ctypes.c_void_p * 1, ctypes.c_int * 1
+
+    def call(opts, stages=3, T=16):
+        return L.smlm_lora_fwd_multi_ex(1, VP(p), VP(p), None, VP(p), VP(p), 2, CI(64), CI(64), p, p, 1 << 30,
+                                        T, 2, 16, 0, 0.0, None, stages, ctypes.byref(opts), None)
+    o = lib.LoraOpts()
+    o.build_seg_indptr = p
+    assert call(o) == -1                  # the adapter ids are missing
+    o.build_seg_adapter = p
+    assert call(o, stages=2) == -1        # the plan is built with the shrink
+    assert call(o, T=0) == 0              # empty batch: nothing to build, nothing launched
+    assert ctypes.sizeof(lib.LoraOpts) == 40
 
 
 def test_rms_norm_argument_validation_codes(lib):
