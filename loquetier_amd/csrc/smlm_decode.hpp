@@ -23,6 +23,7 @@
 namespace smlm {
 
 constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of the route; = threads of a workgroup
+constexpr int kSelfPlanWaveScan = 256;  // up to this many, every wave scans the adapters' tile counts by itself
 
 struct SelfPlanArgs {
   ShrinkArgs sh;        // sh.plan is not read (the plan does not exist yet), except w_rank
@@ -120,16 +121,36 @@ __global__ __launch_bounds__(kPlanThreads) void shrink_self_planned_kernel(SelfP
   F.wtab[tid] = wp;
   F.rtab[tid] = wr;
   __syncthreads();
-  // first tile of every adapter (adapters in ascending order, as the plan's groups are)
-  const uint32_t nt = tid < NA ? (uint32_t)((F.hist[tid] + kTileRows - 1) / kTileRows) : 0u;
-  uint32_t last;
-  const uint32_t first = block_scan_excl_1(nt, F.tot_a, &last);
-  if ((uint32_t)tile >= first && (uint32_t)tile < last) {
-    F.sel[0] = tid;
-    F.sel[1] = tile - (int)first;
+  // first tile of every adapter (adapters in ascending order, as the plan's groups are) -> the
+  // adapter that owns `tile` and the tile's index among that adapter's tiles
+  int wid = -1, sub = 0;
+  if (NA <= kSelfPlanWaveScan) {
+    // few adapters: every wave walks the table by itself, 64 adapters a step, and needs no barrier
+    uint32_t carry = 0;
+    for (int a0 = 0; a0 < NA; a0 += kWaveSize) {
+      const uint32_t n = a0 + lane < NA ? (uint32_t)((F.hist[a0 + lane] + kTileRows - 1) / kTileRows) : 0u;
+      const uint32_t last = carry + wave_scan_incl_u32(n), first = last - n;
+      const uint64_t hit = __ballot((uint32_t)tile >= first && (uint32_t)tile < last);
+      if (hit) {  // uniform over the wave; at most one lane
+        const int l = __builtin_ctzll(hit);
+        wid = a0 + l;
+        sub = tile - (int)__builtin_amdgcn_readlane((int)first, l);
+        break;
+      }
+      carry = (uint32_t)__builtin_amdgcn_readlane((int)last, kWaveSize - 1);
+    }
+  } else {
+    const uint32_t nt = tid < NA ? (uint32_t)((F.hist[tid] + kTileRows - 1) / kTileRows) : 0u;
+    uint32_t last;
+    const uint32_t first = block_scan_excl_1(nt, F.tot_a, &last);
+    if ((uint32_t)tile >= first && (uint32_t)tile < last) {
+      F.sel[0] = tid;
+      F.sel[1] = tile - (int)first;
+    }
+    __syncthreads();
+    wid = F.sel[0];
+    sub = F.sel[1];
   }
-  __syncthreads();
-  const int wid = F.sel[0];
   if (wid < 0) return;  // past the last tile; uniform over the workgroup
   const uint16_t* W = reinterpret_cast<const uint16_t*>(F.wtab[wid]);
   int nlim = P.d_out;  // weight rows at or past it are zero padding
@@ -153,7 +174,7 @@ __global__ __launch_bounds__(kPlanThreads) void shrink_self_planned_kernel(SelfP
   load_w(kbeg, wf);
 
   // rows of the adapter in segment order: tile j of the adapter holds its rows 16j .. 16j+15
-  const int q_lo = F.sel[1] * kTileRows;
+  const int q_lo = sub * kTileRows;
   const uint32_t mine = (counted && key == wid) ? (uint32_t)len : 0u;
   uint32_t hi_u;
   const int lo = (int)block_scan_excl_1(mine, F.tot_b, &hi_u);
