@@ -133,3 +133,53 @@ def test_deferred_plan_is_built_by_other_users_first(K, gpu_device):
     # pointer-keyed plans are never deferred
     p3 = K.SegmentPlan(seg, torch.tensor([32, 16], dtype=torch.int64, device=d), 9, defer=True)
     assert p3.built
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_decode_batches(K, gpu_device, seed):
+    """Random segment tables (empty segments, several rows a segment, uncovered rows, adapters that own
+    nothing, a few negative ids = segments no adapter serves): deferred and prebuilt plans agree."""
+    rng = np.random.default_rng(700 + seed)
+    d, tdt = gpu_device, [torch.float16, torch.bfloat16][seed % 2]
+    NA = int(rng.choice([1, 3, 40, 64, 65, 200, 257, 900]))
+    S = int(rng.integers(1, 400))
+    lens = rng.integers(0, 4, S)
+    lens[rng.random(S) < 0.05] = int(rng.integers(10, 60))
+    while lens.sum() >= 1000:
+        lens[int(np.argmax(lens))] = 1
+    seg = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ids = rng.integers(0, NA, S).astype(np.int32)
+    ids[rng.random(S) < 0.03] = -1
+    T = int(seg[-1]) + int(rng.integers(0, 20))
+    if T == 0:
+        T = 8
+    r = int(rng.choice([8, 16, 32, 64]))
+    h_in, h_out = 2048, int(rng.choice([64, 136, 512]))
+    gen = torch.Generator().manual_seed(int(seed))
+    used = sorted(set(int(i) for i in ids if i >= 0))
+    wa = {a: (torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for a in used}
+    wb = {a: (torch.randn(h_out, r, generator=gen) / r ** 0.5).to(tdt).to(d) for a in used}
+    tab = lambda w: torch.tensor([w[a].data_ptr() if a in w else 16 for a in range(NA)], dtype=torch.int64, device=d)
+    ta, tb = tab(wa), tab(wb)
+    x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    y0 = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    seg_t, ids_t = torch.tensor(seg, device=d), torch.tensor(ids, device=d)
+    sc = (torch.rand(S, generator=gen) + 0.5).to(d)
+    nbytes = max(K.SegmentPlan.nbytes(T, S), 64)
+    out = []
+    for defer in (False, True):
+        plan = K.SegmentPlan(seg_t, ids_t, T, buf=torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=d), defer=defer)
+        y, v = y0.clone(), torch.full((T, r), 3.0, dtype=tdt, device=d)
+        K.smlm_lora_forward(y, x, ta, tb, plan, r, seg_scale=sc, beta=1.0, v_out=v)
+        torch.cuda.synchronize()
+        out.append((y, v, plan.buf))
+    for a, b in zip(*out):
+        assert torch.equal(a, b)
+    # rows that belong to no served segment keep their y
+    served = np.zeros(T, dtype=bool)
+    for i in range(S):
+        if ids[i] >= 0:
+            served[seg[i]:seg[i + 1]] = True
+    idle = torch.tensor(~served, device=d)
+    assert torch.equal(out[1][0][idle], y0[idle])
+    assert not torch.equal(out[1][0][~idle], y0[~idle]) or not served.any()
