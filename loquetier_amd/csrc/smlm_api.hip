@@ -71,16 +71,17 @@ struct ShrinkCfg {
   int NB, U, MT, NW, ksplit, k_per_wave, zblocks;
 };
 
-constexpr int kDecodeSplit = 2;  // k halves of the sixteen-wave shrink
+constexpr int kDecodeWaves = 8;  // waves of the decode shrink's workgroups ...
+constexpr int kDecodeSplit = 4;  // ... and its k split over workgroups, folded by the expand kernel
 constexpr int kMaxExpandFold = kMaxVsplit;  // most partials the expand kernel folds itself
 
 // waves per shrink workgroup, one choice for all projections of a launch: small
-// batches whose every projection has a long enough k use sixteen waves
+// batches whose every projection has a long enough k use eight waves and split k in four
 int shrink_waves(int T, int nproj, const int* d_in, int d_out) {
-  const int kq = 32 * (d_out > 32 ? 2 : 4);  // k per wave and load batch of the sixteen-wave kernels
+  const int kq = 32 * (d_out > 32 ? 2 : 4);  // k per wave and load batch of the decode kernels
   bool all_long = tiles_per_wave(T) == 1;
   for (int i = 0; i < nproj; ++i) all_long = all_long && d_in[i] >= 16 * kq;
-  return all_long ? 16 : kFwdWaves;
+  return all_long ? kDecodeWaves : kFwdWaves;
 }
 
 ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
@@ -97,9 +98,9 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   // k split over workgroups: enough of them to fill the chip, but every split writes and
   // re-reads an fp32 partial of the output (8*r bytes a row against 2*d_in of input), so
   // beyond 256 workgroups the split stops where the partials reach an eighth of the input.
-  // Sixteen-wave workgroups (decode batches: few tiles) split k in two, which doubles the
-  // number of CUs at work; the expand kernel adds the two halves.
-  int want = c.NW == 16 ? kDecodeSplit : ceil_div(1024, units);
+  // Eight-wave workgroups (decode batches: few tiles) split k in four, which quadruples the
+  // number of CUs at work; the expand kernel adds the four partials.
+  int want = c.NW == kDecodeWaves ? kDecodeSplit : ceil_div(1024, units);
   const int cheap = d_in / (32 * d_out), fill = ceil_div(256, units);
   const int cap = cheap > fill ? cheap : fill;
   if (want > cap) want = cap;
@@ -114,7 +115,7 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
 
 // most k-split partials a shrink of this shape can leave behind, whichever wave count it runs with
 int fwd_ksplit_bound(int T, int d_in, int d_out) {
-  const int a = shrink_cfg(T, d_in, d_out, kFwdWaves).ksplit, b = shrink_cfg(T, d_in, d_out, 16).ksplit;
+  const int a = shrink_cfg(T, d_in, d_out, kFwdWaves).ksplit, b = shrink_cfg(T, d_in, d_out, kDecodeWaves).ksplit;
   return a > b ? a : b;
 }
 
@@ -163,13 +164,13 @@ int launch_shrink_dt(bool row_major, int NB, int MT, int NW, dim3 grid, hipStrea
     return launch_shrink_nb<DT, kFwdWaves, true, DIRECT>(NB, grid, st, a);
   if (a.drop.seg_p) {  // dropout of the training rows: x in the usual layout, weights [n][k]
     if (MT == 1)
-      return NW == 16 ? launch_shrink_nb<DT, 16, false, DIRECT, true>(NB, grid, st, a)
-                      : launch_shrink_nb<DT, kFwdWaves, false, DIRECT, true>(NB, grid, st, a);
+      return NW == kDecodeWaves ? launch_shrink_nb<DT, kDecodeWaves, false, DIRECT, true>(NB, grid, st, a)
+                                : launch_shrink_nb<DT, kFwdWaves, false, DIRECT, true>(NB, grid, st, a);
     return launch_shrink_block<DT, DIRECT, false, true>(NB, grid, st, a);
   }
   if (MT == 1)
-    return NW == 16 ? launch_shrink_nb<DT, 16, false, DIRECT>(NB, grid, st, a)
-                    : launch_shrink_nb<DT, kFwdWaves, false, DIRECT>(NB, grid, st, a);
+    return NW == kDecodeWaves ? launch_shrink_nb<DT, kDecodeWaves, false, DIRECT>(NB, grid, st, a)
+                              : launch_shrink_nb<DT, kFwdWaves, false, DIRECT>(NB, grid, st, a);
   return a.w_kn ? launch_shrink_block<DT, DIRECT, true>(NB, grid, st, a)
                 : launch_shrink_block<DT, DIRECT, false>(NB, grid, st, a);
 }
@@ -193,22 +194,22 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
 
 template <int DT>
 int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
-  const dim3 block(kPlanThreads);  // U must match shrink_cfg
+  const dim3 block(kSelfPlanThreads);  // U must match shrink_cfg
   if (NB == 1) return launch(shrink_self_planned_kernel<DT, 1, 4>, grid, block, st, a);
   if (NB == 2) return launch(shrink_self_planned_kernel<DT, 2, 4>, grid, block, st, a);
   return launch(shrink_self_planned_kernel<DT, 4, 2>, grid, block, st, a);
 }
 
-// batches this route takes: a decode-size batch (one-workgroup plan, sixteen-wave shrink),
+// batches this route takes: a decode-size batch (one-workgroup plan, eight-wave shrink),
 // adapter ids that index a table of at most kSelfPlanWeights entries
 bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
-  return tiles_per_wave(T) == 1 && S <= kPlanSmallSegs && nt_max <= kPlanSmallTiles && n_weights >= 1 &&
+  return tiles_per_wave(T) == 1 && S <= kSelfPlanSegs && nt_max <= 4 * kSelfPlanSegs && n_weights >= 1 &&
          n_weights <= kSelfPlanWeights && tile_units_max(T, S, n_weights, 1) < kMaxGridY;
 }
 
 int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups, const PlanSortArgs& build,
                                hipStream_t st, const ShrinkArgs& a) {
-  if (c.NW != 16 || c.MT != 1) return SMLM_ERR_ARG;
+  if (c.NW * kWaveSize != kSelfPlanThreads || c.MT != 1) return SMLM_ERR_ARG;
   SelfPlanArgs sp{};
   sp.sh = a;
   sp.plan = build;
@@ -382,7 +383,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   // counters) was measured and dropped: the device-scope release/acquire it needs writes back
   // and invalidates a whole L2 per workgroup on this multi-XCD part and cost 5-10x the launch
   // it saves.
-  // `build`: the plan does not exist yet -- the sixteen-wave shrink whose workgroups find their
+  // `build`: the plan does not exist yet -- the decode shrink whose workgroups find their
   // own tile, with one more workgroup that builds the plan (the caller has checked the limits)
   int rc = build ? launch_shrink_self_planned(dtype, c0, S, groups, *build, st, a)
                  : launch_shrink(dtype, row_major, c0, S, groups, st, a);
@@ -703,13 +704,13 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   plan_carve(const_cast<void*>(plan), T, S, &pv);
 
   // shrink: every projection's v, rounded to 16 bits (into v_out when the caller wants it).
-  // Decode batches (sixteen-wave shrink, one-tile expand) skip the fold launch: the expand
+  // Decode batches (eight-wave shrink, one-tile expand) skip the fold launch: the expand
   // kernel adds the few partials while it loads v.
   float* partial[kMaxProj];
   void* v16[kMaxProj];
   int vsplit[kMaxProj];
   const int nw = shrink_waves(T, n_proj, h_in, r);
-  bool expand_folds = nw == 16 && tiles_per_wave(T) == 1;
+  bool expand_folds = nw == kDecodeWaves && tiles_per_wave(T) == 1;
   {
     char* w = reinterpret_cast<char*>(workspace);
     for (int i = 0; i < n_proj; ++i) {

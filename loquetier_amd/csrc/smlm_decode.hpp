@@ -2,7 +2,7 @@
 //
 // A model step usually builds its tile plan once and every layer reuses it.  The first
 // fused forward of a step can skip that launch: the batch's segment table and adapter ids
-// go straight to the sixteen-wave shrink.  Every workgroup derives the tile it would have
+// go straight to the decode shrink (eight waves).  Every workgroup derives the tile it would have
 // looked up -- the adapter and the (at most sixteen) rows of tile t, numbered exactly as
 // the plan numbers them -- from the segment table itself, and ONE extra workgroup of the
 // same launch builds the plan proper (the body of plan_small_kernel) for the expand launch
@@ -22,7 +22,9 @@
 
 namespace smlm {
 
-constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of the route; = threads of a workgroup
+constexpr int kSelfPlanThreads = 512;   // eight waves, as the decode shrink_kernel
+constexpr int kSelfPlanSegs = 512;      // most segments of the route: one per thread
+constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of the route: two per thread
 constexpr int kSelfPlanWaveScan = 256;  // up to this many, every wave scans the adapters' tile counts by itself
 
 struct SelfPlanArgs {
@@ -39,7 +41,7 @@ struct SelfPlanScratch {
   int32_t hist[kSelfPlanWeights];   // rows per adapter
   uint64_t wtab[kSelfPlanWeights];  // this projection's weight table
   int32_t rtab[kSelfPlanWeights];   // true ranks, when given
-  uint32_t tot_a[16], tot_b[16];    // wave totals of the two scans
+  uint32_t tot_a[8], tot_b[8];      // wave totals of the two scans
   int32_t rows16[kTileRows], rseg16[kTileRows];
   int32_t sel[2];                   // adapter of the tile (-1: no such tile), tile's index within the adapter
 };
@@ -48,18 +50,19 @@ struct SelfPlanScratch {
 // (ranks up to 32) and over it otherwise.
 template <int NB>
 struct SelfPlanWork {
-  static constexpr bool kOverlay = sizeof(SelfPlanScratch) + sizeof(f32x4) * 16 * NB * kWaveSize > sizeof(PlanSmallLds);
+  static constexpr bool kOverlay =
+      sizeof(SelfPlanScratch) + sizeof(f32x4) * 8 * NB * kWaveSize > sizeof(PlanSmallLdsT<kSelfPlanSegs>);
   SelfPlanScratch find;
-  f32x4 red[kOverlay ? 1 : 16][NB][kWaveSize];
+  f32x4 red[kOverlay ? 1 : 8][NB][kWaveSize];
 };
 template <int NB>
 union SelfPlanLds {
-  PlanSmallLds plan;                  // the plan-building workgroup
+  PlanSmallLdsT<kSelfPlanSegs> plan;  // the plan-building workgroup
   SelfPlanWork<NB> work;              // the others: finding their tile, then the cross-wave sum
-  f32x4 red[16][NB][kWaveSize];       // ... which reuses the scratch's memory when the two do not fit side by side
+  f32x4 red[8][NB][kWaveSize];        // ... which reuses the scratch's memory when the two do not fit side by side
 };
 
-// Exclusive prefix of v over the workgroup (16 waves) with ONE barrier: every wave leaves its
+// Exclusive prefix of v over the workgroup (8 waves) with ONE barrier: every wave leaves its
 // total, every thread adds the totals of the waves before its own.  `tot` must not be in use.
 __device__ __forceinline__ uint32_t block_scan_excl_1(uint32_t v, uint32_t* tot, uint32_t* incl_out) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -68,16 +71,16 @@ __device__ __forceinline__ uint32_t block_scan_excl_1(uint32_t v, uint32_t* tot,
   __syncthreads();
   uint32_t before = 0;
 #pragma unroll
-  for (int w = 0; w < 15; ++w) before += w < wave ? tot[w] : 0u;
+  for (int w = 0; w < 7; ++w) before += w < wave ? tot[w] : 0u;
   *incl_out = before + in_wave;
   return before + in_wave - v;
 }
 
 template <int DT, int NB, int U>
-__global__ __launch_bounds__(kPlanThreads) void shrink_self_planned_kernel(SelfPlanArgs a) {
-  static_assert(kPlanThreads == 16 * kWaveSize && kSelfPlanWeights == kPlanThreads, "one thread per table entry");
+__global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(SelfPlanArgs a) {
+  static_assert(kSelfPlanSegs <= kSelfPlanThreads && kSelfPlanWeights == 2 * kSelfPlanThreads, "entries per thread");
   __shared__ SelfPlanLds<NB> sm;
-  constexpr int NW = 16;
+  constexpr int NW = kSelfPlanThreads / kWaveSize;
   constexpr bool kOverlay = SelfPlanWork<NB>::kOverlay;
   const int tid = threadIdx.x;
   if ((int)blockIdx.y == a.units) {  // the extra row of the grid: one workgroup builds the plan
@@ -106,20 +109,23 @@ __global__ __launch_bounds__(kPlanThreads) void shrink_self_planned_kernel(SelfP
     const int s1 = ((const SMLM_GLOBAL int32_t*)a.plan.s)[tid + 1];
     len = s1 > s0 ? s1 - s0 : 0;
   }
-  uint64_t wp = 0;
-  int wr = 0;
-  if (tid < NA) {
-    wp = ((const SMLM_GLOBAL uint64_t*)P.w_ptrs)[tid];
-    if (a.sh.plan.w_rank) wr = ((const SMLM_GLOBAL int32_t*)a.sh.plan.w_rank)[tid];
-  }
-  F.hist[tid] = 0;
+  uint64_t wp[2] = {0, 0};  // table entries 2 tid and 2 tid + 1
+  int wr[2] = {0, 0};
+#pragma unroll
+  for (int e = 0; e < 2; ++e)
+    if (2 * tid + e < NA) {
+      wp[e] = ((const SMLM_GLOBAL uint64_t*)P.w_ptrs)[2 * tid + e];
+      if (a.sh.plan.w_rank) wr[e] = ((const SMLM_GLOBAL int32_t*)a.sh.plan.w_rank)[2 * tid + e];
+    }
+  F.hist[2 * tid] = 0;
+  F.hist[2 * tid + 1] = 0;
   if (tid < kTileRows) F.rows16[tid] = -1, F.rseg16[tid] = -1;
   if (tid == 0) F.sel[0] = -1;
   __syncthreads();
   const bool counted = len > 0 && key >= 0 && key < NA;  // ids outside the table own no tile here
   if (counted) atomicAdd(&F.hist[key], len);              // integer adds: the total does not depend on their order
-  F.wtab[tid] = wp;
-  F.rtab[tid] = wr;
+#pragma unroll
+  for (int e = 0; e < 2; ++e) F.wtab[2 * tid + e] = wp[e], F.rtab[2 * tid + e] = wr[e];
   __syncthreads();
   // first tile of every adapter (adapters in ascending order, as the plan's groups are) -> the
   // adapter that owns `tile` and the tile's index among that adapter's tiles
@@ -140,12 +146,15 @@ __global__ __launch_bounds__(kPlanThreads) void shrink_self_planned_kernel(SelfP
       carry = (uint32_t)__builtin_amdgcn_readlane((int)last, kWaveSize - 1);
     }
   } else {
-    const uint32_t nt = tid < NA ? (uint32_t)((F.hist[tid] + kTileRows - 1) / kTileRows) : 0u;
+    // many adapters: one scan over the workgroup, a thread holding two neighbouring adapters
+    const uint32_t t0 = 2 * tid < NA ? (uint32_t)((F.hist[2 * tid] + kTileRows - 1) / kTileRows) : 0u;
+    const uint32_t t1 = 2 * tid + 1 < NA ? (uint32_t)((F.hist[2 * tid + 1] + kTileRows - 1) / kTileRows) : 0u;
     uint32_t last;
-    const uint32_t first = block_scan_excl_1(nt, F.tot_a, &last);
+    const uint32_t first = block_scan_excl_1(t0 + t1, F.tot_a, &last);
     if ((uint32_t)tile >= first && (uint32_t)tile < last) {
-      F.sel[0] = tid;
-      F.sel[1] = tile - (int)first;
+      const int e = (uint32_t)tile >= first + t0 ? 1 : 0;
+      F.sel[0] = 2 * tid + e;
+      F.sel[1] = tile - (int)(first + (e ? t0 : 0u));
     }
     __syncthreads();
     wid = F.sel[0];
@@ -190,7 +199,7 @@ __global__ __launch_bounds__(kPlanThreads) void shrink_self_planned_kernel(SelfP
   const int row = F.rows16[c], rseg = F.rseg16[c];
   if (kOverlay) __syncthreads();  // every wave holds its tile: the scratch turns into the sum's staging area
 
-  // ---- the product, as the sixteen-wave shrink_kernel does it
+  // ---- the product, as the eight-wave shrink_kernel does it
   f32x4 acc[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};

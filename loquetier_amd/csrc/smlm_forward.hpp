@@ -209,7 +209,7 @@ struct ShrinkArgs {
 // slice, 64-column block, tile).  The NW waves of a workgroup take consecutive k
 // ranges; their accumulators are summed through LDS in wave order and written
 // either as an fp32 partial (k split over workgroups, or a consumer that folds)
-// or as the final 16-bit value.  NW = 16 is for decode batches: few tiles, long k.
+// or as the final 16-bit value.  NW = 8 is for decode batches: few tiles, long k.
 template <int DT, int NB, int U, int NW, bool ROWMAJOR, bool DIRECT, bool DROP = false>
 __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
   __shared__ f32x4 red[NW][NB][kWaveSize];
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         if (k + 64 * U < kend) load_batch(k + 64 * U, xa, wa);
         multiply(k + 32 * U, xb, wb);
       }
-    } else {  // sixteen waves share the VGPR file: one batch at a time (k is usually one batch)
+    } else {  // sixteen waves and more share the VGPR file: one batch at a time
 #pragma unroll 1
       for (int k = kbeg; k < kend; k += 32 * U) {
         u32x4 xf[U], wf[NB][U];
@@ -297,7 +297,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         // all NW reads are issued before the first add waits for one (left to itself the
-        // compiler keeps two in flight, and the sixteen-wave kernel spends as long here as
+        // compiler keeps two in flight, and a many-wave kernel spends as long here as
         // in its k loop)
         f32x4 part[NW];
 #pragma unroll

@@ -152,20 +152,23 @@ __device__ __forceinline__ int count_below(const T* keys, T key, int j0, int j1)
 // The workgroup's LDS of the one-launch route, as a struct so that another kernel can lend the
 // same memory to a workgroup that builds a plan (it is only ever reached by name through a
 // reference that the compiler resolves at compile time, never through a stored pointer).
-struct PlanSmallLds {
-  uint64_t K[kPlanSmallSegs], K0[kPlanSmallSegs];
-  int32_t start0[kPlanSmallSegs], len0[kPlanSmallSegs];  // by segment
-  int32_t sseg[kPlanSmallSegs], rowpos[kPlanSmallSegs + 1];  // by sorted position
-  int32_t grow[kPlanSmallSegs + 1], gtile[kPlanSmallSegs + 1], gblk[kPlanSmallSegs + 1];
-  int32_t gseg[kPlanSmallSegs], gid[kPlanSmallSegs];
-  int32_t gpos[kPlanSmallSegs + 1];  // group -> sorted position of its first segment, [NG] = S
+template <int CAP>
+struct PlanSmallLdsT {  // CAP segments, at most 4 * CAP possible tiles
+  uint64_t K[CAP], K0[CAP];
+  int32_t start0[CAP], len0[CAP];  // by segment
+  int32_t sseg[CAP], rowpos[CAP + 1];  // by sorted position
+  int32_t grow[CAP + 1], gtile[CAP + 1], gblk[CAP + 1];
+  int32_t gseg[CAP], gid[CAP];
+  int32_t gpos[CAP + 1];  // group -> sorted position of its first segment, [NG] = S
   uint64_t wave_tot[17];
   int bad_key, wide_key;
 };
+using PlanSmallLds = PlanSmallLdsT<kPlanSmallSegs>;
 
-// the whole plan of a batch of at most kPlanSmallSegs segments, built by the calling workgroup
-// (kPlanThreads threads)
-__device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSmallLds& L) {
+// the whole plan of a batch of at most CAP segments and 4 * CAP possible tiles, built by the
+// calling workgroup (at least as many threads as segments, a multiple of 64)
+template <int CAP>
+__device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSmallLdsT<CAP>& L) {
   auto& K = L.K; auto& K0 = L.K0;
   auto& start0 = L.start0; auto& len0 = L.len0;
   auto& sseg = L.sseg; auto& rowpos = L.rowpos;

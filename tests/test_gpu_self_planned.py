@@ -43,8 +43,9 @@ CASES = [
     ("ragged-empty-uncovered",) + ragged(4, 90, 9, 12) + (12, 0, 16, [(2048, 512), (2048, 256)]),
     ("one-adapter-many-tiles", [0, 300, 301, 640], [5, 5, 5], 8, 700, 32, [(2048, 320)]),
     ("absent-adapters", list(range(0, 200, 2)), [(7 * i) % 600 for i in range(99)], 1024, 198, 8, [(2048, 128)]),
-    ("1024-segments", list(range(0, 1000)) + [1000] * 25, [(i * 37) % 1000 for i in range(1024)], 1000, 1000, 16,
+    ("1024-segments-fall-back", list(range(0, 1000)) + [1000] * 25, [(i * 37) % 1000 for i in range(1024)], 1000, 1000, 16,
      [(2048, 256)]),
+    ("512-segments", list(range(0, 500)) + [500] * 13, [(i * 37) % 300 for i in range(512)], 300, 500, 16, [(2048, 256)]),
     ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
     ("short-k-falls-back", list(range(41)), decode_ids(40, 4, 8), 4, 40, 16, [(512, 256)]),   # four-wave shrink: plan launch first
     ("tile-blocks-fall-back", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 16, [(2048, 320)]),
