@@ -269,7 +269,7 @@ typedef struct smlm_dropout {
  *                  for every later call on the stream) and uses it.  The reference sets its
  *                  problems up inside every call as well (precompute_smlm_forward_args,
  *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  For
- *                  decode batches (T < 1024, S <= 1024, n_weights <= 1024, every h_in >= 2048,
+ *                  decode batches (T < 1024, S <= 512, n_weights <= 1024, every h_in >= 2048,
  *                  no dropout) this costs no launch: the shrink's workgroups derive their own
  *                  tiles from the two arrays while one more workgroup of the same launch writes
  *                  the plan; other batches get the plan launch first.  Adapter ids must lie in
