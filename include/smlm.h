@@ -86,7 +86,9 @@ SMLM_API int smlm_tmp_size(int num_problems, size_t* bytes);
  * table has one entry per adapter -- the gather wa_ptrs[lora_ids] of
  * src/loquetier_src/models/mixed_lora.py:182 done inside the kernel); any other
  * plan makes them read w_ptrs[i] for segment i (one entry per segment).
- * Segments that share a key must share their weights.
+ * Segments that share a key must share their weights.  A negative SMLM_KEY_I32 key marks a
+ * segment that no adapter serves (a request without LoRA in a mixed batch): the forward entry
+ * points leave its rows of y alone (its rows of v are undefined).
  */
 SMLM_API int smlm_plan_size(int T, int S, size_t* bytes);
 SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr,

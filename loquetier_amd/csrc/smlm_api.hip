@@ -200,25 +200,39 @@ int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs
   return launch(shrink_self_planned_kernel<DT, 4, 2>, grid, block, st, a);
 }
 
-// batches this route takes: a decode-size batch (one-workgroup plan, eight-wave shrink),
+template <int DT>
+int launch_self_planned_block_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
+  const dim3 block(kFwdThreads);  // U must match shrink_cfg
+  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4>, grid, block, st, a);
+  return launch(shrink_block_self_planned_kernel<DT, 4, 4>, grid, block, st, a);
+}
+
+// batches this route takes: few enough segments for the plan-building workgroup of the launch
+// (one segment per thread: 512 in the eight-wave decode shrink, 256 in the tile-block shrink),
 // adapter ids that index a table of at most kSelfPlanWeights entries
 bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
-  return tiles_per_wave(T) == 1 && S <= kSelfPlanSegs && nt_max <= 4 * kSelfPlanSegs && n_weights >= 1 &&
-         n_weights <= kSelfPlanWeights && tile_units_max(T, S, n_weights, 1) < kMaxGridY;
+  const int mt = tiles_per_wave(T), segs = mt == 1 ? kSelfPlanSegs : kSelfPlanBlkSegs;
+  return S <= segs && nt_max <= 4 * segs && n_weights >= 1 && n_weights <= kSelfPlanWeights &&
+         tile_units_max(T, S, n_weights, mt) < kMaxGridY;
 }
 
 int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups, const PlanSortArgs& build,
                                hipStream_t st, const ShrinkArgs& a) {
-  if (c.NW * kWaveSize != kSelfPlanThreads || c.MT != 1) return SMLM_ERR_ARG;
+  if (c.MT == 1 && c.NW * kWaveSize != kSelfPlanThreads) return SMLM_ERR_ARG;
+  if (c.MT > 1 && (a.w_kn || c.NW != kFwdWaves)) return SMLM_ERR_ARG;
   SelfPlanArgs sp{};
   sp.sh = a;
   sp.plan = build;
   sp.n_weights = groups;
-  sp.units = tile_units_max(a.T, S, groups, 1);
+  sp.units = tile_units_max(a.T, S, groups, c.MT);
   int rows = 1;
   for (int i = 0; i < a.items.nproj; ++i)
     if (a.items.row_start[i + 1] - a.items.row_start[i] > rows) rows = a.items.row_start[i + 1] - a.items.row_start[i];
   const dim3 grid((unsigned)rows, (unsigned)sp.units + 1u, (unsigned)a.items.nproj);
+  if (c.MT > 1)
+    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16>(c.NB, grid, st, sp)
+                                   : launch_self_planned_block_nb<SMLM_DTYPE_BF16>(c.NB, grid, st, sp);
   if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16>(c.NB, grid, st, sp);
   return launch_self_planned_nb<SMLM_DTYPE_BF16>(c.NB, grid, st, sp);
 }
@@ -725,7 +739,8 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   // A plan still to be built (opts->build_*): decode batches build it inside the shrink launch,
   // every other batch with the plan launch first.
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, S, next_pow2(S)};
-  const bool self_planned = build_s && expand_folds && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max);
+  const bool self_planned = build_s && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max) &&
+                            (tiles_per_wave(T) > 1 || expand_folds);
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, S, st))) return rc;
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,

@@ -1,69 +1,67 @@
-// Decode batches without a plan launch: a shrink whose workgroups find their own tile.
+// Forward shrinks that need no plan launch: their workgroups find their own tiles.
 //
 // A model step usually builds its tile plan once and every layer reuses it.  The first
 // fused forward of a step can skip that launch: the batch's segment table and adapter ids
-// go straight to the decode shrink (eight waves).  Every workgroup derives the tile it would have
-// looked up -- the adapter and the (at most sixteen) rows of tile t, numbered exactly as
-// the plan numbers them -- from the segment table itself, and ONE extra workgroup of the
-// same launch builds the plan proper (the body of plan_small_kernel) for the expand launch
-// that follows and for every later call.  This takes the place of the reference's
-// per-call set-up kernel precompute_smlm_forward_args
-// (kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46), which also runs inside
-// every call there.
+// go straight to the shrink.  Every workgroup derives the unit of work it would have looked
+// up -- the adapter and the rows of tile t (decode batches, eight-wave shrink) or of tile
+// block b (larger batches, tile-block shrink), numbered exactly as the plan numbers them --
+// from the segment table itself, and a few extra workgroups of the same launch build the plan
+// proper (the body of plan_small_kernel, its table writes dealt out among them) for the
+// launches that follow and for every later call.  This takes the place of the reference's per-call set-up kernel
+// precompute_smlm_forward_args (kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46),
+// which also runs inside every call there.
 //
 // Adapter ids are table indices (SMLM_KEY_I32 with ids in [0, n_weights)), so grouping by
 // adapter needs no sort: a histogram of rows per adapter in LDS, a scan over the adapters
-// for the first tile of each, and a scan over the segments of the tile's adapter for its
+// for the first unit of each, and a scan over the segments of the unit's adapter for its
 // rows.  The plan orders groups by ascending id and a group's segments by index, which is
-// what the two scans walk, so tile t here is tile t of the plan.
+// what the two scans walk, so unit u here is unit u of the plan.
 #pragma once
 #include "smlm_forward.hpp"
 #include "smlm_plan.hpp"
 
 namespace smlm {
 
-constexpr int kSelfPlanThreads = 512;   // eight waves, as the decode shrink_kernel
-constexpr int kSelfPlanSegs = 512;      // most segments of the route: one per thread
-constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of the route: two per thread
-constexpr int kSelfPlanWaveScan = 256;  // up to this many, every wave scans the adapters' tile counts by itself
+constexpr int kSelfPlanThreads = 512;   // decode route: eight waves, as the decode shrink_kernel
+constexpr int kSelfPlanSegs = 512;      //   most segments: one per thread
+constexpr int kSelfPlanBlkSegs = 256;   // tile-block route (256 threads): most segments
+constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of either route
+constexpr int kSelfPlanBuilders = 8;     // workgroups of the launch that share the writing of the plan
+constexpr int kSelfPlanWaveScan = 256;  // up to this many, every wave scans the adapters' unit counts by itself
 
 struct SelfPlanArgs {
   ShrinkArgs sh;        // sh.plan is not read (the plan does not exist yet), except w_rank
-  PlanSortArgs plan;    // what the extra workgroup builds; key_kind = SMLM_KEY_I32
+  PlanSortArgs plan;    // what the extra workgroups build; key_kind = SMLM_KEY_I32
   int n_weights;
-  int units;            // tile bound = grid.y - 1; workgroups with blockIdx.y == units: the plan builder
+  int units;            // unit bound = grid.y - 1; workgroups with blockIdx.y == units: the plan builders
 };
 
 // sixteen zero bytes for predicated-off loads (the other kernels read the plan header's)
 __device__ __attribute__((aligned(16))) uint32_t self_plan_zeros[4];
 
-struct SelfPlanScratch {
+// ---- finding a unit of work (UT tiles of one adapter) without a plan ------------------------
+template <int THREADS>
+struct FindLds {
   int32_t hist[kSelfPlanWeights];   // rows per adapter
   uint64_t wtab[kSelfPlanWeights];  // this projection's weight table
   int32_t rtab[kSelfPlanWeights];   // true ranks, when given
-  uint32_t tot_a[8], tot_b[8];      // wave totals of the two scans
-  int32_t rows16[kTileRows], rseg16[kTileRows];
-  int32_t sel[2];                   // adapter of the tile (-1: no such tile), tile's index within the adapter
+  uint32_t tot_a[THREADS / kWaveSize], tot_b[THREADS / kWaveSize];  // wave totals of the two scans
+  int32_t rows[kBlkTiles * kTileRows], rseg[kBlkTiles * kTileRows];
+  int32_t sel[2];                   // adapter of the unit (-1: no such unit), unit's index within the adapter
+};
+struct FindSeg {  // the segment a thread holds
+  int key, s0, len;
+  bool counted;   // has rows and an adapter id inside the table
+};
+struct FoundUnit {
+  int wid;        // adapter (table index), -1: the unit lies past the last one
+  int sub;        // index of the unit among the adapter's units
+  int tiles;      // tiles of the unit (1 .. UT)
 };
 
-// The sum's staging area lies behind the scratch where both fit under the plan builder's LDS
-// (ranks up to 32) and over it otherwise.
-template <int NB>
-struct SelfPlanWork {
-  static constexpr bool kOverlay =
-      sizeof(SelfPlanScratch) + sizeof(f32x4) * 8 * NB * kWaveSize > sizeof(PlanSmallLdsT<kSelfPlanSegs>);
-  SelfPlanScratch find;
-  f32x4 red[kOverlay ? 1 : 8][NB][kWaveSize];
-};
-template <int NB>
-union SelfPlanLds {
-  PlanSmallLdsT<kSelfPlanSegs> plan;  // the plan-building workgroup
-  SelfPlanWork<NB> work;              // the others: finding their tile, then the cross-wave sum
-  f32x4 red[8][NB][kWaveSize];        // ... which reuses the scratch's memory when the two do not fit side by side
-};
-
-// Exclusive prefix of v over the workgroup (8 waves) with ONE barrier: every wave leaves its
-// total, every thread adds the totals of the waves before its own.  `tot` must not be in use.
+// Exclusive prefix of v over the workgroup with ONE barrier: every wave leaves its total,
+// every thread adds the totals of the waves before its own.  `tot` must not be in use.
+template <int THREADS>
 __device__ __forceinline__ uint32_t block_scan_excl_1(uint32_t v, uint32_t* tot, uint32_t* incl_out) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t in_wave = wave_scan_incl_u32(v);
@@ -71,27 +69,157 @@ __device__ __forceinline__ uint32_t block_scan_excl_1(uint32_t v, uint32_t* tot,
   __syncthreads();
   uint32_t before = 0;
 #pragma unroll
-  for (int w = 0; w < 7; ++w) before += w < wave ? tot[w] : 0u;
+  for (int w = 0; w < THREADS / kWaveSize - 1; ++w) before += w < wave ? tot[w] : 0u;
   *incl_out = before + in_wave;
   return before + in_wave - v;
 }
 
+// Which adapter owns unit `unit` (a unit = UT consecutive tiles of one adapter; adapters in
+// ascending order, as the plan's groups are).  Everything global is requested at once; the
+// first barrier (LDS cleared) passes while those loads are on their way.  THREADS >= S.
+template <int THREADS, int UT>
+__device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const PlanSortArgs& pa,
+                                                  const void* const* w_ptrs, const int32_t* w_rank, int NA,
+                                                  int unit, FindSeg* seg) {
+  constexpr int kEnt = kSelfPlanWeights / THREADS;  // table entries a thread holds: kEnt * tid ...
+  const int tid = threadIdx.x, lane = tid & 63;
+  int key = -1, s0 = 0, len = 0;
+  if (tid < pa.S) {
+    key = ((const SMLM_GLOBAL int32_t*)pa.key)[tid];
+    s0 = ((const SMLM_GLOBAL int32_t*)pa.s)[tid];
+    const int s1 = ((const SMLM_GLOBAL int32_t*)pa.s)[tid + 1];
+    len = s1 > s0 ? s1 - s0 : 0;
+  }
+  uint64_t wp[kEnt];
+  int wr[kEnt];
+#pragma unroll
+  for (int e = 0; e < kEnt; ++e) {
+    wp[e] = 0, wr[e] = 0;
+    if (kEnt * tid + e < NA) {
+      wp[e] = ((const SMLM_GLOBAL uint64_t*)w_ptrs)[kEnt * tid + e];
+      if (w_rank) wr[e] = ((const SMLM_GLOBAL int32_t*)w_rank)[kEnt * tid + e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kEnt; ++e) F.hist[kEnt * tid + e] = 0;
+  if (tid < UT * kTileRows) F.rows[tid] = -1, F.rseg[tid] = -1;
+  if (tid == 0) F.sel[0] = -1;
+  __syncthreads();
+  const bool counted = len > 0 && key >= 0 && key < NA;  // ids outside the table own no unit here
+  if (counted) atomicAdd(&F.hist[key], len);              // integer adds: the total does not depend on their order
+#pragma unroll
+  for (int e = 0; e < kEnt; ++e) F.wtab[kEnt * tid + e] = wp[e], F.rtab[kEnt * tid + e] = wr[e];
+  __syncthreads();
+  *seg = FindSeg{key, s0, len, counted};
+
+  auto units_of = [&](int a) -> uint32_t {
+    return a < NA ? (uint32_t)((F.hist[a] + UT * kTileRows - 1) / (UT * kTileRows)) : 0u;
+  };
+  FoundUnit u{-1, 0, 0};
+  if (NA <= kSelfPlanWaveScan) {
+    // few adapters: every wave walks the table by itself, 64 adapters a step, and needs no barrier
+    uint32_t carry = 0;
+    for (int a0 = 0; a0 < NA; a0 += kWaveSize) {
+      const uint32_t n = units_of(a0 + lane);
+      const uint32_t last = carry + wave_scan_incl_u32(n), first = last - n;
+      const uint64_t hit = __ballot((uint32_t)unit >= first && (uint32_t)unit < last);
+      if (hit) {  // uniform over the wave; at most one lane
+        const int l = __builtin_ctzll(hit);
+        u.wid = a0 + l;
+        u.sub = unit - (int)__builtin_amdgcn_readlane((int)first, l);
+        break;
+      }
+      carry = (uint32_t)__builtin_amdgcn_readlane((int)last, kWaveSize - 1);
+    }
+  } else {
+    // many adapters: one scan over the workgroup, a thread holding kEnt neighbouring adapters
+    uint32_t n[kEnt], sum = 0;
+#pragma unroll
+    for (int e = 0; e < kEnt; ++e) n[e] = units_of(kEnt * tid + e), sum += n[e];
+    uint32_t last;
+    uint32_t first = block_scan_excl_1<THREADS>(sum, F.tot_a, &last);
+    if ((uint32_t)unit >= first && (uint32_t)unit < last) {
+#pragma unroll
+      for (int e = 0; e < kEnt; ++e) {
+        if ((uint32_t)unit >= first && (uint32_t)unit < first + n[e]) {
+          F.sel[0] = kEnt * tid + e;
+          F.sel[1] = unit - (int)first;
+        }
+        first += n[e];
+      }
+    }
+    __syncthreads();
+    u.wid = F.sel[0];
+    u.sub = F.sel[1];
+  }
+  if (u.wid >= 0) {
+    const int tiles_a = (F.hist[u.wid] + kTileRows - 1) / kTileRows;
+    u.tiles = tiles_a - UT * u.sub < UT ? tiles_a - UT * u.sub : UT;
+  }
+  return u;
+}
+
+// The rows of the unit, into F.rows / F.rseg (slot 16 w + c = row c of the unit's tile w; -1 =
+// empty): the adapter's rows in segment order, of which the unit holds 16 UT sub ... + 16 UT - 1.
+template <int THREADS, int UT>
+__device__ __forceinline__ void find_rows(FindLds<THREADS>& F, const FindSeg& seg, const FoundUnit& u) {
+  const int q_lo = u.sub * UT * kTileRows;
+  const uint32_t mine = (seg.counted && seg.key == u.wid) ? (uint32_t)seg.len : 0u;
+  uint32_t hi_u;
+  const int lo = (int)block_scan_excl_1<THREADS>(mine, F.tot_b, &hi_u);
+  const int hi = (int)hi_u;
+  const int q0 = lo > q_lo ? lo : q_lo, q1 = hi < q_lo + UT * kTileRows ? hi : q_lo + UT * kTileRows;
+  // every segment that reaches into the unit is written out by its whole wave, a lane a row (a long
+  // segment fills the unit by itself: one lane writing 64 rows in turn is what this avoids)
+  static_assert(UT * kTileRows <= kWaveSize, "a lane per row of the unit");
+  const int lane = threadIdx.x & 63;
+  uint64_t todo = __ballot(q0 < q1);
+  while (todo) {  // uniform over the wave
+    const int l = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    const int b0 = __builtin_amdgcn_readlane(q0, l), b1 = __builtin_amdgcn_readlane(q1, l);
+    const int r0 = __builtin_amdgcn_readlane(seg.s0 + (q0 - lo), l);
+    if (b0 + lane < b1) {
+      F.rows[b0 + lane - q_lo] = r0 + lane;
+      F.rseg[b0 + lane - q_lo] = (int)(threadIdx.x - lane) + l;
+    }
+  }
+  __syncthreads();
+}
+
+// ---- decode batches: the eight-wave shrink_kernel ------------------------------------------
+// The sum's staging area lies behind the finder's LDS where both fit under the plan builder's
+// (ranks up to 32) and over it otherwise.
+template <int NB>
+struct SelfPlanWork {
+  static constexpr bool kOverlay = sizeof(FindLds<kSelfPlanThreads>) + sizeof(f32x4) * 8 * NB * kWaveSize >
+                                   sizeof(PlanSmallLdsT<kSelfPlanSegs>);
+  FindLds<kSelfPlanThreads> find;
+  f32x4 red[kOverlay ? 1 : 8][NB][kWaveSize];
+};
+template <int NB>
+union SelfPlanLds {
+  PlanSmallLdsT<kSelfPlanSegs> plan;  // the plan-building workgroup
+  SelfPlanWork<NB> work;              // the others: finding their tile, then the cross-wave sum
+  f32x4 red[8][NB][kWaveSize];        // ... which reuses the finder's memory when the two do not fit side by side
+};
+
 template <int DT, int NB, int U>
 __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(SelfPlanArgs a) {
-  static_assert(kSelfPlanSegs <= kSelfPlanThreads && kSelfPlanWeights == 2 * kSelfPlanThreads, "entries per thread");
+  static_assert(kSelfPlanSegs <= kSelfPlanThreads, "one segment per thread");
   __shared__ SelfPlanLds<NB> sm;
   constexpr int NW = kSelfPlanThreads / kWaveSize;
   constexpr bool kOverlay = SelfPlanWork<NB>::kOverlay;
   const int tid = threadIdx.x;
-  if ((int)blockIdx.y == a.units) {  // the extra row of the grid: one workgroup builds the plan
-    if (blockIdx.x == 0 && blockIdx.z == 0) plan_small_body(a.plan, sm.plan);
+  if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
+    const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
+    if (part < kSelfPlanBuilders) plan_small_body(a.plan, sm.plan, part, all < kSelfPlanBuilders ? all : kSelfPlanBuilders);
     return;
   }
   const int pj = blockIdx.z, yy = blockIdx.x, tile = blockIdx.y;
   if (yy >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
   const ShrinkProj P = a.sh.p[pj];
-  const int S = a.plan.S, NA = a.n_weights;
-  SelfPlanScratch& F = sm.work.find;
+  FindLds<kSelfPlanThreads>& F = sm.work.find;
   const int wave = tid >> 6, lane = tid & 63;
   const int c = lane & 15, g = lane >> 4;
   const int kz = yy % P.ksplit, zb = yy / P.ksplit;
@@ -100,66 +228,10 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
   const int kend = min(kbeg + P.k_per_wave, P.d_in);
   const uint16_t* zeros = reinterpret_cast<const uint16_t*>(self_plan_zeros);
 
-  // ---- which adapter and which rows make up tile `tile`.  Everything global is requested at
-  // once; the first barrier (LDS cleared) passes while those loads are on their way.
-  int key = -1, s0 = 0, len = 0;
-  if (tid < S) {
-    key = ((const SMLM_GLOBAL int32_t*)a.plan.key)[tid];
-    s0 = ((const SMLM_GLOBAL int32_t*)a.plan.s)[tid];
-    const int s1 = ((const SMLM_GLOBAL int32_t*)a.plan.s)[tid + 1];
-    len = s1 > s0 ? s1 - s0 : 0;
-  }
-  uint64_t wp[2] = {0, 0};  // table entries 2 tid and 2 tid + 1
-  int wr[2] = {0, 0};
-#pragma unroll
-  for (int e = 0; e < 2; ++e)
-    if (2 * tid + e < NA) {
-      wp[e] = ((const SMLM_GLOBAL uint64_t*)P.w_ptrs)[2 * tid + e];
-      if (a.sh.plan.w_rank) wr[e] = ((const SMLM_GLOBAL int32_t*)a.sh.plan.w_rank)[2 * tid + e];
-    }
-  F.hist[2 * tid] = 0;
-  F.hist[2 * tid + 1] = 0;
-  if (tid < kTileRows) F.rows16[tid] = -1, F.rseg16[tid] = -1;
-  if (tid == 0) F.sel[0] = -1;
-  __syncthreads();
-  const bool counted = len > 0 && key >= 0 && key < NA;  // ids outside the table own no tile here
-  if (counted) atomicAdd(&F.hist[key], len);              // integer adds: the total does not depend on their order
-#pragma unroll
-  for (int e = 0; e < 2; ++e) F.wtab[2 * tid + e] = wp[e], F.rtab[2 * tid + e] = wr[e];
-  __syncthreads();
-  // first tile of every adapter (adapters in ascending order, as the plan's groups are) -> the
-  // adapter that owns `tile` and the tile's index among that adapter's tiles
-  int wid = -1, sub = 0;
-  if (NA <= kSelfPlanWaveScan) {
-    // few adapters: every wave walks the table by itself, 64 adapters a step, and needs no barrier
-    uint32_t carry = 0;
-    for (int a0 = 0; a0 < NA; a0 += kWaveSize) {
-      const uint32_t n = a0 + lane < NA ? (uint32_t)((F.hist[a0 + lane] + kTileRows - 1) / kTileRows) : 0u;
-      const uint32_t last = carry + wave_scan_incl_u32(n), first = last - n;
-      const uint64_t hit = __ballot((uint32_t)tile >= first && (uint32_t)tile < last);
-      if (hit) {  // uniform over the wave; at most one lane
-        const int l = __builtin_ctzll(hit);
-        wid = a0 + l;
-        sub = tile - (int)__builtin_amdgcn_readlane((int)first, l);
-        break;
-      }
-      carry = (uint32_t)__builtin_amdgcn_readlane((int)last, kWaveSize - 1);
-    }
-  } else {
-    // many adapters: one scan over the workgroup, a thread holding two neighbouring adapters
-    const uint32_t t0 = 2 * tid < NA ? (uint32_t)((F.hist[2 * tid] + kTileRows - 1) / kTileRows) : 0u;
-    const uint32_t t1 = 2 * tid + 1 < NA ? (uint32_t)((F.hist[2 * tid + 1] + kTileRows - 1) / kTileRows) : 0u;
-    uint32_t last;
-    const uint32_t first = block_scan_excl_1(t0 + t1, F.tot_a, &last);
-    if ((uint32_t)tile >= first && (uint32_t)tile < last) {
-      const int e = (uint32_t)tile >= first + t0 ? 1 : 0;
-      F.sel[0] = 2 * tid + e;
-      F.sel[1] = tile - (int)(first + (e ? t0 : 0u));
-    }
-    __syncthreads();
-    wid = F.sel[0];
-    sub = F.sel[1];
-  }
+  FindSeg seg;
+  const FoundUnit un =
+      find_adapter<kSelfPlanThreads, 1>(F, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tile, &seg);
+  const int wid = un.wid;
   if (wid < 0) return;  // past the last tile; uniform over the workgroup
   const uint16_t* W = reinterpret_cast<const uint16_t*>(F.wtab[wid]);
   int nlim = P.d_out;  // weight rows at or past it are zero padding
@@ -182,22 +254,9 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
   u32x4 wf[NB][U];
   load_w(kbeg, wf);
 
-  // rows of the adapter in segment order: tile j of the adapter holds its rows 16j .. 16j+15
-  const int q_lo = sub * kTileRows;
-  const uint32_t mine = (counted && key == wid) ? (uint32_t)len : 0u;
-  uint32_t hi_u;
-  const int lo = (int)block_scan_excl_1(mine, F.tot_b, &hi_u);
-  {
-    const int hi = (int)hi_u;
-    const int q0 = lo > q_lo ? lo : q_lo, q1 = hi < q_lo + kTileRows ? hi : q_lo + kTileRows;
-    for (int q = q0; q < q1; ++q) {
-      F.rows16[q - q_lo] = s0 + (q - lo);
-      F.rseg16[q - q_lo] = tid;
-    }
-  }
-  __syncthreads();
-  const int row = F.rows16[c], rseg = F.rseg16[c];
-  if (kOverlay) __syncthreads();  // every wave holds its tile: the scratch turns into the sum's staging area
+  find_rows<kSelfPlanThreads, 1>(F, seg, un);
+  const int row = F.rows[c], rseg = F.rseg[c];
+  if (kOverlay) __syncthreads();  // every wave holds its tile: the finder's LDS turns into the sum's staging area
 
   // ---- the product, as the eight-wave shrink_kernel does it
   f32x4 acc[NB];
@@ -242,6 +301,138 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
         *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.sh.T + row) * P.d_out + n) = sum;
       else
         store4<DT>(P.out + (long)row * P.d_out + n, sum, scale, a.sh.beta);
+    }
+  }
+}
+
+// ---- batches of 1024 rows and more: the tile-block shrink_block_kernel ([n][k] weights) ------
+template <int NB, int U>
+struct SelfPlanBlockStage {
+  static constexpr int kPitch = 32 * U + 8;
+  uint16_t wlds[2][16 * NB * kPitch];
+};
+template <int NB, int U>
+union SelfPlanBlockLds {
+  PlanSmallLdsT<kSelfPlanBlkSegs> plan;  // the plan-building workgroup
+  FindLds<kFwdThreads> find;             // the others: first while they find their tile block ...
+  SelfPlanBlockStage<NB, U> stage;       // ... then the staged weight batches
+};
+
+template <int DT, int NB, int U>
+__global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(SelfPlanArgs a) {
+  static_assert(kSelfPlanBlkSegs <= kFwdThreads, "one segment per thread");
+  constexpr int KB = 32 * U;                 // k per batch
+  constexpr int kRowsW = 16 * NB;            // weight rows (output columns) per workgroup
+  constexpr int kPitch = SelfPlanBlockStage<NB, U>::kPitch;
+  constexpr int kPieces = kRowsW * (KB / 8); // 16-byte pieces of one staged batch
+  constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
+  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U> sm;
+  if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
+    const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
+    if (part < kSelfPlanBuilders) plan_small_body(a.plan, sm.plan, part, all < kSelfPlanBuilders ? all : kSelfPlanBuilders);
+    return;
+  }
+  const int pj = blockIdx.z, yy = blockIdx.x, tb = blockIdx.y;
+  if (yy >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
+  const ShrinkProj P = a.sh.p[pj];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const uint16_t* zeros = reinterpret_cast<const uint16_t*>(self_plan_zeros);
+  const int kz = yy % P.ksplit, zb = yy / P.ksplit;
+  const int n0 = zb * 64;
+  const int kbeg = kz * kFwdWaves * P.k_per_wave;
+  const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
+
+  FindSeg seg;
+  const FoundUnit un =
+      find_adapter<kFwdThreads, kBlkTiles>(sm.find, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tb, &seg);
+  if (un.wid < 0) return;  // past the last tile block; uniform over the workgroup
+  const uint16_t* W = reinterpret_cast<const uint16_t*>(sm.find.wtab[un.wid]);
+  int nlim = P.d_out;  // weight rows at or past it are zero padding
+  if (a.sh.plan.w_rank) {
+    const int r8 = (sm.find.rtab[un.wid] + 7) & ~7;
+    nlim = r8 < nlim ? r8 : nlim;
+  }
+  const int ldw = P.ldw;
+  auto load_w = [&](int kb, u32x4 (&st)[kPer]) {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int idx = threadIdx.x + j * kFwdThreads;
+      const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
+      st[j] = ldg16_or(W + (long)(n0 + nl) * ldw + kb + k8, idx < kPieces && n0 + nl < nlim && kb + k8 < kend,
+                       zeros);
+    }
+  };
+  auto stage_w = [&](int buf, const u32x4 (&st)[kPer]) {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int idx = threadIdx.x + j * kFwdThreads;
+      const int r_ = idx / (KB / 8), c_ = (idx % (KB / 8)) * 8;
+      if (idx < kPieces) *reinterpret_cast<u32x4*>(&sm.stage.wlds[buf][r_ * kPitch + c_]) = st[j];
+    }
+  };
+  // the adapter is known: its first weight batch is requested while the rows are still being found
+  u32x4 wst[kPer];
+  load_w(kbeg, wst);
+
+  find_rows<kFwdThreads, kBlkTiles>(sm.find, seg, un);
+  const bool active = wave < un.tiles;
+  const int row = active ? sm.find.rows[wave * kTileRows + c] : -1;
+  const int rseg = active ? sm.find.rseg[wave * kTileRows + c] : -1;
+  const uint16_t* xrow = P.x + (long)(row < 0 ? 0 : row) * P.d_in;
+  auto load_x = [&](int kb, u32x4 (&xf)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = kb + 32 * u + 8 * g;
+      xf[u] = ldg16_or(xrow + kk, row >= 0 && kk < kend, zeros);
+    }
+  };
+
+  f32x4 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- the product, as shrink_block_kernel does it
+  u32x4 xf[U];
+  load_x(kbeg, xf);
+  __syncthreads();  // every wave holds its rows: the finder's LDS turns into the weight staging area
+  stage_w(0, wst);
+  int buf = 0;
+#pragma unroll 1
+  for (int kb = kbeg; kb < kend; kb += KB) {
+    u32x4 xn[U], wn[kPer];
+    load_x(kb + KB, xn);
+    load_w(kb + KB, wn);
+    __syncthreads();  // buffer `buf` is written; buffer `buf ^ 1` is no longer read
+    if (active) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const u32x4 wfrag =
+              *reinterpret_cast<const u32x4*>(&sm.stage.wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
+          acc[nb] = Num<DT>::mfma(wfrag, xf[u], acc[nb]);
+        }
+      }
+    }
+    stage_w(buf ^ 1, wn);
+    buf ^= 1;
+#pragma unroll
+    for (int u = 0; u < U; ++u) xf[u] = xn[u];
+  }
+
+  if (row >= 0) {
+    const bool as_partial = P.ksplit > 1 || P.to_partial;
+    float scale = 1.0f;
+    if (!as_partial && a.sh.seg_scale) scale = a.sh.seg_scale[rseg];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const int n = n0 + 16 * nb + 4 * g;  // lane holds columns n .. n+3 of its token
+      if (n >= P.d_out) continue;
+      if (as_partial)
+        *(SMLM_GLOBAL f32x4*)(P.partial + ((long)kz * a.sh.T + row) * P.d_out + n) = acc[nb];
+      else
+        store4<DT>(P.out + (long)row * P.d_out + n, acc[nb], scale, a.sh.beta);
     }
   }
 }

@@ -154,6 +154,7 @@ __device__ __forceinline__ void pick_tiles(const TileArgs& p, int tb, int* t0, i
     *t0 = packed >> 3;
     *cnt = packed & 7;
     *wid = *cnt ? uload(p.tile_wid, *t0) : -1;
+    if (*wid < 0) *cnt = 0;  // a negative adapter id: rows that no adapter serves
   }
 }
 
@@ -816,6 +817,7 @@ void expand_block_kernel(ExpandArgs a) {
     const int t0 = packed >> 3, cnt = packed & 7;
     if (cnt == 0) continue;  // past the last block (direct mode); uniform over the workgroup
     const int wid = uload(a.plan.tile_wid, t0);
+    if (wid < 0) continue;  // a negative adapter id: rows that no adapter serves
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
     const int ldw = WKN ? P.ldw : rank_ld(a.plan, P.ldw, klim);  // [k][n] weights (A) have whole rows per rank

@@ -167,8 +167,12 @@ using PlanSmallLds = PlanSmallLdsT<kPlanSmallSegs>;
 
 // the whole plan of a batch of at most CAP segments and 4 * CAP possible tiles, built by the
 // calling workgroup (at least as many threads as segments, a multiple of 64)
+// Several workgroups may share the work (part p of nparts): each of them sorts and scans for
+// itself and writes the same small tables, and they deal the per-tile and per-block entries,
+// which take the longest to write, out among themselves.
 template <int CAP>
-__device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSmallLdsT<CAP>& L) {
+__device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSmallLdsT<CAP>& L, int part = 0,
+                                                int nparts = 1) {
   auto& K = L.K; auto& K0 = L.K0;
   auto& start0 = L.start0; auto& len0 = L.len0;
   auto& sseg = L.sseg; auto& rowpos = L.rowpos;
@@ -314,7 +318,8 @@ __device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSm
   __syncthreads();
   // tile blocks; entries past the last one say "no tiles" (kernels launched over an
   // upper bound of the block count stop there without reading the header)
-  for (int b = tid; b < pv.nt_max; b += blockDim.x) {
+  const int first = part * (int)blockDim.x + tid, stride = nparts * (int)blockDim.x;
+  for (int b = first; b < pv.nt_max; b += stride) {
     int packed = 0;
     if (b < n_blocks) {
       const int G = last_le(gblk, NG, b);
@@ -328,8 +333,8 @@ __device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSm
   // fill: one thread per tile slot; tiles past the last one get weight index -1.  The group
   // of a tile comes from the table above and the segment of a row is searched among the
   // group's own segments only, which keeps the chains of dependent LDS reads short.
-  for (int tile = n_tiles + tid; tile < pv.nt_max; tile += blockDim.x) pv.tile_wid[tile] = -1;
-  for (int slot = tid; slot < n_tiles * kTileRows; slot += blockDim.x) {
+  for (int tile = n_tiles + first; tile < pv.nt_max; tile += stride) pv.tile_wid[tile] = -1;
+  for (int slot = first; slot < n_tiles * kTileRows; slot += stride) {
     const int tile = slot / kTileRows, c = slot % kTileRows;
     const int G = gt[tile];
     const int q = grow[G] + (tile - gtile[G]) * kTileRows + c;

@@ -48,7 +48,16 @@ CASES = [
     ("512-segments", list(range(0, 500)) + [500] * 13, [(i * 37) % 300 for i in range(512)], 300, 500, 16, [(2048, 256)]),
     ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
     ("short-k-falls-back", list(range(41)), decode_ids(40, 4, 8), 4, 40, 16, [(512, 256)]),   # four-wave shrink: plan launch first
-    ("tile-blocks-fall-back", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 16, [(2048, 320)]),
+    # 1024 rows and more: the tile-block shrink finds its tile blocks (up to 256 segments)
+    ("tile-blocks", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 16, [(2048, 320)]),
+    ("tile-blocks-finetune-serve", [0, 1024, 2048, 3072, 4096] + list(range(4097, 4225)),
+     [0, 1, 2, 3] + [4 + i % 32 for i in range(128)], 36, 4224, 16, [(4096, 512)]),
+    ("tile-blocks-prefill-mlp", [0, 512, 1024, 1536, 2048] + list(range(2049, 2113)), [i % 16 for i in range(68)], 16, 2112,
+     32, [(1024, 704), (1024, 704), (2752, 256)]),
+    ("tile-blocks-256-segments", [5 * i for i in range(257)], [(i * 7) % 300 for i in range(256)], 300, 1300, 64,
+     [(512, 128)]),
+    ("tile-blocks-257-segments-fall-back", [5 * i for i in range(258)], [(i * 7) % 300 for i in range(257)], 300, 1300, 8,
+     [(512, 128)]),
 ]
 
 
@@ -136,6 +145,52 @@ def test_deferred_plan_is_built_by_other_users_first(K, gpu_device):
     assert p3.built
 
 
+@pytest.mark.parametrize("seed", range(12, 20))
+def test_random_tile_block_batches(K, gpu_device, seed):
+    """The same for batches of 1024 rows and more (tile blocks of up to 64 rows of one adapter)."""
+    rng = np.random.default_rng(800 + seed)
+    d, tdt = gpu_device, [torch.float16, torch.bfloat16][seed % 2]
+    NA = int(rng.choice([2, 9, 64, 100, 300, 1024]))
+    S = int(rng.integers(2, 257))
+    lens = rng.integers(0, 12, S)
+    big = rng.random(S) < 0.08
+    lens[big] = rng.integers(100, 700, int(big.sum()))
+    if lens.sum() < 1024:
+        lens[0] += 1100
+    seg = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ids = rng.integers(0, NA, S).astype(np.int32)
+    ids[rng.random(S) < 0.03] = -1
+    T = int(seg[-1]) + int(rng.integers(0, 40))
+    r = int(rng.choice([8, 16, 32, 64]))
+    h_in, h_out = int(rng.choice([256, 1024])), int(rng.choice([64, 136]))
+    gen = torch.Generator().manual_seed(int(seed))
+    used = sorted(set(int(i) for i in ids if i >= 0))
+    wa = {a: (torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for a in used}
+    wb = {a: (torch.randn(h_out, r, generator=gen) / r ** 0.5).to(tdt).to(d) for a in used}
+    tab = lambda w: torch.tensor([w[a].data_ptr() if a in w else 16 for a in range(NA)], dtype=torch.int64, device=d)
+    ta, tb = tab(wa), tab(wb)
+    x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    y0 = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    seg_t, ids_t = torch.tensor(seg, device=d), torch.tensor(ids, device=d)
+    sc = (torch.rand(S, generator=gen) + 0.5).to(d)
+    nbytes = max(K.SegmentPlan.nbytes(T, S), 64)
+    out = []
+    for defer in (False, True):
+        plan = K.SegmentPlan(seg_t, ids_t, T, buf=torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=d), defer=defer)
+        y, v = y0.clone(), torch.full((T, r), 3.0, dtype=tdt, device=d)
+        K.smlm_lora_forward(y, x, ta, tb, plan, r, seg_scale=sc, beta=1.0, v_out=v)
+        torch.cuda.synchronize()
+        out.append((y, v, plan.buf))
+    served = np.zeros(T, dtype=bool)  # v of rows that no adapter serves is undefined
+    for i in range(S):
+        if ids[i] >= 0:
+            served[seg[i]:seg[i + 1]] = True
+    keep = torch.tensor(served, device=d)
+    assert torch.equal(out[0][0], out[1][0]) and torch.equal(out[0][1][keep], out[1][1][keep])
+    assert torch.equal(out[0][2], out[1][2])
+    assert torch.equal(out[1][0][~keep], y0[~keep]) and not torch.equal(out[1][0][keep], y0[keep])
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_random_decode_batches(K, gpu_device, seed):
     """Random segment tables (empty segments, several rows a segment, uncovered rows, adapters that own
@@ -184,3 +239,31 @@ def test_random_decode_batches(K, gpu_device, seed):
     idle = torch.tensor(~served, device=d)
     assert torch.equal(out[1][0][idle], y0[idle])
     assert not torch.equal(out[1][0][~idle], y0[~idle]) or not served.any()
+
+
+@pytest.mark.parametrize("rows", [40, 400], ids=["single-tiles", "tile-blocks"])
+def test_segments_without_adapter_are_left_alone(K, gpu_device, rows):
+    """A negative adapter id marks a segment that no adapter serves (a request without LoRA in a mixed
+    batch): its rows of y stay as they are, the other segments get the oracle's result."""
+    d, tdt = gpu_device, torch.float16
+    h_in, h_out, r = 256, 192, 16
+    seg = [0, rows, 2 * rows, 2 * rows + 7, 3 * rows + 7, 4 * rows]
+    ids = [1, -1, 0, -1, 1]
+    T = seg[-1]
+    gen = torch.Generator().manual_seed(5)
+    A = [(torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for _ in range(2)]
+    B = [(torch.randn(h_out, r, generator=gen) / r ** 0.5).to(tdt).to(d) for _ in range(2)]
+    x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    y0 = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    plan = K.SegmentPlan(torch.tensor(seg, dtype=torch.int32, device=d), torch.tensor(ids, dtype=torch.int32, device=d), T)
+    y = y0.clone()
+    K.smlm_lora_forward(y, x, ptrs(A, d), ptrs(B, d), plan, r, beta=1.0)
+    from oracle import torch_segments as ref
+    for i, a in enumerate(ids):
+        lo, hi = seg[i], seg[i + 1]
+        if a < 0:
+            assert torch.equal(y[lo:hi], y0[lo:hi])
+        else:
+            want, _ = ref.add_lora_forward(x[lo:hi].cpu(), [A[a].cpu()], [B[a].cpu()], [0, hi - lo],
+                                           y=y0[lo:hi].cpu().clone(), beta=1.0)
+            assert torch.allclose(y[lo:hi].cpu().float(), want.float(), rtol=1e-2, atol=4e-3)
