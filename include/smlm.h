@@ -270,12 +270,13 @@ typedef struct smlm_dropout {
  *                  build_seg_adapter, SMLM_KEY_I32, T, S) would build, writes it to `plan` (valid
  *                  for every later call on the stream) and uses it.  The reference sets its
  *                  problems up inside every call as well (precompute_smlm_forward_args,
- *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  For
- *                  decode batches (T < 1024, S <= 512, n_weights <= 1024, every h_in >= 2048,
- *                  no dropout) this costs no launch: the shrink's workgroups derive their own
- *                  tiles from the two arrays while one more workgroup of the same launch writes
- *                  the plan; other batches get the plan launch first.  Adapter ids must lie in
- *                  [0, n_weights); stages must include SMLM_STAGE_SHRINK.
+ *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  With
+ *                  n_weights <= 1024, no dropout and either T < 1024, S <= 512 and every
+ *                  h_in >= 2048, or T >= 1024, S <= 256 and T / 16 + S < 1024, this costs no
+ *                  launch: the shrink's workgroups derive their own tiles from the two arrays
+ *                  while a few more workgroups of the same launch write the plan; other batches
+ *                  get the plan launch first.  Adapter ids must lie below n_weights (negative:
+ *                  no adapter, see the tile plan above); stages must include SMLM_STAGE_SHRINK.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;
