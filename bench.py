@@ -468,7 +468,8 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         fwd(st)
         if P:
             if build_plan or "bplan" not in st:
-                st["bplan"] = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"])
+                st["bplan"] = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"],
+                                            defer=not args.plan_launch)
             bplan = st["bplan"]
             for i, d in enumerate(st["proj"]):
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],

@@ -264,7 +264,7 @@ typedef struct smlm_dropout {
  *                  rank-8 adapter beside rank-64 ones then costs 16 bytes of B per output
  *                  column instead of a 128-byte line.  Results equal the padded computation
  *                  bit for bit; v, dV and the workspace keep the launch's rank r.
- *   build_seg_indptr, build_seg_adapter (smlm_lora_fwd_multi_ex only; both or neither):
+ *   build_seg_indptr, build_seg_adapter (both or neither):
  *                  `plan` is a buffer of smlm_plan_size(T, S) bytes that holds NO plan yet; the
  *                  call builds the plan smlm_plan_build(plan, ..., build_seg_indptr,
  *                  build_seg_adapter, SMLM_KEY_I32, T, S) would build, writes it to `plan` (valid
@@ -277,6 +277,9 @@ typedef struct smlm_dropout {
  *                  while a few more workgroups of the same launch write the plan; other batches
  *                  get the plan launch first.  Adapter ids must lie below n_weights (negative:
  *                  no adapter, see the tile plan above); stages must include SMLM_STAGE_SHRINK.
+ *                  smlm_lora_bwd_ex takes the pair (part_indptr, part_adapter) the same way and
+ *                  builds its plan inside the dV launch when n_rows >= 1024, P <= 256, v is given
+ *                  and there is no dropout.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;

@@ -200,12 +200,12 @@ int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs
   return launch(shrink_self_planned_kernel<DT, 4, 2>, grid, block, st, a);
 }
 
-template <int DT>
+template <int DT, bool WKN>
 int launch_self_planned_block_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
   const dim3 block(kFwdThreads);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4>, grid, block, st, a);
-  return launch(shrink_block_self_planned_kernel<DT, 4, 4>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4, WKN>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4, WKN>, grid, block, st, a);
+  return launch(shrink_block_self_planned_kernel<DT, 4, 4, WKN>, grid, block, st, a);
 }
 
 // batches this route takes: few enough segments for the plan-building workgroup of the launch
@@ -220,7 +220,7 @@ bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
 int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups, const PlanSortArgs& build,
                                hipStream_t st, const ShrinkArgs& a) {
   if (c.MT == 1 && c.NW * kWaveSize != kSelfPlanThreads) return SMLM_ERR_ARG;
-  if (c.MT > 1 && (a.w_kn || c.NW != kFwdWaves)) return SMLM_ERR_ARG;
+  if (c.MT > 1 && c.NW != kFwdWaves) return SMLM_ERR_ARG;
   SelfPlanArgs sp{};
   sp.sh = a;
   sp.plan = build;
@@ -230,9 +230,12 @@ int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups,
   for (int i = 0; i < a.items.nproj; ++i)
     if (a.items.row_start[i + 1] - a.items.row_start[i] > rows) rows = a.items.row_start[i + 1] - a.items.row_start[i];
   const dim3 grid((unsigned)rows, (unsigned)sp.units + 1u, (unsigned)a.items.nproj);
+  if (c.MT > 1 && a.w_kn)
+    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16, true>(c.NB, grid, st, sp)
+                                   : launch_self_planned_block_nb<SMLM_DTYPE_BF16, true>(c.NB, grid, st, sp);
   if (c.MT > 1)
-    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16>(c.NB, grid, st, sp)
-                                   : launch_self_planned_block_nb<SMLM_DTYPE_BF16>(c.NB, grid, st, sp);
+    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16, false>(c.NB, grid, st, sp)
+                                   : launch_self_planned_block_nb<SMLM_DTYPE_BF16, false>(c.NB, grid, st, sp);
   if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16>(c.NB, grid, st, sp);
   return launch_self_planned_nb<SMLM_DTYPE_BF16>(c.NB, grid, st, sp);
 }
@@ -844,6 +847,16 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   PlanView pv{};
   plan_carve(const_cast<void*>(plan), n_rows, P, &pv);
 
+  // A plan still to be built (opts->build_*): the dV shrink builds it inside its launch when it is
+  // the first launch to use it (tile-block route, v given, no dropout); else the plan launch first.
+  const int32_t* build_s = opts ? opts->build_seg_indptr : nullptr;
+  const int32_t* build_k = opts ? opts->build_seg_adapter : nullptr;
+  if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
+  PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, P, next_pow2(P)};
+  const bool self_planned = build_s && v && !drop.seg_p && tiles_per_wave(n_rows) > 1 && r <= 64 &&
+                            self_planned_ok(n_rows, P, NA, pv.nt_max);
+  if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, P, st))) return rc;
+
   // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The
   // tile-block kernels (1024 rows and more) read the weights as they lie in memory; smaller
   // batches work on transposed copies At [h_in, r], Bt [r, h_out] made here.
@@ -886,7 +899,8 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   const void* const* btp = in_place ? b_ptrs : bt_ptrs;
   const int b_ld = in_place ? r : h_out;
   if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
-                       0.0f, nullptr, st, true, in_place, nullptr, w_rank, in_place ? packed : 0)))
+                       0.0f, nullptr, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
+                       self_planned ? &build : nullptr)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5

@@ -305,28 +305,29 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
   }
 }
 
-// ---- batches of 1024 rows and more: the tile-block shrink_block_kernel ([n][k] weights) ------
-template <int NB, int U>
+// ---- batches of 1024 rows and more: the tile-block shrink_block_kernel ------------------------
+// WKN: the weights are stored [k][n], as B is for the backward's dV = dY B.
+template <int NB, int U, bool WKN>
 struct SelfPlanBlockStage {
-  static constexpr int kPitch = 32 * U + 8;
-  uint16_t wlds[2][16 * NB * kPitch];
+  static constexpr int kPitch = WKN ? 16 * NB + 8 : 32 * U + 8;
+  uint16_t wlds[2][(WKN ? 32 * U : 16 * NB) * kPitch];
 };
-template <int NB, int U>
+template <int NB, int U, bool WKN>
 union SelfPlanBlockLds {
-  PlanSmallLdsT<kSelfPlanBlkSegs> plan;  // the plan-building workgroup
+  PlanSmallLdsT<kSelfPlanBlkSegs> plan;  // the plan-building workgroups
   FindLds<kFwdThreads> find;             // the others: first while they find their tile block ...
-  SelfPlanBlockStage<NB, U> stage;       // ... then the staged weight batches
+  SelfPlanBlockStage<NB, U, WKN> stage;  // ... then the staged weight batches
 };
 
-template <int DT, int NB, int U>
+template <int DT, int NB, int U, bool WKN>
 __global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(SelfPlanArgs a) {
   static_assert(kSelfPlanBlkSegs <= kFwdThreads, "one segment per thread");
   constexpr int KB = 32 * U;                 // k per batch
   constexpr int kRowsW = 16 * NB;            // weight rows (output columns) per workgroup
-  constexpr int kPitch = SelfPlanBlockStage<NB, U>::kPitch;
+  constexpr int kPitch = SelfPlanBlockStage<NB, U, WKN>::kPitch;
   constexpr int kPieces = kRowsW * (KB / 8); // 16-byte pieces of one staged batch
   constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
-  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U> sm;
+  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U, WKN> sm;
   if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
     const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
     if (part < kSelfPlanBuilders) plan_small_body(a.plan, sm.plan, part, all < kSelfPlanBuilders ? all : kSelfPlanBuilders);
@@ -353,23 +354,38 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(
     const int r8 = (sm.find.rtab[un.wid] + 7) & ~7;
     nlim = r8 < nlim ? r8 : nlim;
   }
-  const int ldw = P.ldw;
+  const int ldw = WKN ? rank_ld(a.sh.plan, P.ldw, nlim) : P.ldw;  // [k][n] weights (B) have the rank contiguous
   auto load_w = [&](int kb, u32x4 (&st)[kPer]) {
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int idx = threadIdx.x + j * kFwdThreads;
-      const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
-      st[j] = ldg16_or(W + (long)(n0 + nl) * ldw + kb + k8, idx < kPieces && n0 + nl < nlim && kb + k8 < kend,
-                       zeros);
+      if (WKN) {
+        const int kl = idx / (kRowsW / 8), n8 = (idx % (kRowsW / 8)) * 8;
+        st[j] = ldg16_or(W + (long)(kb + kl) * ldw + n0 + n8, idx < kPieces && n0 + n8 < nlim && kb + kl < kend,
+                         zeros);
+      } else {
+        const int nl = idx / (KB / 8), k8 = (idx % (KB / 8)) * 8;
+        st[j] = ldg16_or(W + (long)(n0 + nl) * ldw + kb + k8, idx < kPieces && n0 + nl < nlim && kb + k8 < kend,
+                         zeros);
+      }
     }
   };
   auto stage_w = [&](int buf, const u32x4 (&st)[kPer]) {
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int idx = threadIdx.x + j * kFwdThreads;
-      const int r_ = idx / (KB / 8), c_ = (idx % (KB / 8)) * 8;
+      const int r_ = WKN ? idx / (kRowsW / 8) : idx / (KB / 8);
+      const int c_ = WKN ? (idx % (kRowsW / 8)) * 8 : (idx % (KB / 8)) * 8;
       if (idx < kPieces) *reinterpret_cast<u32x4*>(&sm.stage.wlds[buf][r_ * kPitch + c_]) = st[j];
     }
+  };
+  auto weight_frag = [&](int buf, int u, int nb) -> u32x4 {
+    if (WKN) {  // as in shrink_block_kernel: four consecutive k rows of one column per transposing read
+      const uint16_t* base = &sm.stage.wlds[buf][(32 * u + 8 * g + (c >> 2)) * kPitch + 16 * nb + 4 * (c & 3)];
+      const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 4 * kPitch);
+      return u32x4{q0[0], q0[1], q1[0], q1[1]};
+    }
+    return *reinterpret_cast<const u32x4*>(&sm.stage.wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
   };
   // the adapter is known: its first weight batch is requested while the rows are still being found
   u32x4 wst[kPer];
@@ -408,11 +424,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const u32x4 wfrag =
-              *reinterpret_cast<const u32x4*>(&sm.stage.wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
-          acc[nb] = Num<DT>::mfma(wfrag, xf[u], acc[nb]);
-        }
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(weight_frag(buf, u, nb), xf[u], acc[nb]);
       }
     }
     stage_w(buf ^ 1, wn);

@@ -135,7 +135,8 @@ class MixedLoraContext:
             if n_parts == 0 or tp[-1] == 0:
                 return None, part_adapter
             plan = kernel.SegmentPlan(torch.tensor(tp, dtype=torch.int32, device=device),
-                                      torch.tensor(part_adapter, dtype=torch.int32, device=device), tp[-1])
+                                      torch.tensor(part_adapter, dtype=torch.int32, device=device), tp[-1],
+                                      defer=True)  # built by the step's first backward call
             return plan, part_adapter
         return self.memo(("backward", device), build)
 

@@ -177,9 +177,9 @@ class SegmentPlan:
     smlm_forward_cutlass.cuh:76-79).
 
     defer=True (plans keyed by int32 adapter ids): nothing is launched here; the first
-    smlm_lora_forward(_multi) call that gets the plan builds it -- for decode batches
-    inside its shrink launch, at no launch of its own -- and every other user builds it
-    with the plan launch first (ensure_built)."""
+    smlm_lora_forward(_multi) or smlm_lora_backward call that gets the plan builds it --
+    for batches of few enough segments inside its first launch, at no launch of its own --
+    and every other user builds it with the plan launch first (ensure_built)."""
 
     def __init__(self, segment: torch.Tensor, seg_key: Optional[torch.Tensor], T: int,
                  buf: Optional[torch.Tensor] = None, defer: bool = False):
@@ -431,7 +431,6 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     if plan.kind != _lib.SMLM_KEY_I32:
         raise RuntimeError("the backward plan must be built from int32 adapter ids")
     n_rows = plan.T
-    plan.ensure_built()
     if dy.size(0) < n_rows or x.size(0) < n_rows or dx.size(0) < n_rows:
         raise RuntimeError("dy, x and dx need at least plan.T rows")
     if dx.dtype != dy.dtype or x.dtype != dy.dtype or (v is not None and v.dtype != dy.dtype):
@@ -450,6 +449,10 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
         opts = _opts(plan, dropout, h_in, adapter_rank, NA, packed_ranks)
+        if not plan.built:  # a deferred plan: this call builds it (inside its first launch where it can)
+            opts = opts or _lib.LoraOpts()
+            opts.build_seg_indptr = plan.segment.data_ptr()
+            opts.build_seg_adapter = plan.seg_key.data_ptr()
         rc = _lib.load().smlm_lora_bwd_ex(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
                                                dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
                                                b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
@@ -457,6 +460,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                                                _ptr(part_scale), None if opts is None else C.byref(opts),
                                                _stream(dev))
     _lib.check(rc, "smlm_lora_backward")
+    plan.built = True
 
 
 def rms_norm(output: torch.Tensor, rms_output: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,

@@ -267,3 +267,55 @@ def test_segments_without_adapter_are_left_alone(K, gpu_device, rows):
             want, _ = ref.add_lora_forward(x[lo:hi].cpu(), [A[a].cpu()], [B[a].cpu()], [0, hi - lo],
                                            y=y0[lo:hi].cpu().clone(), beta=1.0)
             assert torch.allclose(y[lo:hi].cpu().float(), want.float(), rtol=1e-2, atol=4e-3)
+
+
+# name, train partitions, adapter of each, NA, h_in, h_out, rank, v given
+BWD_CASES = [
+    ("tile-blocks", [0, 500, 520, 1300], [2, 0, 2], 3, 256, 192, 16, True),
+    ("finetune-batch", [0, 1024, 2048, 3072, 4096], [0, 1, 2, 3], 4, 1024, 512, 16, True),
+    ("rank64-many-parts", [0] + [37 * i + 900 for i in range(1, 200)], [i % 5 for i in range(199)], 5, 320, 128, 64, True),
+    ("v-recomputed-falls-back", [0, 700, 1400], [0, 1], 2, 256, 128, 32, False),
+    ("single-tiles-fall-back", [0, 35, 90], [0, 1], 2, 192, 320, 16, True),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("case", BWD_CASES, ids=[c[0] for c in BWD_CASES])
+def test_backward_deferred_plan_equals_built_plan(K, gpu_device, case, dt):
+    """The backward builds a deferred plan too -- inside its dV shrink when that is the first launch to
+    need it (1024 rows and more, v given, no dropout), with the plan launch otherwise."""
+    name, tp, part_ad, NA, h_in, h_out, r, with_v = case
+    d, tdt = gpu_device, TDT[dt]
+    n_rows = tp[-1]
+    gen = torch.Generator().manual_seed(71)
+    A = [(torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for _ in range(NA)]
+    B = [(torch.randn(h_out, r, generator=gen) / r ** 0.5).to(tdt).to(d) for _ in range(NA)]
+    x = torch.randn(n_rows, h_in, generator=gen).to(tdt).to(d)
+    g = torch.randn(n_rows, h_out, generator=gen).to(tdt).to(d)
+    tp_t = torch.tensor(tp, dtype=torch.int32, device=d)
+    ad_t = torch.tensor(part_ad, dtype=torch.int32, device=d)
+    sc = (torch.rand(len(part_ad), generator=gen) + 0.5).to(d)
+    nbytes = max(K.SegmentPlan.nbytes(n_rows, len(part_ad)), 64)
+    fresh = lambda: torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=d)
+    built = K.SegmentPlan(tp_t, ad_t, n_rows, buf=fresh())
+    v = None
+    if with_v:
+        v = torch.zeros(n_rows, r, dtype=tdt, device=d)
+        K.smlm_lora_forward(torch.zeros(n_rows, h_out, dtype=tdt, device=d), x, ptrs(A, d), ptrs(B, d), built, r, v_out=v)
+
+    def run(plan):
+        dA, dB = [torch.full_like(a, 5.0) for a in A], [torch.full_like(b, 5.0) for b in B]
+        dx = torch.full((n_rows, h_in), 5.0, dtype=tdt, device=d)
+        K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), g, x, v, ptrs(A, d), ptrs(B, d), plan, r, sc)
+        torch.cuda.synchronize()
+        return [dx] + dA + dB
+
+    ref = run(built)
+    deferred = K.SegmentPlan(tp_t, ad_t, n_rows, buf=fresh(), defer=True)
+    assert not deferred.built
+    out = run(deferred)
+    assert deferred.built and torch.equal(deferred.buf, built.buf)
+    for a, b in zip(ref, out):
+        assert torch.equal(a, b)
+    for a, b in zip(ref, run(deferred)):   # the plan it left serves the next call
+        assert torch.equal(a, b)
