@@ -47,6 +47,8 @@ CASES = [
      [(2048, 256)]),
     ("512-segments", list(range(0, 500)) + [500] * 13, [(i * 37) % 300 for i in range(512)], 300, 500, 16, [(2048, 256)]),
     ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
+    ("rank128", list(range(0, 100, 2)), decode_ids(49, 5, 9), 5, 98, 128, [(4096, 256)]),
+    ("rank72-tile-blocks", [0, 600, 1200, 1210], [1, 0, 1], 2, 1210, 72, [(512, 128)]),
     ("short-k-falls-back", list(range(41)), decode_ids(40, 4, 8), 4, 40, 16, [(512, 256)]),   # four-wave shrink: plan launch first
     # 1024 rows and more: the tile-block shrink finds its tile blocks (up to 256 segments)
     ("tile-blocks", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 16, [(2048, 320)]),
