@@ -321,3 +321,50 @@ def test_backward_deferred_plan_equals_built_plan(K, gpu_device, case, dt):
         assert torch.equal(a, b)
     for a, b in zip(ref, run(deferred)):   # the plan it left serves the next call
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("packed", [False, True], ids=["padded", "packed"])
+@pytest.mark.parametrize("rows", [60, 1400], ids=["single-tiles", "tile-blocks"])
+def test_deferred_plans_with_true_ranks(K, gpu_device, rows, packed):
+    """Adapters of different ranks (padded to one rank, or stored at their own): the routes that build
+    the plan themselves read the rank table as the planned ones do, forward and backward."""
+    d, tdt = gpu_device, torch.bfloat16
+    h_in, h_out, r_pad, NA = 2048, 256, 64, 4
+    ranks = [8, 16, 32, 64]
+    seg = [0, rows // 3, rows // 3 + 1, 2 * rows // 3, rows]
+    ids = [2, 0, 3, 1]
+    T = rows
+    gen = torch.Generator().manual_seed(81)
+    A, B = [], []
+    for a in range(NA):
+        wa, wb = torch.zeros(r_pad, h_in), torch.zeros(h_out, r_pad)
+        wa[:ranks[a]] = torch.randn(ranks[a], h_in, generator=gen) / h_in ** 0.5
+        wb[:, :ranks[a]] = torch.randn(h_out, ranks[a], generator=gen) / ranks[a] ** 0.5
+        if packed:
+            wa, wb = wa[:ranks[a]].contiguous(), wb[:, :ranks[a]].contiguous()
+        A.append(wa.to(tdt).to(d))
+        B.append(wb.to(tdt).to(d))
+    x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    y0 = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    g = torch.randn(T, h_out, generator=gen).to(tdt).to(d)
+    seg_t, ids_t = torch.tensor(seg, dtype=torch.int32, device=d), torch.tensor(ids, dtype=torch.int32, device=d)
+    rk = torch.tensor(ranks, dtype=torch.int32, device=d)
+    sc = torch.full((len(ids),), 0.5, device=d)
+    nbytes = max(K.SegmentPlan.nbytes(T, len(ids)), 64)
+    outs = []
+    for defer in (False, True):
+        fresh = lambda: torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=d)
+        plan = K.SegmentPlan(seg_t, ids_t, T, buf=fresh(), defer=defer)
+        y, v = y0.clone(), torch.zeros(T, r_pad, dtype=tdt, device=d)
+        K.smlm_lora_forward(y, x, ptrs(A, d), ptrs(B, d), plan, r_pad, seg_scale=sc, beta=1.0, v_out=v,
+                            adapter_rank=rk, packed_ranks=packed)
+        bplan = K.SegmentPlan(seg_t, ids_t, T, buf=fresh(), defer=defer)   # every segment trains here
+        dA, dB = [torch.full_like(a, 5.0) for a in A], [torch.full_like(b, 5.0) for b in B]
+        dx = torch.full((T, h_in), 5.0, dtype=tdt, device=d)
+        K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), g, x, v, ptrs(A, d), ptrs(B, d), bplan, r_pad, sc,
+                             adapter_rank=rk, packed_ranks=packed)
+        torch.cuda.synchronize()
+        outs.append([y, v, dx, plan.buf, bplan.buf] + dA + dB)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert not torch.isnan(outs[1][2].float()).any()
