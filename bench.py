@@ -277,45 +277,66 @@ def model_step_bench(args, torch, K):
     w, ctx, layers, tdt = build("cfg2", [])
     cap = torch.cuda.Stream()
 
-    def fwd_step():
-        update(w, ctx, [])
-        for layer, x in layers:
-            layer(x)
-    with torch.no_grad(), torch.cuda.stream(cap):
-        for _ in range(3):
+    def measure_decode(layers):
+        def fwd_step():
+            update(w, ctx, [])
+            for layer, x in layers:
+                layer(x)
+        with torch.no_grad(), torch.cuda.stream(cap):
+            for _ in range(3):
+                fwd_step()
+            torch.cuda.synchronize()
+            n_eager = max(1, min(args.steps, 50))
+            t0 = time.perf_counter()
+            for _ in range(n_eager):
+                fwd_step()
+            host_us = (time.perf_counter() - t0) * 1e6 / (n_eager * len(layers))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_eager):
+                fwd_step()
+            torch.cuda.synchronize()
+            eager_us = (time.perf_counter() - t0) * 1e6 / (n_eager * len(layers))
+        g = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(g, stream=cap):
             fwd_step()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(2):
+            g.replay()
+        a.record()
+        for _ in range(10):
+            g.replay()
+        b.record()
         torch.cuda.synchronize()
-        n_eager = max(1, min(args.steps, 50))
-        t0 = time.perf_counter()
-        for _ in range(n_eager):
-            fwd_step()
-        host_us = (time.perf_counter() - t0) * 1e6 / (n_eager * len(layers))
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(n_eager):
-            fwd_step()
-        torch.cuda.synchronize()
-        eager_us = (time.perf_counter() - t0) * 1e6 / (n_eager * len(layers))
-    g = torch.cuda.CUDAGraph()
-    with torch.no_grad(), torch.cuda.graph(g, stream=cap):
-        fwd_step()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(2):
-        g.replay()
-    a.record()
-    for _ in range(10):
-        g.replay()
-    b.record()
-    torch.cuda.synchronize()
-    graph_us = a.elapsed_time(b) * 1e3 / (10 * len(layers))
+        return host_us, eager_us, a.elapsed_time(b) * 1e3 / (10 * len(layers))
+
+    host_us, eager_us, graph_us = measure_decode(layers)
+    # the same step with q/k/v and gate/up of every layer sharing their input tensor and one shrink
+    # launch (ProjectionGroup: not in the reference, whose layers each run both GEMMs)
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    n_sh = len(shapes)
+    grouped = list(layers)
+    for li in range(n_layers):
+        q, gate = li * n_sh, li * n_sh + 4
+        ProjectionGroup([grouped[q + i][0] for i in range(3)])
+        ProjectionGroup([grouped[gate + i][0] for i in range(2)])
+        for i in (1, 2):
+            grouped[q + i] = (grouped[q + i][0], grouped[q][1])
+        grouped[gate + 1] = (grouped[gate + 1][0], grouped[gate][1])
+    g_host_us, _, g_graph_us = measure_decode(grouped)
     T = w["seg"][-1]
     step_bytes = sum(algorithmic_bytes(w, hi, ho) for _, hi, ho in shapes) * n_layers
     out["decode_forward"] = dict(workload=w["name"], calls_per_step=len(layers), host_us_per_call=round(host_us, 2),
                                  eager_us_per_call=round(eager_us, 2), graph_gpu_us_per_call=round(graph_us, 2),
                                  graph_ms_per_model_step=round(graph_us * len(layers) / 1e3, 4),
                                  step_hbm_gbps=round(step_bytes / (graph_us * len(layers) * 1e-6) / 1e9, 1),
-                                 tokens_per_s=round(T / (graph_us * len(layers) * 1e-6), 1))
-    del layers, g
+                                 tokens_per_s=round(T / (graph_us * len(layers) * 1e-6), 1),
+                                 grouped_qkv_gate_up=dict(host_us_per_call=round(g_host_us, 2),
+                                                          graph_gpu_us_per_call=round(g_graph_us, 2),
+                                                          graph_ms_per_model_step=round(g_graph_us * len(layers) / 1e3, 4),
+                                                          tokens_per_s=round(T / (g_graph_us * len(layers) * 1e-6), 1)))
+    del grouped
+    del layers
     torch.cuda.empty_cache()
 
     # ---- fine-tune + serve batch, forward + backward through autograd (eager)
@@ -342,6 +363,7 @@ def model_step_bench(args, torch, K):
         t1 = time.perf_counter()
         torch.cuda.synchronize()
         t2 = time.perf_counter()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record(cap)
         train_step()
         b.record(cap)

@@ -176,9 +176,12 @@ SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* cons
  * projections may differ in h_in / h_out.  `stages` is SMLM_STAGE_SHRINK |
  * SMLM_STAGE_EXPAND for the whole forward; a caller may also issue the two
  * stages as separate calls with the same arguments and workspace (the expand
- * stage reads what the shrink stage left there).  No counterpart in the
- * reference, which calls its kernel once per linear layer
- * (mixed_lora.py:198-205).
+ * stage reads what the shrink stage left there).  A shrink-only call may pass
+ * NULL for every y, an expand-only call NULL for every x; an expand-only call
+ * skips the projections whose y is NULL, so the projections of one shrink call
+ * (q, k, v of one input) can be expanded one at a time, each when its y is
+ * ready, with the other arguments unchanged.  No counterpart in the reference,
+ * which calls its kernel once per linear layer (mixed_lora.py:198-205).
  */
 SMLM_API int smlm_lora_fwd_multi_workspace_size(int n_proj, int T, const int* h_in, int r,
                                                 size_t* bytes);

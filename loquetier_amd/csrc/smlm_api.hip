@@ -706,8 +706,14 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   if (T == 0 || S == 0) return SMLM_OK;
   if (!plan || !workspace) return SMLM_ERR_ARG;
   if (!aligned16(workspace) || !aligned16(plan)) return SMLM_ERR_ALIGN;
+  // A call that runs one stage only need not name what the other stage works on: a shrink-only
+  // call no y, an expand-only call no x -- and an expand-only call skips the projections whose y
+  // is NULL (the projections of one shrink call may be expanded one at a time, each when its y
+  // is ready).
+  const bool shrink_only = stages == SMLM_STAGE_SHRINK, expand_only = stages == SMLM_STAGE_EXPAND;
   for (int i = 0; i < n_proj; ++i) {
-    if (!y[i] || !x[i] || !a_ptrs[i] || !b_ptrs[i]) return SMLM_ERR_ARG;
+    if (!a_ptrs[i] || !b_ptrs[i]) return SMLM_ERR_ARG;
+    if ((!y[i] && !shrink_only && !expand_only) || (!x[i] && !expand_only)) return SMLM_ERR_ARG;
     if (!aligned16(y[i]) || !aligned16(x[i]) || (v_out && v_out[i] && !aligned16(v_out[i])))
       return SMLM_ERR_ALIGN;
   }

@@ -699,6 +699,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     int pj, yy, tile;
     if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tile)) break;
     const ExpandProj P = a.p[pj];
+    if (!P.y) continue;  // a projection this call leaves out (uniform over the workgroup)
     const int ncol0 = (yy * kFwdWaves + wave) * 32 * NQ;
     if (ncol0 >= P.d_out) continue;
     const int wid = uload(a.plan.tile_wid, tile);
@@ -812,6 +813,7 @@ void expand_block_kernel(ExpandArgs a) {
     int pj, yy, tb;
     if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tb)) break;
     const ExpandProj P = a.p[pj];
+    if (!P.y) continue;  // a projection this call leaves out (uniform over the workgroup)
     const int ncol0 = yy * 32 * NQ;
     const int packed = uload(a.plan.blk, tb);
     const int t0 = packed >> 3, cnt = packed & 7;

@@ -90,6 +90,14 @@ class MixedLoraContext:
             ws = self._workspaces[device] = kernel.Workspace(device)
         return ws
 
+    def group_workspace(self, device: torch.device) -> "kernel.Workspace":
+        """Scratch memory that holds the shrink results of ONE open projection group (ProjectionGroup)
+        between the group's members' calls; apart from `workspace`, which any layer call overwrites."""
+        ws = self._workspaces.get(("group", device))
+        if ws is None:
+            ws = self._workspaces[("group", device)] = kernel.Workspace(device)
+        return ws
+
     def next_dropout_offset(self) -> int:
         """Offset of the next dropout mask stream: a host-side counter, so drawing it waits for nothing
         (eight projections' worth of offsets apart)."""
@@ -296,6 +304,61 @@ class LayerStep:
         return build() if self.memo is None else self.memo(("gather", id(table), id(index)), build)
 
 
+class ProjectionGroup:
+    """Layers that read the SAME input tensor in one pass -- q/k/v of an attention block, gate/up of
+    an MLP.  In a serving step (no training rows) the first member to be called shrinks the input for
+    all of them in one launch (three projections cost little more than one there: the launch is
+    mostly fixed cost), and every member then expands only its own projection onto its base layer's
+    output.  Results are those of the ungrouped calls, bit for bit.  No counterpart in the reference,
+    whose layers each run both GEMMs themselves (mixed_lora.py:198-205).
+
+    The members must be fused layers of one rank, dtype, device and set of true ranks, and must be
+    handed the same tensor object (same storage, not modified in between); a member that is called
+    with anything else, or twice, or after another group has started its pass, simply shrinks
+    again -- grouping never changes a result.  Call ProjectionGroup([q, k, v]) once after the layers
+    are built."""
+
+    def __init__(self, layers):
+        self.layers = list(layers)
+        first = self.layers[0]
+        for l in self.layers:
+            if not (l.fused and l.rank == first.rank and l.dtype == first.dtype and l.device == first.device
+                    and l.packed == first.packed and l.root_context is first.root_context):
+                raise ValueError("the layers of a group must be fused layers of one context, rank, dtype and device")
+            ra, rb = l.adapter_rank, first.adapter_rank
+            if (ra is None) != (rb is None) or (ra is not None and not torch.equal(ra, rb)):
+                raise ValueError("the layers of a group must hold adapters of the same true ranks")
+        for i, l in enumerate(self.layers):
+            l._group = (self, i)
+
+    def dims(self):
+        return [(l.adapters[0].wa.size(1), l.adapters[0].wb.size(0)) for l in self.layers]
+
+    def expand_member(self, i: int, result: torch.Tensor, x: torch.Tensor, seg_scale, plan) -> None:
+        """result += scale * v_i B^T for member i, shrinking x for the whole group first when this is
+        the first member to see x."""
+        first, n = self.layers[0], len(self.layers)
+        ctx = first.root_context
+        ws = ctx.group_workspace(first.device)
+        a_tabs, b_tabs = [l.wa_ptrs for l in self.layers], [l.wb_ptrs for l in self.layers]
+        key = (x.data_ptr(), x._version, tuple(x.shape), x.dtype)
+        state = ctx._step.get("open_group")
+        if state is None or state["group"] is not self or state["key"] != key or i not in state["pending"]:
+            kernel.smlm_lora_forward_multi([None] * n, [x] * n, a_tabs, b_tabs, plan, first.rank, stages=1,
+                                           adapter_rank=first.adapter_rank, workspace=ws, packed_ranks=first.packed,
+                                           dims=self.dims())
+            # (x is kept so that its address cannot be handed to another tensor while the pass is open)
+            state = ctx._step["open_group"] = {"group": self, "key": key, "pending": set(range(n)), "x": x}
+        ys = [None] * n
+        ys[i] = result
+        kernel.smlm_lora_forward_multi(ys, [None] * n, a_tabs, b_tabs, plan, first.rank, seg_scale=seg_scale,
+                                       beta=1.0, stages=2, adapter_rank=first.adapter_rank, workspace=ws,
+                                       packed_ranks=first.packed, dims=self.dims())
+        state["pending"].discard(i)
+        if not state["pending"]:
+            del ctx._step["open_group"]
+
+
 class MixedLoraLinear(nn.Module):
     """A linear layer plus the LoRA terms of every resident adapter
     (reference: mixed_lora.py:86-218)."""
@@ -304,6 +367,7 @@ class MixedLoraLinear(nn.Module):
                  rank: int, dtype: torch.dtype, is_scaled: bool = False, fused: bool = True):
         super().__init__()
         self.root_context = root_context
+        self._group = None  # (ProjectionGroup, index) once the layer shares its input with siblings
         self.base_layer = base_layer
         self.device = base_layer.weight.device
         self.dtype = dtype
@@ -441,6 +505,11 @@ class MixedLoraLinear(nn.Module):
             if not x.is_contiguous():
                 x = x.contiguous()
             plan = ctx.plan(self.device, x.size(0))
+            if self._group is not None and blen.tlen == 0 and not weights and not (
+                    torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):
+                # a serving step: the group's members share one shrink launch
+                self._group[0].expand_member(self._group[1], result, x, seg_scale, plan)
+                return result.to(torch_result_dtype)
             step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed)
             if weights and blen.tlen > 0:
                 step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)

@@ -357,11 +357,15 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
                             v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None,
                             adapter_rank: Optional[torch.Tensor] = None,
-                            workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
+                            workspace: Optional[Workspace] = None, packed_ranks: bool = False,
+                            dims=None) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
     in two launches.  Lists of equal length; entries of xs may be the same tensor.
     stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
-    arguments on the same stream), 3 = both.  dropout: the training rows of x are
+    arguments, workspace and stream), 3 = both.  A shrink-only call may pass None for
+    the ys, an expand-only call None for the xs, and an expand-only call skips the
+    projections whose y is None (q, k and v of one shrink call can be expanded one at a
+    time); `dims` = [(h_in, h_out), ...] then names the shapes the missing tensors have.  dropout: the training rows of x are
     dropped inside the shrink kernel; projection i uses the stream offset + i.
     adapter_rank (int32, indexed like the tables): true ranks of adapters stored
     zero-padded to `rank`; the padding is then not read.  packed_ranks: the adapters are stored
@@ -371,25 +375,36 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
             (v_out is not None and len(v_out) != n):
         raise RuntimeError("between 1 and 8 projections, all lists of one length")
     _check_scale(seg_scale, plan)
+    given = [t for t in list(xs) + list(ys) if t is not None]
+    if not given:
+        raise RuntimeError("nothing to work on: every x and y is None")
+    first = given[0]
     for i in range(n):
-        _check_input(ys[i], "y")
-        _check_input(xs[i], "x")
-        _check_dim(2, ys[i], "y")
-        _check_dim(2, xs[i], "x")
+        if (ys[i] is None and stages == 3) or (xs[i] is None and stages != 2):
+            raise RuntimeError("only a shrink-only call may leave out y, only an expand-only call x")
+        if (xs[i] is None or ys[i] is None) and dims is None:
+            raise RuntimeError("dims=[(h_in, h_out), ...] must name the shapes of the tensors left out")
+        for t, name in ((ys[i], "y"), (xs[i], "x")):
+            if t is None:
+                continue
+            _check_input(t, name)
+            _check_dim(2, t, name)
+            if t.dtype != first.dtype or t.size(0) != plan.T or t.device != first.device:
+                raise RuntimeError("x [T,h_in] and y [T,h_out] must share dtype, device and T with the plan")
+            if dims is not None and t.size(1) != dims[i][0 if name == "x" else 1]:
+                raise RuntimeError(f"{name} of projection {i} does not have the width dims names")
         _check_table(a_ptrs[i], plan, "a_ptrs")
         _check_table(b_ptrs[i], plan, "b_ptrs")
-        if ys[i].dtype != xs[0].dtype or xs[i].dtype != xs[0].dtype or ys[i].size(0) != plan.T \
-                or xs[i].size(0) != plan.T or ys[i].device != xs[0].device:
-            raise RuntimeError("x [T,h_in] and y [T,h_out] must share dtype, device and T with the plan")
         if v_out is not None and v_out[i] is not None:
             vo = v_out[i]
-            if vo.dtype != xs[0].dtype or tuple(vo.shape) != (plan.T, rank) or not vo.is_contiguous():
+            if vo.dtype != first.dtype or tuple(vo.shape) != (plan.T, rank) or not vo.is_contiguous():
                 raise RuntimeError("v_out must be a contiguous [T, rank] tensor of x's dtype")
-    code = _dtype_code(xs[0])
-    dev = xs[0].device
+    code = _dtype_code(first)
+    dev = first.device
     VP, CI = C.c_void_p * n, C.c_int * n
-    h_in = CI(*[x.size(1) for x in xs])
-    h_out = CI(*[y.size(1) for y in ys])
+    widths_in = [dims[i][0] if xs[i] is None else xs[i].size(1) for i in range(n)]
+    h_in = CI(*widths_in)
+    h_out = CI(*[dims[i][1] if ys[i] is None else ys[i].size(1) for i in range(n)])
     vo_arr = None if v_out is None else VP(*[_ptr(t) for t in v_out])
     with torch.cuda.device(dev):
         need = C.c_size_t(0)
@@ -397,7 +412,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
                    "smlm_lora_fwd_multi_workspace_size")
         ws = _workspace(dev, need.value, workspace)
         n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
-        opts = _opts(plan, dropout, [x.size(1) for x in xs], adapter_rank, n_weights, packed_ranks)
+        opts = _opts(plan, dropout, widths_in, adapter_rank, n_weights, packed_ranks)
         if not plan.built:
             if stages & _lib.SMLM_STAGE_SHRINK:  # a deferred plan: this call builds it
                 opts = opts or _lib.LoraOpts()
@@ -406,7 +421,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
             else:
                 plan.ensure_built()
         rc = _lib.load().smlm_lora_fwd_multi_ex(
-            n, VP(*[t.data_ptr() for t in ys]), VP(*[t.data_ptr() for t in xs]), vo_arr,
+            n, VP(*[_ptr(t) for t in ys]), VP(*[_ptr(t) for t in xs]), vo_arr,
             VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
             n_weights, h_in, h_out,
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),

@@ -1,0 +1,143 @@
+"""ProjectionGroup: layers that read one input (q/k/v, gate/up) share one shrink launch in a serving
+step.  Grouping must never change a result: the grouped layers' outputs equal the ungrouped layers'
+bit for bit, whatever order the members are called in and whatever else happens between their calls."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K(gpu_device):
+    from loquetier_amd import _lib
+    from loquetier_amd.ops import _kernels
+    _lib.load()
+    return _kernels
+
+
+def build(d, tdt, widths, h_in, r, NA, seed, true_ranks=None):
+    """One context and, for every width, a pair of identical fused layers: [0] to be grouped, [1] left alone."""
+    from loquetier_amd.mixed_lora import MixedLoraContext, MixedLoraLinear, NamedLoraLayer
+    gen = torch.Generator().manual_seed(seed)
+    ctx = MixedLoraContext()
+    pairs = []
+    for h_out in widths:
+        base = torch.nn.Linear(h_in, h_out, bias=False, device=d, dtype=tdt)
+        base.weight.data.copy_((torch.randn(h_out, h_in, generator=gen) / h_in ** 0.5).to(tdt))
+        base.weight.requires_grad_(False)
+        ads = []
+        for a in range(NA):
+            ra = r if true_ranks is None else true_ranks[a % len(true_ranks)]
+            wa, wb = torch.zeros(r, h_in), torch.zeros(h_out, r)
+            wa[:ra] = torch.randn(ra, h_in, generator=gen) / h_in ** 0.5
+            wb[:, :ra] = torch.randn(h_out, ra, generator=gen) / ra ** 0.5
+            ads.append(NamedLoraLayer(f"a{a}", wa.to(tdt).to(d), wb.to(tdt).to(d), torch.nn.Identity(), 0.5 + a,
+                                      true_rank=None if true_ranks is None else ra))
+        pairs.append([MixedLoraLinear(ctx, base, list(ads), r, tdt, is_scaled=False, fused=True) for _ in range(2)])
+    return ctx, pairs
+
+
+def serve_step(ctx, d, req_ids, req_len):
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.segments import build_segments
+    lora_ids, lora_len, segment = build_segments(req_ids, req_len, d)
+    n_dec = sum(1 for n in req_len if n == 1)
+    blen = BatchLenInfo([], [n for n in req_len if n > 1], n_dec, [], d)
+    ctx.update(blen=blen, lora_ids=lora_ids, lora_len=lora_len, segment=segment, train_idx=[])
+
+
+@pytest.mark.parametrize("case", ["decode-qkv", "prefill-gate-up", "true-ranks"])
+def test_grouped_layers_equal_ungrouped(K, gpu_device, case):
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    d, tdt = gpu_device, torch.float16
+    if case == "decode-qkv":
+        h_in, widths, r, NA, ranks = 2048, [2048, 512, 512], 16, 6, None
+        req_ids, req_len = [int(i) for i in np.random.default_rng(3).integers(0, 6, 70)], [1] * 70
+    elif case == "prefill-gate-up":
+        h_in, widths, r, NA, ranks = 1024, [2752, 2752], 32, 3, None
+        req_ids, req_len = [0, 2, 1, 1, 0], [700, 500, 1, 1, 1]
+    else:
+        h_in, widths, r, NA, ranks = 2048, [256, 256, 128], 64, 4, [8, 16, 32, 64]
+        req_ids, req_len = [3, 0, 1, 2, 2, 1], [40, 1, 1, 1, 30, 1]
+    ctx, pairs = build(d, tdt, widths, h_in, r, NA, 5, ranks)
+    group = ProjectionGroup([p[0] for p in pairs])
+    T = sum(req_len)
+    gen = torch.Generator().manual_seed(9)
+    with torch.no_grad():
+        for step in range(3):                     # several steps: the group's state must not leak across them
+            serve_step(ctx, d, req_ids, req_len)
+            x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+            want = [p[1](x) for p in pairs]
+            order = [(i + step) % len(pairs) for i in range(len(pairs))]   # any order of the members
+            got = [None] * len(pairs)
+            for i in order:
+                got[i] = pairs[i][0](x)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b)
+    assert "open_group" not in ctx._step
+
+
+def test_grouping_survives_misuse(K, gpu_device):
+    """Members called with different tensors, twice, with the input changed in between, or interleaved
+    with another group: every call still gives the ungrouped result."""
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    d, tdt = gpu_device, torch.bfloat16
+    h_in, r, NA = 2048, 16, 4
+    ctx, pairs = build(d, tdt, [256, 256, 384, 384], h_in, r, NA, 6)
+    g1 = ProjectionGroup([pairs[0][0], pairs[1][0]])
+    g2 = ProjectionGroup([pairs[2][0], pairs[3][0]])
+    req_ids, req_len = [1, 0, 3, 2, 1, 0, 0], [1, 1, 1, 1, 1, 1, 17]
+    T = sum(req_len)
+    gen = torch.Generator().manual_seed(10)
+    x1 = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    x2 = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    with torch.no_grad():
+        serve_step(ctx, d, req_ids, req_len)
+        ref = lambda i, x: pairs[i][1](x)
+        grp = lambda i, x: pairs[i][0](x)
+        # a member of one group, then a member of the other, then the first group's second member
+        a0, c0, b0 = grp(0, x1), grp(2, x1), grp(1, x1)
+        assert torch.equal(a0, ref(0, x1)) and torch.equal(c0, ref(2, x1)) and torch.equal(b0, ref(1, x1))
+        # different inputs within one group
+        a1, b1 = grp(0, x1), grp(1, x2)
+        assert torch.equal(a1, ref(0, x1)) and torch.equal(b1, ref(1, x2))
+        # the same member twice
+        d1, d2 = grp(3, x2), grp(3, x2)
+        assert torch.equal(d1, ref(3, x2)) and torch.equal(d2, ref(3, x2))
+        # the input modified in place between the members' calls
+        a2 = grp(0, x1)
+        want_a2 = ref(0, x1)
+        x1.mul_(0.5)
+        b2 = grp(1, x1)
+        assert torch.equal(a2, want_a2) and torch.equal(b2, ref(1, x1))
+        # an ordinary layer call between the members of a group (it uses the context's other workspace)
+        a3, mid, b3 = grp(0, x2), ref(2, x2), grp(1, x2)
+        assert torch.equal(a3, ref(0, x2)) and torch.equal(b3, ref(1, x2)) and torch.equal(mid, ref(2, x2))
+
+
+def test_training_steps_are_not_grouped(K, gpu_device):
+    """With training rows in the batch the grouped layers take the ordinary path (autograd, dropout)."""
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    from loquetier_amd.segments import build_segments
+    d, tdt = gpu_device, torch.bfloat16
+    h_in, r, NA = 512, 16, 3
+    ctx, pairs = build(d, tdt, [256, 256], h_in, r, NA, 7)
+    ProjectionGroup([p[0] for p in pairs])
+    for p in pairs:
+        for l in p:
+            l.set_trainable([1])
+    req_ids, req_len = [1, 0, 2], [24, 1, 1]
+    lora_ids, lora_len, segment = build_segments(req_ids, req_len, d)
+    ctx.update(blen=BatchLenInfo([(1, 24)], [], 2, [], d), lora_ids=lora_ids, lora_len=lora_len, segment=segment,
+               train_idx=[1])
+    x = torch.randn(26, h_in, generator=torch.Generator().manual_seed(1)).to(tdt).to(d)
+    outs = []
+    for k in range(2):
+        xs = x.clone().requires_grad_(True)
+        y = pairs[0][k](xs) .float().sum() + pairs[1][k](xs).float().sum()
+        y.backward()
+        outs.append((xs.grad.clone(), pairs[0][k].get_parameter("lora-1-A").grad.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert "open_group" not in ctx._step
