@@ -111,6 +111,11 @@ def test_plan_on_first_use_argument_validation(lib):
     assert call(o, stages=2) == -1        # the plan is built with the shrink
     assert call(o, T=0) == 0              # empty batch: nothing to build, nothing launched
     assert ctypes.sizeof(lib.LoraOpts) == 40
+    # stage-by-stage calls: only a call that runs one stage may leave out the other stage's tensors
+    full = lambda y, x, stages: L.smlm_lora_fwd_multi(1, VP(y), VP(x), None, VP(p), VP(p), 2, CI(64), CI(64), p, p,
+                                                       1 << 30, 16, 2, 16, 0, 0.0, None, stages, None)
+    assert full(None, p, 3) == -1 and full(p, None, 3) == -1
+    assert full(p, None, 1) == -1                     # the shrink needs x
 
 
 def test_rms_norm_argument_validation_codes(lib):
