@@ -697,11 +697,9 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
     return SMLM_ERR_ARG;
   if (stages < 1 || stages > (SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND)) return SMLM_ERR_ARG;
   if (r & 7) return SMLM_ERR_ALIGN;
-  int max_h_out = 0;
   for (int i = 0; i < n_proj; ++i) {
     if (h_in[i] <= 0 || h_out[i] <= 0) return SMLM_ERR_ARG;
     if ((h_in[i] & 7) || (h_out[i] & 7)) return SMLM_ERR_ALIGN;
-    if (h_out[i] > max_h_out) max_h_out = h_out[i];
   }
   if (T == 0 || S == 0) return SMLM_OK;
   if (!plan || !workspace) return SMLM_ERR_ARG;
@@ -766,12 +764,15 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   ea.seg_scale = seg_scale;
   ea.beta = beta;
   ea.T = T; ea.nt_max = pv.nt_max;
+  int n_exp = 0, exp_h_out = 0;  // an expand-only call launches only the projections it names a y for
   for (int i = 0; i < n_proj; ++i) {
-    ExpandProj& P = ea.p[i];
+    if (!y[i]) continue;
+    ExpandProj& P = ea.p[n_exp++];
     P.y = reinterpret_cast<uint16_t*>(y[i]);
     P.v = reinterpret_cast<const uint16_t*>(v16[i]);
     P.w_ptrs = b_ptrs[i];
     P.d_in = r; P.d_out = h_out[i]; P.ldw = r;
+    if (h_out[i] > exp_h_out) exp_h_out = h_out[i];
     if (expand_folds) {
       P.vpart = partial[i];
       P.vsplit = vsplit[i];
@@ -779,7 +780,8 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
       if (v_out && v_out[i]) P.v_out = reinterpret_cast<uint16_t*>(v_out[i]);
     }
   }
-  return launch_expand(dtype, false, expand_nq(T, max_h_out), tiles_per_wave(T), S, n_weights, n_proj, r,
+  if (n_exp == 0) return SMLM_OK;
+  return launch_expand(dtype, false, expand_nq(T, exp_h_out), tiles_per_wave(T), S, n_weights, n_exp, r,
                        st, ea);
 }
 
