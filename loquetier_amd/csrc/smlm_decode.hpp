@@ -16,6 +16,11 @@
 // for the first unit of each, and a scan over the segments of the unit's adapter for its
 // rows.  The plan orders groups by ascending id and a group's segments by index, which is
 // what the two scans walk, so unit u here is unit u of the plan.
+//
+// The products themselves repeat shrink_kernel / shrink_block_kernel step for step (same MFMA
+// sequence over k, same cross-wave sum): a call that builds its plan here and a call over the
+// finished plan give the same bits, which the tests hold them to.  What differs is the order of
+// the loads -- the weights are requested as soon as the adapter is known, before the rows are.
 #pragma once
 #include "smlm_forward.hpp"
 #include "smlm_plan.hpp"
