@@ -345,7 +345,11 @@ def model_step_bench(args, torch, K):
     gen = torch.Generator(device="cpu").manual_seed(12)
     grads = {h: torch.randn(w["seg"][-1], h, generator=gen).to(dev).to(tdt) for h in (4096, 11008)}
 
+    params = [p for layer, _ in layers for p in layer.parameters() if p.requires_grad]
+
     def train_step():
+        for p in params:  # what optimizer.zero_grad() does by default: the backward then hands its buffers over
+            p.grad = None
         update(w, ctx, [0, 1, 2, 3])
         outs = []
         for layer, x in layers:

@@ -103,7 +103,14 @@ def check(code: int, what: str) -> None:
         raise RuntimeError(f"{what}: {strerror(code)} (code {code})")
 
 
+_SIZES = {}  # the size queries are pure functions of their arguments: asked once each
+
+
 def size_query(fn_name: str, *args: int) -> int:
-    out = C.c_size_t(0)
-    check(getattr(load(), fn_name)(*args, C.byref(out)), fn_name)
-    return out.value
+    key = (fn_name,) + args
+    n = _SIZES.get(key)
+    if n is None:
+        out = C.c_size_t(0)
+        check(getattr(load(), fn_name)(*args, C.byref(out)), fn_name)
+        n = _SIZES[key] = out.value
+    return n

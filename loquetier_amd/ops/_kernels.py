@@ -55,6 +55,24 @@ def _stream(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(dev: torch.device):
+    """Context that makes `dev` the current device; nothing to do (and nothing spent) when it already is."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(dev)
+
+
 def _workspace(dev: torch.device, nbytes: int, own: Optional[Workspace] = None) -> torch.Tensor:
     if own is not None:
         buf = own.reserve(nbytes)
@@ -128,7 +146,7 @@ def smlm_forward_cutlass(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, 
     code = _dtype_code(x)
     T = x.size(0)
     dev = tmp.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         need = _lib.size_query("smlm_gemm_workspace_size", T, num_problems, d_in, d_out)
         ws = _workspace(dev, need)
         rc = _lib.load().smlm_gemm(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s.data_ptr(),
@@ -162,7 +180,7 @@ def smlm_forward_cutlass_static(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.T
     code = _dtype_code(x)
     d_in, d_out = x.size(1), y.size(1)
     dev = x.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = _lib.load().smlm_gemm_static(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s.data_ptr(),
                                           x.size(0), num_problems, d_in, d_out,
                                           d_out if is_row_major else d_in, int(bool(is_row_major)), code,
@@ -218,7 +236,7 @@ class SegmentPlan:
         if self.built:
             return
         dev = self.segment.device
-        with torch.cuda.device(dev):
+        with _on(dev):
             rc = _lib.load().smlm_plan_build(self.buf.data_ptr(), self.buf.numel(), self.segment.data_ptr(),
                                              _ptr(self.seg_key), self.kind, self.T, self.S, _stream(dev))
         _lib.check(rc, "smlm_plan_build")
@@ -268,7 +286,7 @@ def smlm_gemm_planned(y: torch.Tensor, x: torch.Tensor, w_ptrs: torch.Tensor, pl
     T, d_in, d_out = x.size(0), x.size(1), y.size(1)
     w_ld = d_out if is_row_major else d_in
     dev = x.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         need = _lib.size_query("smlm_gemm_planned_workspace_size", T, d_in, d_out)
         ws = _workspace(dev, need, workspace)
         rc = _lib.load().smlm_gemm_planned(y.data_ptr(), x.data_ptr(), w_ptrs.data_ptr(), w_ptrs.size(0),
@@ -353,6 +371,21 @@ def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_
                             adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks)
 
 
+_FWD_MULTI_SIZES: Dict[Tuple, int] = {}
+
+
+def _fwd_multi_workspace_size(T: int, widths_in: Tuple[int, ...], rank: int) -> int:
+    key = (T, widths_in, rank)
+    n = _FWD_MULTI_SIZES.get(key)
+    if n is None:
+        need = C.c_size_t(0)
+        arr = (C.c_int * len(widths_in))(*widths_in)
+        _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(len(widths_in), T, arr, rank, C.byref(need)),
+                   "smlm_lora_fwd_multi_workspace_size")
+        n = _FWD_MULTI_SIZES[key] = need.value
+    return n
+
+
 def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
                             seg_scale: Optional[torch.Tensor] = None, beta: float = 0.0,
                             v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None,
@@ -406,11 +439,8 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
     h_in = CI(*widths_in)
     h_out = CI(*[dims[i][1] if ys[i] is None else ys[i].size(1) for i in range(n)])
     vo_arr = None if v_out is None else VP(*[_ptr(t) for t in v_out])
-    with torch.cuda.device(dev):
-        need = C.c_size_t(0)
-        _lib.check(_lib.load().smlm_lora_fwd_multi_workspace_size(n, plan.T, h_in, rank, C.byref(need)),
-                   "smlm_lora_fwd_multi_workspace_size")
-        ws = _workspace(dev, need.value, workspace)
+    with _on(dev):
+        ws = _workspace(dev, _fwd_multi_workspace_size(plan.T, tuple(widths_in), rank), workspace)
         n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
         opts = _opts(plan, dropout, widths_in, adapter_rank, n_weights, packed_ranks)
         if not plan.built:
@@ -458,7 +488,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     code = _dtype_code(dy)
     h_in, h_out = x.size(1), dy.size(1)
     dev = dy.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         need = _lib.size_query("smlm_lora_bwd_workspace_size", n_rows, plan.S, NA, h_in, h_out, rank)
         ws = _workspace(dev, need, workspace)
         if dropout is not None and dropout.rows < n_rows:
@@ -505,7 +535,7 @@ def rms_norm(output: torch.Tensor, rms_output: torch.Tensor, input: torch.Tensor
     if input.dtype not in _DTYPE_CODE or cols % 8 != 0:
         raise RuntimeError(f"No suitable kernel. dtype={input.dtype} columns={cols}")
     dev = input.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = _lib.load().smlm_rms_norm_fwd(output.data_ptr(), rms_output.data_ptr(), input.data_ptr(),
                                            weight.data_ptr(), rows, cols, float(epsilon),
                                            _DTYPE_CODE[input.dtype], _stream(dev))
@@ -528,7 +558,7 @@ def rms_norm_backward(dx: torch.Tensor, dw: torch.Tensor, grad_output: torch.Ten
     rows, cols = x.shape
     code = _dtype_code(x)
     dev = x.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         need = _lib.size_query("smlm_rms_norm_bwd_workspace_size", rows, cols)
         ws = _workspace(dev, need)
         rc = _lib.load().smlm_rms_norm_bwd(dx.data_ptr(), dw.data_ptr(), grad_output.data_ptr(),
@@ -558,7 +588,7 @@ def segments_build(req_adapter: torch.Tensor, req_len: torch.Tensor):
     seg_len = torch.empty(R, dtype=torch.int32, device=dev)
     seg_indptr = torch.empty(R + 1, dtype=torch.int32, device=dev)
     n_seg = torch.empty(2, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = _lib.load().smlm_segments_build(_ptr(req_adapter), _ptr(req_len), R, _ptr(seg_adapter),
                                              _ptr(seg_len), seg_indptr.data_ptr(), n_seg.data_ptr(),
                                              _stream(dev))
