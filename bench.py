@@ -698,6 +698,10 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                    sample=f"{n} whole step{'s' if n > 1 else ''} of the same workload ({el:.1f} s), per-segment "
                           f"torch.matmul in fp32 on {w['dtype']} data (oracle/torch_segments.py)")
 
+    # whether the library builds this batch's plan inside the forward's shrink launch (the limits of
+    # the route, include/smlm.h: segments, possible tiles)
+    in_launch = not args.plan_launch and not (args.dropout and P) and (
+        S <= 512 if T < 1024 else (S <= 256 and T // 16 + S + 1 <= 1024))
     out = {
         "metric": METRIC, "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
@@ -705,7 +709,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         "dtype": "f16" if w["dtype"] == "fp16" else "bf16", "data": "synthetic",
         "config": {"workload": w["name"], "tokens_per_step": T, "segments": S, "adapters": NA, "rank": r,
                    "projections": [f"{n}:{a}->{b}" for n, a, b in w["proj"]],
-                   "buffer_sets_rotated": R, "step_includes": "plan build (" + ("own launch" if args.plan_launch or T >= 1024 else "inside the shrink launch")
+                   "buffer_sets_rotated": R, "step_includes": "plan build (" + ("inside the shrink launch" if in_launch else "own launch")
                    + ") + fused forward per projection"
                    + (" + backward" if P else ""), "graph_replay": not args.eager,
                    "dropout": args.dropout if P else 0.0,
