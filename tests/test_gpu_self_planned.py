@@ -46,6 +46,9 @@ CASES = [
     ("1024-segments-fall-back", list(range(0, 1000)) + [1000] * 25, [(i * 37) % 1000 for i in range(1024)], 1000, 1000, 16,
      [(2048, 256)]),
     ("512-segments", list(range(0, 500)) + [500] * 13, [(i * 37) % 300 for i in range(512)], 300, 500, 16, [(2048, 256)]),
+    ("513-segments-fall-back", list(range(0, 513)) + [513], [(i * 11) % 40 for i in range(513)], 40, 513, 16, [(2048, 128)]),
+    ("1023-rows", [0, 1000, 1023], [1, 0], 2, 1023, 16, [(2048, 128)]),
+    ("1024-rows", [0, 1000, 1024], [1, 0], 2, 1024, 16, [(2048, 128)]),
     ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
     ("rank128", list(range(0, 100, 2)), decode_ids(49, 5, 9), 5, 98, 128, [(4096, 256)]),
     ("rank72-tile-blocks", [0, 600, 1200, 1210], [1, 0, 1], 2, 1210, 72, [(512, 128)]),
