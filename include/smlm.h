@@ -274,7 +274,7 @@ typedef struct smlm_dropout {
  *                  for every later call on the stream) and uses it.  The reference sets its
  *                  problems up inside every call as well (precompute_smlm_forward_args,
  *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  With
- *                  n_weights <= 1024, no dropout and either T < 1024, S <= 512 and every
+ *                  n_weights <= 1024, no dropout and either T < 1024, S <= 1024 and every
  *                  h_in >= 2048, or T >= 1024, S <= 256 and T / 16 + S < 1024, this costs no
  *                  launch: the shrink's workgroups derive their own tiles from the two arrays
  *                  while a few more workgroups of the same launch write the plan; other batches

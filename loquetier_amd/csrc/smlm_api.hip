@@ -192,12 +192,12 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
              : launch_shrink_dt<SMLM_DTYPE_BF16, false>(row_major, c.NB, MT, c.NW, grid, st, a);
 }
 
-template <int DT>
+template <int DT, int THREADS>
 int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
-  const dim3 block(kSelfPlanThreads);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_self_planned_kernel<DT, 1, 4>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_self_planned_kernel<DT, 2, 4>, grid, block, st, a);
-  return launch(shrink_self_planned_kernel<DT, 4, 2>, grid, block, st, a);
+  const dim3 block(THREADS);  // U must match shrink_cfg
+  if (NB == 1) return launch(shrink_self_planned_kernel<DT, 1, 4, THREADS>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_self_planned_kernel<DT, 2, 4, THREADS>, grid, block, st, a);
+  return launch(shrink_self_planned_kernel<DT, 4, 2, THREADS>, grid, block, st, a);
 }
 
 template <int DT, bool WKN>
@@ -208,11 +208,12 @@ int launch_self_planned_block_nb(int NB, dim3 grid, hipStream_t st, const SelfPl
   return launch(shrink_block_self_planned_kernel<DT, 4, 4, WKN>, grid, block, st, a);
 }
 
-// batches this route takes: few enough segments for the plan-building workgroup of the launch
-// (one segment per thread: 512 in the eight-wave decode shrink, 256 in the tile-block shrink),
+// batches this route takes: few enough segments for the plan-building workgroups of the launch
+// (one segment per thread: 512 or 1024 in the decode shrink, 256 in the tile-block shrink),
 // adapter ids that index a table of at most kSelfPlanWeights entries
 bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
-  const int mt = tiles_per_wave(T), segs = mt == 1 ? kSelfPlanSegs : kSelfPlanBlkSegs;
+  const int mt = tiles_per_wave(T);
+  const int segs = mt > 1 ? kSelfPlanBlkSegs : (S <= kSelfPlanThreads ? kSelfPlanThreads : kSelfPlanSegs);
   return S <= segs && nt_max <= 4 * segs && n_weights >= 1 && n_weights <= kSelfPlanWeights &&
          tile_units_max(T, S, n_weights, mt) < kMaxGridY;
 }
@@ -229,15 +230,22 @@ int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups,
   int rows = 1;
   for (int i = 0; i < a.items.nproj; ++i)
     if (a.items.row_start[i + 1] - a.items.row_start[i] > rows) rows = a.items.row_start[i + 1] - a.items.row_start[i];
-  const dim3 grid((unsigned)rows, (unsigned)sp.units + 1u, (unsigned)a.items.nproj);
+  dim3 grid((unsigned)rows, (unsigned)sp.units + 1u, (unsigned)a.items.nproj);
+  if (c.MT == 1 && S > kSelfPlanThreads) {
+    // more segments than the eight-wave workgroup has threads: workgroups of two such groups of
+    // waves, each taking two neighbouring k slices (the caller has checked that the splits are even)
+    grid.x = (unsigned)ceil_div(rows, 2);
+    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_nb<SMLM_DTYPE_F16, 2 * kSelfPlanThreads>(c.NB, grid, st, sp)
+                                   : launch_self_planned_nb<SMLM_DTYPE_BF16, 2 * kSelfPlanThreads>(c.NB, grid, st, sp);
+  }
   if (c.MT > 1 && a.w_kn)
     return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16, true>(c.NB, grid, st, sp)
                                    : launch_self_planned_block_nb<SMLM_DTYPE_BF16, true>(c.NB, grid, st, sp);
   if (c.MT > 1)
     return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16, false>(c.NB, grid, st, sp)
                                    : launch_self_planned_block_nb<SMLM_DTYPE_BF16, false>(c.NB, grid, st, sp);
-  if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16>(c.NB, grid, st, sp);
-  return launch_self_planned_nb<SMLM_DTYPE_BF16>(c.NB, grid, st, sp);
+  if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16, kSelfPlanThreads>(c.NB, grid, st, sp);
+  return launch_self_planned_nb<SMLM_DTYPE_BF16, kSelfPlanThreads>(c.NB, grid, st, sp);
 }
 
 int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
@@ -746,8 +754,10 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   // A plan still to be built (opts->build_*): decode batches build it inside the shrink launch,
   // every other batch with the plan launch first.
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, S, next_pow2(S)};
+  bool even_splits = true;  // (the decode route pairs k slices up beyond 512 segments)
+  for (int i = 0; i < n_proj; ++i) even_splits = even_splits && (vsplit[i] % 2 == 0);
   const bool self_planned = build_s && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max) &&
-                            (tiles_per_wave(T) > 1 || expand_folds);
+                            (tiles_per_wave(T) > 1 || (expand_folds && (S <= kSelfPlanThreads || even_splits)));
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, S, st))) return rc;
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,

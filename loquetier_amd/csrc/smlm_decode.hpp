@@ -27,8 +27,8 @@
 
 namespace smlm {
 
-constexpr int kSelfPlanThreads = 512;   // decode route: eight waves, as the decode shrink_kernel
-constexpr int kSelfPlanSegs = 512;      //   most segments: one per thread
+constexpr int kSelfPlanThreads = 512;   // decode route: eight waves, as the decode shrink_kernel, up to 512 segments;
+constexpr int kSelfPlanSegs = 1024;     //   beyond, up to here, two such groups of waves share a workgroup (one segment per thread)
 constexpr int kSelfPlanBlkSegs = 256;   // tile-block route (256 threads): most segments
 constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of either route
 constexpr int kSelfPlanBuilders = 8;     // workgroups of the launch that share the writing of the plan
@@ -193,39 +193,49 @@ __device__ __forceinline__ void find_rows(FindLds<THREADS>& F, const FindSeg& se
 }
 
 // ---- decode batches: the eight-wave shrink_kernel ------------------------------------------
-// The sum's staging area lies behind the finder's LDS where both fit under the plan builder's
-// (ranks up to 32) and over it otherwise.
-template <int NB>
+// THREADS = 512: a workgroup is the eight waves of shrink_kernel and takes one k slice of its tile.
+// THREADS = 1024 (more than 512 segments; the finder and the plan builders hold a segment per
+// thread): two such groups of eight waves, which take two neighbouring k slices of the tile and sum
+// each for itself -- the same sums as two workgroups of the 512-thread kind.
+// The sums' staging area lies behind the finder's LDS where both fit under the plan builders'
+// and over it otherwise.
+template <int NB, int THREADS>
 struct SelfPlanWork {
-  static constexpr bool kOverlay = sizeof(FindLds<kSelfPlanThreads>) + sizeof(f32x4) * 8 * NB * kWaveSize >
-                                   sizeof(PlanSmallLdsT<kSelfPlanSegs>);
-  FindLds<kSelfPlanThreads> find;
-  f32x4 red[kOverlay ? 1 : 8][NB][kWaveSize];
+  static constexpr int kWaves = THREADS / kWaveSize;
+  static constexpr bool kOverlay = sizeof(FindLds<THREADS>) + sizeof(f32x4) * kWaves * NB * kWaveSize >
+                                   sizeof(PlanSmallLdsT<THREADS>);
+  FindLds<THREADS> find;
+  f32x4 red[kOverlay ? 1 : kWaves][NB][kWaveSize];
 };
-template <int NB>
+template <int NB, int THREADS>
 union SelfPlanLds {
-  PlanSmallLdsT<kSelfPlanSegs> plan;  // the plan-building workgroup
-  SelfPlanWork<NB> work;              // the others: finding their tile, then the cross-wave sum
-  f32x4 red[8][NB][kWaveSize];        // ... which reuses the finder's memory when the two do not fit side by side
+  PlanSmallLdsT<THREADS> plan;                      // the plan-building workgroups
+  SelfPlanWork<NB, THREADS> work;                   // the others: finding their tile, then the cross-wave sums
+  f32x4 red[THREADS / kWaveSize][NB][kWaveSize];    // ... which reuse the finder's memory when the two do not fit side by side
 };
 
-template <int DT, int NB, int U>
-__global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(SelfPlanArgs a) {
-  static_assert(kSelfPlanSegs <= kSelfPlanThreads, "one segment per thread");
-  __shared__ SelfPlanLds<NB> sm;
-  constexpr int NW = kSelfPlanThreads / kWaveSize;
-  constexpr bool kOverlay = SelfPlanWork<NB>::kOverlay;
+template <int DT, int NB, int U, int THREADS>
+__global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanArgs a) {
+  static_assert(THREADS == kSelfPlanThreads || THREADS == 2 * kSelfPlanThreads, "one or two groups of eight waves");
+  __shared__ SelfPlanLds<NB, THREADS> sm;
+  constexpr int NW = kSelfPlanThreads / kWaveSize;  // waves that sum one k slice
+  constexpr int HALVES = THREADS / kSelfPlanThreads;
+  constexpr bool kOverlay = SelfPlanWork<NB, THREADS>::kOverlay;
   const int tid = threadIdx.x;
   if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
     const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
     if (part < kSelfPlanBuilders) plan_small_body(a.plan, sm.plan, part, all < kSelfPlanBuilders ? all : kSelfPlanBuilders);
     return;
   }
-  const int pj = blockIdx.z, yy = blockIdx.x, tile = blockIdx.y;
-  if (yy >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
+  // grid x: (k slice, 64-column block) of the projection, k slices fastest -- in pairs when a
+  // workgroup takes two (the host launches that kind only when every k split is even)
+  const int pj = blockIdx.z, tile = blockIdx.y;
+  if ((int)blockIdx.x * HALVES >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
   const ShrinkProj P = a.sh.p[pj];
-  FindLds<kSelfPlanThreads>& F = sm.work.find;
-  const int wave = tid >> 6, lane = tid & 63;
+  FindLds<THREADS>& F = sm.work.find;
+  const int wave_all = tid >> 6, lane = tid & 63;
+  const int wave = wave_all % NW;           // wave within its group of eight
+  const int yy = (int)blockIdx.x * HALVES + wave_all / NW;
   const int c = lane & 15, g = lane >> 4;
   const int kz = yy % P.ksplit, zb = yy / P.ksplit;
   const int n0 = zb * 64;
@@ -235,7 +245,7 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
 
   FindSeg seg;
   const FoundUnit un =
-      find_adapter<kSelfPlanThreads, 1>(F, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tile, &seg);
+      find_adapter<THREADS, 1>(F, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tile, &seg);
   const int wid = un.wid;
   if (wid < 0) return;  // past the last tile; uniform over the workgroup
   const uint16_t* W = reinterpret_cast<const uint16_t*>(F.wtab[wid]);
@@ -259,7 +269,7 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
   u32x4 wf[NB][U];
   load_w(kbeg, wf);
 
-  find_rows<kSelfPlanThreads, 1>(F, seg, un);
+  find_rows<THREADS, 1>(F, seg, un);
   const int row = F.rows[c], rseg = F.rseg[c];
   if (kOverlay) __syncthreads();  // every wave holds its tile: the finder's LDS turns into the sum's staging area
 
@@ -282,8 +292,9 @@ __global__ __launch_bounds__(kSelfPlanThreads) void shrink_self_planned_kernel(S
       for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(wf[nb][u], xf[u], acc[nb]);
   }
 
-  f32x4 (*red)[NB][kWaveSize] = kOverlay ? sm.red : sm.work.red;  // decided at compile time
-  // cross-wave sum in wave order; wave 0 writes the tile
+  // decided at compile time; every group of eight waves has its own part of the area
+  f32x4 (*red)[NB][kWaveSize] = (kOverlay ? sm.red : sm.work.red) + (wave_all - wave);
+  // cross-wave sum in wave order; the group's first wave writes the tile
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) red[wave][nb][lane] = acc[nb];
   __syncthreads();

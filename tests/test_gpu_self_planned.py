@@ -43,10 +43,10 @@ CASES = [
     ("ragged-empty-uncovered",) + ragged(4, 90, 9, 12) + (12, 0, 16, [(2048, 512), (2048, 256)]),
     ("one-adapter-many-tiles", [0, 300, 301, 640], [5, 5, 5], 8, 700, 32, [(2048, 320)]),
     ("absent-adapters", list(range(0, 200, 2)), [(7 * i) % 600 for i in range(99)], 1024, 198, 8, [(2048, 128)]),
-    ("1024-segments-fall-back", list(range(0, 1000)) + [1000] * 25, [(i * 37) % 1000 for i in range(1024)], 1000, 1000, 16,
+    ("1024-segments", list(range(0, 1000)) + [1000] * 25, [(i * 37) % 1000 for i in range(1024)], 1000, 1000, 16,
      [(2048, 256)]),
     ("512-segments", list(range(0, 500)) + [500] * 13, [(i * 37) % 300 for i in range(512)], 300, 500, 16, [(2048, 256)]),
-    ("513-segments-fall-back", list(range(0, 513)) + [513], [(i * 11) % 40 for i in range(513)], 40, 513, 16, [(2048, 128)]),
+    ("513-segments", list(range(0, 513)) + [513], [(i * 11) % 40 for i in range(513)], 40, 513, 16, [(2048, 128)]),
     ("1023-rows", [0, 1000, 1023], [1, 0], 2, 1023, 16, [(2048, 128)]),
     ("1024-rows", [0, 1000, 1024], [1, 0], 2, 1024, 16, [(2048, 128)]),
     ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
@@ -203,8 +203,8 @@ def test_random_decode_batches(K, gpu_device, seed):
     rng = np.random.default_rng(700 + seed)
     d, tdt = gpu_device, [torch.float16, torch.bfloat16][seed % 2]
     NA = int(rng.choice([1, 3, 40, 64, 65, 200, 257, 900]))
-    S = int(rng.integers(1, 400))
-    lens = rng.integers(0, 4, S)
+    S = int(rng.integers(1, 400)) if seed % 3 else int(rng.integers(513, 1025))   # beyond 512: two groups of waves a workgroup
+    lens = rng.integers(0, 4, S) if S < 400 else rng.integers(0, 2, S)
     lens[rng.random(S) < 0.05] = int(rng.integers(10, 60))
     while lens.sum() >= 1000:
         lens[int(np.argmax(lens))] = 1
