@@ -701,7 +701,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
     # whether the library builds this batch's plan inside the forward's shrink launch (the limits of
     # the route, include/smlm.h: segments, possible tiles)
     in_launch = not args.plan_launch and not (args.dropout and P) and (
-        S <= 1024 if T < 1024 else (S <= 256 and T // 16 + S + 1 <= 1024))
+        S <= 1024 if T < 1024 else (S <= 512 and T // 16 + S + 1 <= 1024))
     out = {
         "metric": METRIC, "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),

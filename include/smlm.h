@@ -275,13 +275,13 @@ typedef struct smlm_dropout {
  *                  problems up inside every call as well (precompute_smlm_forward_args,
  *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  With
  *                  n_weights <= 1024, no dropout and either T < 1024, S <= 1024 and every
- *                  h_in >= 2048, or T >= 1024, S <= 256 and T / 16 + S < 1024, this costs no
+ *                  h_in >= 2048, or T >= 1024, S <= 512 and T / 16 + S < 1024, this costs no
  *                  launch: the shrink's workgroups derive their own tiles from the two arrays
  *                  while a few more workgroups of the same launch write the plan; other batches
  *                  get the plan launch first.  Adapter ids must lie below n_weights (negative:
  *                  no adapter, see the tile plan above); stages must include SMLM_STAGE_SHRINK.
  *                  smlm_lora_bwd_ex takes the pair (part_indptr, part_adapter) the same way and
- *                  builds its plan inside the dV launch when n_rows >= 1024, P <= 256, v is given
+ *                  builds its plan inside the dV launch when n_rows >= 1024, P <= 512, v is given
  *                  and there is no dropout.
  */
 typedef struct smlm_lora_opts {

@@ -200,20 +200,29 @@ int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs
   return launch(shrink_self_planned_kernel<DT, 4, 2, THREADS>, grid, block, st, a);
 }
 
-template <int DT, bool WKN>
+template <int DT, bool WKN, int THREADS>
 int launch_self_planned_block_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
-  const dim3 block(kFwdThreads);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4, WKN>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4, WKN>, grid, block, st, a);
-  return launch(shrink_block_self_planned_kernel<DT, 4, 4, WKN>, grid, block, st, a);
+  const dim3 block(THREADS);  // U must match shrink_cfg
+  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4, WKN, THREADS>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4, WKN, THREADS>, grid, block, st, a);
+  return launch(shrink_block_self_planned_kernel<DT, 4, 4, WKN, THREADS>, grid, block, st, a);
+}
+template <int DT, bool WKN>
+int launch_self_planned_block(int NB, int S, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
+  if (S <= kFwdThreads) return launch_self_planned_block_nb<DT, WKN, kFwdThreads>(NB, grid, st, a);
+  // more segments than the four-wave workgroup has threads: two such groups a workgroup, each
+  // taking one of two neighbouring k slices (the caller has checked that the splits are even)
+  grid.x = (grid.x + 1) / 2;
+  return launch_self_planned_block_nb<DT, WKN, 2 * kFwdThreads>(NB, grid, st, a);
 }
 
 // batches this route takes: few enough segments for the plan-building workgroups of the launch
-// (one segment per thread: 512 or 1024 in the decode shrink, 256 in the tile-block shrink),
+// (one segment per thread: 512 or 1024 in the decode shrink, 256 or 512 in the tile-block shrink),
 // adapter ids that index a table of at most kSelfPlanWeights entries
 bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
   const int mt = tiles_per_wave(T);
-  const int segs = mt > 1 ? kSelfPlanBlkSegs : (S <= kSelfPlanThreads ? kSelfPlanThreads : kSelfPlanSegs);
+  const int segs = mt > 1 ? (S <= kFwdThreads ? kFwdThreads : kSelfPlanBlkSegs)
+                          : (S <= kSelfPlanThreads ? kSelfPlanThreads : kSelfPlanSegs);
   return S <= segs && nt_max <= 4 * segs && n_weights >= 1 && n_weights <= kSelfPlanWeights &&
          tile_units_max(T, S, n_weights, mt) < kMaxGridY;
 }
@@ -239,11 +248,11 @@ int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups,
                                    : launch_self_planned_nb<SMLM_DTYPE_BF16, 2 * kSelfPlanThreads>(c.NB, grid, st, sp);
   }
   if (c.MT > 1 && a.w_kn)
-    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16, true>(c.NB, grid, st, sp)
-                                   : launch_self_planned_block_nb<SMLM_DTYPE_BF16, true>(c.NB, grid, st, sp);
+    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block<SMLM_DTYPE_F16, true>(c.NB, S, grid, st, sp)
+                                   : launch_self_planned_block<SMLM_DTYPE_BF16, true>(c.NB, S, grid, st, sp);
   if (c.MT > 1)
-    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block_nb<SMLM_DTYPE_F16, false>(c.NB, grid, st, sp)
-                                   : launch_self_planned_block_nb<SMLM_DTYPE_BF16, false>(c.NB, grid, st, sp);
+    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block<SMLM_DTYPE_F16, false>(c.NB, S, grid, st, sp)
+                                   : launch_self_planned_block<SMLM_DTYPE_BF16, false>(c.NB, S, grid, st, sp);
   if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16, kSelfPlanThreads>(c.NB, grid, st, sp);
   return launch_self_planned_nb<SMLM_DTYPE_BF16, kSelfPlanThreads>(c.NB, grid, st, sp);
 }
@@ -756,8 +765,10 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, S, next_pow2(S)};
   bool even_splits = true;  // (the decode route pairs k slices up beyond 512 segments)
   for (int i = 0; i < n_proj; ++i) even_splits = even_splits && (vsplit[i] % 2 == 0);
+  // (both routes pair k slices up in one workgroup beyond 512 / 256 segments)
   const bool self_planned = build_s && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max) &&
-                            (tiles_per_wave(T) > 1 || (expand_folds && (S <= kSelfPlanThreads || even_splits)));
+                            (tiles_per_wave(T) > 1 ? (S <= kFwdThreads || even_splits)
+                                                   : (expand_folds && (S <= kSelfPlanThreads || even_splits)));
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, S, st))) return rc;
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
@@ -872,7 +883,8 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, P, next_pow2(P)};
   const bool self_planned = build_s && v && !drop.seg_p && tiles_per_wave(n_rows) > 1 && r <= 64 &&
-                            self_planned_ok(n_rows, P, NA, pv.nt_max);
+                            self_planned_ok(n_rows, P, NA, pv.nt_max) &&
+                            (P <= kFwdThreads || L.cfg_dv.ksplit % 2 == 0);  // (k slices in pairs beyond 256 partitions)
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, P, st))) return rc;
 
   // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The

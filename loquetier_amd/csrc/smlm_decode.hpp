@@ -29,7 +29,7 @@ namespace smlm {
 
 constexpr int kSelfPlanThreads = 512;   // decode route: eight waves, as the decode shrink_kernel, up to 512 segments;
 constexpr int kSelfPlanSegs = 1024;     //   beyond, up to here, two such groups of waves share a workgroup (one segment per thread)
-constexpr int kSelfPlanBlkSegs = 256;   // tile-block route (256 threads): most segments
+constexpr int kSelfPlanBlkSegs = 512;   // tile-block route: most segments (256 threads up to 256 segments, 512 beyond)
 constexpr int kSelfPlanWeights = 1024;  // most table entries (adapters) of either route
 constexpr int kSelfPlanBuilders = 8;     // workgroups of the launch that share the writing of the plan
 constexpr int kSelfPlanWaveScan = 256;  // up to this many, every wave scans the adapters' unit counts by itself
@@ -323,46 +323,58 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
 
 // ---- batches of 1024 rows and more: the tile-block shrink_block_kernel ------------------------
 // WKN: the weights are stored [k][n], as B is for the backward's dV = dY B.
-template <int NB, int U, bool WKN>
+// THREADS = 256: a workgroup is the four waves of shrink_block_kernel and takes one k slice of its
+// tile block.  THREADS = 512 (more than 256 segments; finder and plan builders hold a segment per
+// thread): two such groups of four waves, each with its own staging buffers, which take two
+// neighbouring k slices -- the same sums as two workgroups of the 256-thread kind.  Both groups
+// walk a whole slice's worth of batches (past the end of k they multiply zeros) so that they meet
+// at the same barriers.
+template <int NB, int U, bool WKN, int GROUPS>
 struct SelfPlanBlockStage {
   static constexpr int kPitch = WKN ? 16 * NB + 8 : 32 * U + 8;
-  uint16_t wlds[2][(WKN ? 32 * U : 16 * NB) * kPitch];
+  uint16_t wlds[GROUPS][2][(WKN ? 32 * U : 16 * NB) * kPitch];
 };
-template <int NB, int U, bool WKN>
+template <int NB, int U, bool WKN, int THREADS>
 union SelfPlanBlockLds {
-  PlanSmallLdsT<kSelfPlanBlkSegs> plan;  // the plan-building workgroups
-  FindLds<kFwdThreads> find;             // the others: first while they find their tile block ...
-  SelfPlanBlockStage<NB, U, WKN> stage;  // ... then the staged weight batches
+  PlanSmallLdsT<THREADS> plan;                                  // the plan-building workgroups
+  FindLds<THREADS> find;                                        // the others: first while they find their tile block ...
+  SelfPlanBlockStage<NB, U, WKN, THREADS / kFwdThreads> stage;  // ... then the staged weight batches
 };
 
-template <int DT, int NB, int U, bool WKN>
-__global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(SelfPlanArgs a) {
-  static_assert(kSelfPlanBlkSegs <= kFwdThreads, "one segment per thread");
+template <int DT, int NB, int U, bool WKN, int THREADS>
+__global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(SelfPlanArgs a) {
+  static_assert(THREADS == kFwdThreads || THREADS == 2 * kFwdThreads, "one or two groups of four waves");
+  constexpr int GROUPS = THREADS / kFwdThreads;
   constexpr int KB = 32 * U;                 // k per batch
   constexpr int kRowsW = 16 * NB;            // weight rows (output columns) per workgroup
-  constexpr int kPitch = SelfPlanBlockStage<NB, U, WKN>::kPitch;
+  constexpr int kPitch = SelfPlanBlockStage<NB, U, WKN, GROUPS>::kPitch;
   constexpr int kPieces = kRowsW * (KB / 8); // 16-byte pieces of one staged batch
   constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
-  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U, WKN> sm;
+  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U, WKN, THREADS> sm;
   if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
     const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
     if (part < kSelfPlanBuilders) plan_small_body(a.plan, sm.plan, part, all < kSelfPlanBuilders ? all : kSelfPlanBuilders);
     return;
   }
-  const int pj = blockIdx.z, yy = blockIdx.x, tb = blockIdx.y;
-  if (yy >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
+  // grid x: (k slice, 64-column block) of the projection, k slices fastest -- in pairs when a
+  // workgroup takes two (the host launches that kind only when every k split is even)
+  const int pj = blockIdx.z, tb = blockIdx.y;
+  if ((int)blockIdx.x * GROUPS >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
   const ShrinkProj P = a.sh.p[pj];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int grp = threadIdx.x / kFwdThreads, tl = threadIdx.x % kFwdThreads;  // group of four waves, thread in it
+  const int wave = tl >> 6, lane = threadIdx.x & 63;
+  const int yy = (int)blockIdx.x * GROUPS + grp;
   const int c = lane & 15, g = lane >> 4;
   const uint16_t* zeros = reinterpret_cast<const uint16_t*>(self_plan_zeros);
   const int kz = yy % P.ksplit, zb = yy / P.ksplit;
   const int n0 = zb * 64;
   const int kbeg = kz * kFwdWaves * P.k_per_wave;
   const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
+  const int kstop = GROUPS > 1 ? kbeg + kFwdWaves * P.k_per_wave : kend;  // the same number of batches for both groups
 
   FindSeg seg;
   const FoundUnit un =
-      find_adapter<kFwdThreads, kBlkTiles>(sm.find, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tb, &seg);
+      find_adapter<THREADS, kBlkTiles>(sm.find, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tb, &seg);
   if (un.wid < 0) return;  // past the last tile block; uniform over the workgroup
   const uint16_t* W = reinterpret_cast<const uint16_t*>(sm.find.wtab[un.wid]);
   int nlim = P.d_out;  // weight rows at or past it are zero padding
@@ -374,7 +386,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(
   auto load_w = [&](int kb, u32x4 (&st)[kPer]) {
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-      const int idx = threadIdx.x + j * kFwdThreads;
+      const int idx = tl + j * kFwdThreads;
       if (WKN) {
         const int kl = idx / (kRowsW / 8), n8 = (idx % (kRowsW / 8)) * 8;
         st[j] = ldg16_or(W + (long)(kb + kl) * ldw + n0 + n8, idx < kPieces && n0 + n8 < nlim && kb + kl < kend,
@@ -389,25 +401,25 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(
   auto stage_w = [&](int buf, const u32x4 (&st)[kPer]) {
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-      const int idx = threadIdx.x + j * kFwdThreads;
+      const int idx = tl + j * kFwdThreads;
       const int r_ = WKN ? idx / (kRowsW / 8) : idx / (KB / 8);
       const int c_ = WKN ? (idx % (kRowsW / 8)) * 8 : (idx % (KB / 8)) * 8;
-      if (idx < kPieces) *reinterpret_cast<u32x4*>(&sm.stage.wlds[buf][r_ * kPitch + c_]) = st[j];
+      if (idx < kPieces) *reinterpret_cast<u32x4*>(&sm.stage.wlds[grp][buf][r_ * kPitch + c_]) = st[j];
     }
   };
   auto weight_frag = [&](int buf, int u, int nb) -> u32x4 {
     if (WKN) {  // as in shrink_block_kernel: four consecutive k rows of one column per transposing read
-      const uint16_t* base = &sm.stage.wlds[buf][(32 * u + 8 * g + (c >> 2)) * kPitch + 16 * nb + 4 * (c & 3)];
+      const uint16_t* base = &sm.stage.wlds[grp][buf][(32 * u + 8 * g + (c >> 2)) * kPitch + 16 * nb + 4 * (c & 3)];
       const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 4 * kPitch);
       return u32x4{q0[0], q0[1], q1[0], q1[1]};
     }
-    return *reinterpret_cast<const u32x4*>(&sm.stage.wlds[buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
+    return *reinterpret_cast<const u32x4*>(&sm.stage.wlds[grp][buf][(16 * nb + c) * kPitch + 32 * u + 8 * g]);
   };
   // the adapter is known: its first weight batch is requested while the rows are still being found
   u32x4 wst[kPer];
   load_w(kbeg, wst);
 
-  find_rows<kFwdThreads, kBlkTiles>(sm.find, seg, un);
+  find_rows<THREADS, kBlkTiles>(sm.find, seg, un);
   const bool active = wave < un.tiles;
   const int row = active ? sm.find.rows[wave * kTileRows + c] : -1;
   const int rseg = active ? sm.find.rseg[wave * kTileRows + c] : -1;
@@ -431,7 +443,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_self_planned_kernel(
   stage_w(0, wst);
   int buf = 0;
 #pragma unroll 1
-  for (int kb = kbeg; kb < kend; kb += KB) {
+  for (int kb = kbeg; kb < kstop; kb += KB) {
     u32x4 xn[U], wn[kPer];
     load_x(kb + KB, xn);
     load_w(kb + KB, wn);

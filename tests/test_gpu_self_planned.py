@@ -61,8 +61,15 @@ CASES = [
      32, [(1024, 704), (1024, 704), (2752, 256)]),
     ("tile-blocks-256-segments", [5 * i for i in range(257)], [(i * 7) % 300 for i in range(256)], 300, 1300, 64,
      [(512, 128)]),
-    ("tile-blocks-257-segments-fall-back", [5 * i for i in range(258)], [(i * 7) % 300 for i in range(257)], 300, 1300, 8,
-     [(512, 128)]),
+    ("tile-blocks-257-segments-odd-split-falls-back", [5 * i for i in range(258)], [(i * 7) % 300 for i in range(257)], 300,
+     1300, 8, [(512, 128)]),
+    # beyond 256 segments: two groups of four waves a workgroup (the k splits must be even)
+    ("tile-blocks-300-segments", [5 * i for i in range(301)], [(i * 7) % 300 for i in range(300)], 300, 1510, 16,
+     [(2048, 128), (4096, 64)]),
+    ("tile-blocks-512-segments", [3 * i for i in range(513)], [(i * 5) % 37 for i in range(512)], 37, 1540, 32,
+     [(2048, 192)]),
+    ("tile-blocks-513-segments-fall-back", [3 * i for i in range(514)], [(i * 5) % 37 for i in range(513)], 37, 1540, 32,
+     [(2048, 192)]),
 ]
 
 
@@ -156,8 +163,8 @@ def test_random_tile_block_batches(K, gpu_device, seed):
     rng = np.random.default_rng(800 + seed)
     d, tdt = gpu_device, [torch.float16, torch.bfloat16][seed % 2]
     NA = int(rng.choice([2, 9, 64, 100, 300, 1024]))
-    S = int(rng.integers(2, 257))
-    lens = rng.integers(0, 12, S)
+    S = int(rng.integers(2, 257)) if seed % 2 else int(rng.integers(257, 513))
+    lens = rng.integers(0, 12, S) if S < 257 else rng.integers(0, 5, S)
     big = rng.random(S) < 0.08
     lens[big] = rng.integers(100, 700, int(big.sum()))
     if lens.sum() < 1024:
@@ -167,7 +174,7 @@ def test_random_tile_block_batches(K, gpu_device, seed):
     ids[rng.random(S) < 0.03] = -1
     T = int(seg[-1]) + int(rng.integers(0, 40))
     r = int(rng.choice([8, 16, 32, 64]))
-    h_in, h_out = int(rng.choice([256, 1024])), int(rng.choice([64, 136]))
+    h_in, h_out = int(rng.choice([256, 1024, 2048])), int(rng.choice([64, 136]))
     gen = torch.Generator().manual_seed(int(seed))
     used = sorted(set(int(i) for i in ids if i >= 0))
     wa = {a: (torch.randn(r, h_in, generator=gen) / h_in ** 0.5).to(tdt).to(d) for a in used}
@@ -279,6 +286,7 @@ BWD_CASES = [
     ("tile-blocks", [0, 500, 520, 1300], [2, 0, 2], 3, 256, 192, 16, True),
     ("finetune-batch", [0, 1024, 2048, 3072, 4096], [0, 1, 2, 3], 4, 1024, 512, 16, True),
     ("rank64-many-parts", [0] + [37 * i + 900 for i in range(1, 200)], [i % 5 for i in range(199)], 5, 320, 128, 64, True),
+    ("300-partitions", [0] + [7 * i + 100 for i in range(1, 301)], [i % 9 for i in range(300)], 9, 256, 2048, 16, True),
     ("v-recomputed-falls-back", [0, 700, 1400], [0, 1], 2, 256, 128, 32, False),
     ("single-tiles-fall-back", [0, 35, 90], [0, 1], 2, 192, 320, 16, True),
 ]
