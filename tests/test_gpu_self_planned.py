@@ -49,6 +49,7 @@ CASES = [
     ("513-segments", list(range(0, 513)) + [513], [(i * 11) % 40 for i in range(513)], 40, 513, 16, [(2048, 128)]),
     ("1023-rows", [0, 1000, 1023], [1, 0], 2, 1023, 16, [(2048, 128)]),
     ("1024-rows", [0, 1000, 1024], [1, 0], 2, 1024, 16, [(2048, 128)]),
+    ("700-segments-ragged-k", list(range(0, 701)), [(i * 3) % 50 for i in range(700)], 50, 700, 16, [(3400, 72), (2048, 64)]),
     ("rank64", list(range(0, 130, 2)), decode_ids(64, 6, 7), 6, 130, 64, [(4096, 512)]),
     ("rank128", list(range(0, 100, 2)), decode_ids(49, 5, 9), 5, 98, 128, [(4096, 256)]),
     ("rank72-tile-blocks", [0, 600, 1200, 1210], [1, 0, 1], 2, 1210, 72, [(512, 128)]),
@@ -66,6 +67,8 @@ CASES = [
     # beyond 256 segments: two groups of four waves a workgroup (the k splits must be even)
     ("tile-blocks-300-segments", [5 * i for i in range(301)], [(i * 7) % 300 for i in range(300)], 300, 1510, 16,
      [(2048, 128), (4096, 64)]),
+    ("tile-blocks-300-segments-ragged-k", [5 * i for i in range(301)], [(i * 7) % 30 for i in range(300)], 30, 1510, 16,
+     [(3400, 72)]),   # four k slices of 1024, the last one 328 long
     ("tile-blocks-512-segments", [3 * i for i in range(513)], [(i * 5) % 37 for i in range(512)], 37, 1540, 32,
      [(2048, 192)]),
     ("tile-blocks-513-segments-fall-back", [3 * i for i in range(514)], [(i * 5) % 37 for i in range(513)], 37, 1540, 32,
