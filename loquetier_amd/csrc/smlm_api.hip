@@ -971,6 +971,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   wa.pitch = L.pitch;
   wa.h_in = h_in; wa.h_out = h_out; wa.r = r;
   wa.chunks_a = ceil_div(h_in, kWgCols);
+  wa.n_parts = P;
   wa.grp_seg = pv.grp_seg;
   wa.w_rank = w_rank;
   wa.packed = packed;

@@ -91,6 +91,7 @@ struct WgradArgs {
   void* const* db_ptrs;  // [NA] -> [h_out, r]
   long pitch;
   int h_in, h_out, r, chunks_a;  // chunks_a = ceil(h_in/64): blockIdx.x below it works on dA
+  int n_parts;             // partitions the plan was laid out for (>= 1): its group tables hold n_parts + 1 entries
   const int32_t* w_rank;   // optional [NA]: true rank of each adapter (rows of dV / v past it are zero padding)
   int packed;              // with w_rank: dA_a [r_a, h_in] and dB_a [h_out, r_a] are stored at the true rank
   const int32_t* grp_seg;  // DROP kernels: first segment of every group (its adapter's dropout probability)
@@ -143,19 +144,30 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
 
-  // group of this adapter (ids are distinct): every lane looks at one group
+  // Group of this adapter (ids are distinct and ascending).  When every adapter below this one
+  // has rows too, it is group number `ad`: that entry is read together with the group count, so
+  // the usual case costs one round trip; otherwise every lane looks at one group.
+  const int Gs = ad < a.n_parts ? ad : a.n_parts - 1;  // (entries past the last group are allocated, not filled)
   const int NG = uload(a.hdr, 1);
+  const int sid = uload(a.grp_id, Gs), st0 = uload(a.grp_tile, Gs), st1 = uload(a.grp_tile, Gs + 1);
+  const int sseg0 = DROP ? uload(a.grp_seg, Gs) : -1;
   int t_beg = 0, t_end = 0, seg0 = -1;
-  for (int base = 0; base < NG; base += kWaveSize) {
-    const int G = base + lane;
-    const bool hit = G < NG && a.grp_id[G] == ad;
-    const unsigned long long m = __ballot(hit);
-    if (m) {
-      const int Gh = base + __builtin_ctzll(m);
-      t_beg = uload(a.grp_tile, Gh);
-      t_end = uload(a.grp_tile, Gh + 1);
-      if (DROP) seg0 = uload(a.grp_seg, Gh);
-      break;
+  if (Gs < NG && sid == ad) {
+    t_beg = st0;
+    t_end = st1;
+    seg0 = sseg0;
+  } else {
+    for (int base = 0; base < NG; base += kWaveSize) {
+      const int G = base + lane;
+      const bool hit = G < NG && a.grp_id[G] == ad;
+      const unsigned long long m = __ballot(hit);
+      if (m) {
+        const int Gh = base + __builtin_ctzll(m);
+        t_beg = uload(a.grp_tile, Gh);
+        t_end = uload(a.grp_tile, Gh + 1);
+        if (DROP) seg0 = uload(a.grp_seg, Gh);
+        break;
+      }
     }
   }
   int rlim = a.r;

@@ -536,8 +536,10 @@ BWD_CASES = [
     ("rank128", [0, 33, 90], [0, 1], 2, 4, 192, 320, 128),
     ("rank72", [0, 50], [0], 1, 0, 128, 136, 72),
     ("rank256-blocks", [0, 600, 1100], [1, 0], 2, 3, 256, 192, 256),
-    # few rows and long k: the sixteen-wave shrink (k split in two, folded by a launch) for v and dV
+    # few rows and long k: the eight-wave shrink (k split over workgroups, folded by a launch) for v and dV
     ("long-k", [0, 30, 75], [1, 0], 2, 4, 4096, 2048, 16),
+    # more adapters than partitions, most of them without rows (zero gradients), ids not dense
+    ("idle-adapters", [0, 40, 90], [4, 1], 6, 2, 128, 192, 16),
 ]
 
 
