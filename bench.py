@@ -324,6 +324,12 @@ def model_step_bench(args, torch, K):
             grouped[q + i] = (grouped[q + i][0], grouped[q][1])
         grouped[gate + 1] = (grouped[gate + 1][0], grouped[gate][1])
     g_host_us, _, g_graph_us = measure_decode(grouped)
+    # and with q/k/v also sharing ONE expand launch (deferred=True: the terms of all three are added when
+    # v is called, which the reference's attention allows, mixed_llama.py:113-115; gate/up stay as they are,
+    # its MLP reads gate's output before it calls up, mixed_llama.py:77)
+    for li in range(n_layers):
+        ProjectionGroup([grouped[li * n_sh + i][0] for i in range(3)], deferred=True)
+    d_host_us, _, d_graph_us = measure_decode(grouped)
     T = w["seg"][-1]
     step_bytes = sum(algorithmic_bytes(w, hi, ho) for _, hi, ho in shapes) * n_layers
     out["decode_forward"] = dict(workload=w["name"], calls_per_step=len(layers), host_us_per_call=round(host_us, 2),
@@ -334,7 +340,11 @@ def model_step_bench(args, torch, K):
                                  grouped_qkv_gate_up=dict(host_us_per_call=round(g_host_us, 2),
                                                           graph_gpu_us_per_call=round(g_graph_us, 2),
                                                           graph_ms_per_model_step=round(g_graph_us * len(layers) / 1e3, 4),
-                                                          tokens_per_s=round(T / (g_graph_us * len(layers) * 1e-6), 1)))
+                                                          tokens_per_s=round(T / (g_graph_us * len(layers) * 1e-6), 1)),
+                                 grouped_qkv_one_expand=dict(host_us_per_call=round(d_host_us, 2),
+                                                             graph_gpu_us_per_call=round(d_graph_us, 2),
+                                                             graph_ms_per_model_step=round(d_graph_us * len(layers) / 1e3, 4),
+                                                             tokens_per_s=round(T / (d_graph_us * len(layers) * 1e-6), 1)))
     del grouped
     del layers
     torch.cuda.empty_cache()

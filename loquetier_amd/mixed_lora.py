@@ -51,6 +51,9 @@ class MixedLoraContext:
         self._lora_ids = lora_ids
         self._lora_len = lora_len
         self._segment = segment
+        open_group = self._step.get("open_group")
+        if open_group is not None:   # a deferred group whose last member was never called: its adds happen now
+            open_group["group"].flush(open_group)
         self._train_idx = list(train_idx)
         self._plan = None
         self._seg_adapter = None
@@ -316,10 +319,22 @@ class ProjectionGroup:
     handed the same tensor object (same storage, not modified in between); a member that is called
     with anything else, or twice, or after another group has started its pass, simply shrinks
     again -- grouping never changes a result.  Call ProjectionGroup([q, k, v]) once after the layers
-    are built."""
+    are built.
 
-    def __init__(self, layers):
+    deferred=True also gives the members ONE expand launch: a member's call returns its base layer's
+    output with the LoRA term still missing, and the call of the group's last member adds the terms
+    of all of them, in place.  The values are the same, but they are complete only once every member
+    has been called: use it only where nothing reads a member's output before the last member's call
+    returns -- the reference's attention does (q, k and v are projected one after the other,
+    models/mixed_llama.py:113-115), its MLP does not (the activation reads gate's output before up is
+    called, mixed_llama.py:77).  A pass that is cut short (another group or another input starts, or
+    the context's next update arrives) adds what it still owes at that point.  A member whose call
+    cannot hand out the very tensor the expand writes (its base layer's output is of another dtype)
+    is expanded at once."""
+
+    def __init__(self, layers, deferred: bool = False):
         self.layers = list(layers)
+        self.deferred = deferred
         first = self.layers[0]
         for l in self.layers:
             if not (l.fused and l.rank == first.rank and l.dtype == first.dtype and l.device == first.device
@@ -334,28 +349,58 @@ class ProjectionGroup:
     def dims(self):
         return [(l.adapters[0].wa.size(1), l.adapters[0].wb.size(0)) for l in self.layers]
 
-    def expand_member(self, i: int, result: torch.Tensor, x: torch.Tensor, seg_scale, plan) -> None:
+    def _expand(self, ys, seg_scale, plan) -> None:
+        first, n = self.layers[0], len(self.layers)
+        kernel.smlm_lora_forward_multi(ys, [None] * n, [l.wa_ptrs for l in self.layers],
+                                       [l.wb_ptrs for l in self.layers], plan, first.rank, seg_scale=seg_scale,
+                                       beta=1.0, stages=2, adapter_rank=first.adapter_rank,
+                                       workspace=first.root_context.group_workspace(first.device),
+                                       packed_ranks=first.packed, dims=self.dims())
+
+    def flush(self, state) -> None:
+        """The expands a deferred pass still owes: one launch per distinct scale tensor (normally one)."""
+        waiting, state["waiting"] = state.get("waiting", []), []
+        while waiting:
+            scale = waiting[0][2]
+            ys = [None] * len(self.layers)
+            rest = []
+            for i, result, sc in waiting:
+                if sc is scale and ys[i] is None:
+                    ys[i] = result
+                else:
+                    rest.append((i, result, sc))
+            self._expand(ys, scale, state["plan"])
+            waiting = rest
+
+    def expand_member(self, i: int, result: torch.Tensor, x: torch.Tensor, seg_scale, plan,
+                      may_defer: bool = False) -> None:
         """result += scale * v_i B^T for member i, shrinking x for the whole group first when this is
-        the first member to see x."""
+        the first member to see x.  may_defer: the caller hands `result` itself on to its own caller,
+        so a deferred group may add to it later."""
         first, n = self.layers[0], len(self.layers)
         ctx = first.root_context
-        ws = ctx.group_workspace(first.device)
-        a_tabs, b_tabs = [l.wa_ptrs for l in self.layers], [l.wb_ptrs for l in self.layers]
         key = (x.data_ptr(), x._version, tuple(x.shape), x.dtype)
         state = ctx._step.get("open_group")
         if state is None or state["group"] is not self or state["key"] != key or i not in state["pending"]:
-            kernel.smlm_lora_forward_multi([None] * n, [x] * n, a_tabs, b_tabs, plan, first.rank, stages=1,
-                                           adapter_rank=first.adapter_rank, workspace=ws, packed_ranks=first.packed,
-                                           dims=self.dims())
+            if state is not None:
+                state["group"].flush(state)
+            kernel.smlm_lora_forward_multi([None] * n, [x] * n, [l.wa_ptrs for l in self.layers],
+                                           [l.wb_ptrs for l in self.layers], plan, first.rank, stages=1,
+                                           adapter_rank=first.adapter_rank,
+                                           workspace=ctx.group_workspace(first.device),
+                                           packed_ranks=first.packed, dims=self.dims())
             # (x is kept so that its address cannot be handed to another tensor while the pass is open)
-            state = ctx._step["open_group"] = {"group": self, "key": key, "pending": set(range(n)), "x": x}
-        ys = [None] * n
-        ys[i] = result
-        kernel.smlm_lora_forward_multi(ys, [None] * n, a_tabs, b_tabs, plan, first.rank, seg_scale=seg_scale,
-                                       beta=1.0, stages=2, adapter_rank=first.adapter_rank, workspace=ws,
-                                       packed_ranks=first.packed, dims=self.dims())
+            state = ctx._step["open_group"] = {"group": self, "key": key, "pending": set(range(n)), "x": x,
+                                               "plan": plan, "waiting": []}
         state["pending"].discard(i)
+        if self.deferred and may_defer:
+            state["waiting"].append((i, result, seg_scale))
+        else:
+            ys = [None] * n
+            ys[i] = result
+            self._expand(ys, seg_scale, plan)
         if not state["pending"]:
+            self.flush(state)
             del ctx._step["open_group"]
 
 
@@ -508,7 +553,8 @@ class MixedLoraLinear(nn.Module):
             if self._group is not None and blen.tlen == 0 and not weights and not (
                     torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):
                 # a serving step: the group's members share one shrink launch
-                self._group[0].expand_member(self._group[1], result, x, seg_scale, plan)
+                self._group[0].expand_member(self._group[1], result, x, seg_scale, plan,
+                                             may_defer=result.dtype == torch_result_dtype)
                 return result.to(torch_result_dtype)
             step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed)
             if weights and blen.tlen > 0:

@@ -141,3 +141,63 @@ def test_training_steps_are_not_grouped(K, gpu_device):
         outs.append((xs.grad.clone(), pairs[0][k].get_parameter("lora-1-A").grad.clone()))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
     assert "open_group" not in ctx._step
+
+
+def test_deferred_group_adds_everything_with_the_last_member(K, gpu_device):
+    """deferred=True: a member's output lacks its LoRA term until the group's last member has been
+    called; from then on every output equals the ungrouped layer's, bit for bit."""
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    d, tdt = gpu_device, torch.float16
+    h_in, widths, r, NA = 2048, [2048, 512, 512], 16, 6
+    req_ids, req_len = [int(i) for i in np.random.default_rng(4).integers(0, NA, 90)], [1] * 90
+    ctx, pairs = build(d, tdt, widths, h_in, r, NA, 8)
+    ProjectionGroup([p[0] for p in pairs], deferred=True)
+    gen = torch.Generator().manual_seed(12)
+    with torch.no_grad():
+        for step in range(3):
+            serve_step(ctx, d, req_ids, req_len)
+            x = torch.randn(sum(req_len), h_in, generator=gen).to(tdt).to(d)
+            want = [p[1](x) for p in pairs]
+            order = [(i + step) % 3 for i in range(3)]
+            got = [None] * 3
+            for n_called, i in enumerate(order):
+                got[i] = pairs[i][0](x)
+                if n_called < 2:   # still the base layer's output: the add is owed
+                    assert torch.equal(got[i], pairs[i][0].base_layer(x))
+                    assert not torch.equal(got[i], want[i])
+            for a, b in zip(got, want):
+                assert torch.equal(a, b)
+            assert "open_group" not in ctx._step
+
+
+def test_deferred_group_cut_short(K, gpu_device):
+    """A deferred pass that never sees its last member pays what it owes when the next pass or the
+    next step starts; a member whose output tensor is not the one handed out is expanded at once."""
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    d, tdt = gpu_device, torch.bfloat16
+    h_in, r, NA = 2048, 16, 4
+    ctx, pairs = build(d, tdt, [256, 256, 384], h_in, r, NA, 9)
+    ProjectionGroup([p[0] for p in pairs], deferred=True)
+    req_ids, req_len = [1, 0, 3, 2, 1, 0, 0], [1, 1, 1, 1, 1, 1, 17]
+    T = sum(req_len)
+    gen = torch.Generator().manual_seed(13)
+    x1 = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    x2 = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    with torch.no_grad():
+        serve_step(ctx, d, req_ids, req_len)
+        want1 = [p[1](x1) for p in pairs]
+        want2 = [p[1](x2) for p in pairs]
+        a, b = pairs[0][0](x1), pairs[1][0](x1)       # two of three members ...
+        c = pairs[0][0](x2)                           # ... then another input: the first pass is settled
+        assert torch.equal(a, want1[0]) and torch.equal(b, want1[1])
+        assert not torch.equal(c, want2[0])
+        serve_step(ctx, d, req_ids, req_len)          # the next step settles the second pass
+        assert torch.equal(c, want2[0])
+        assert "open_group" not in ctx._step
+        # a base layer that answers in float32: the layer hands out a converted copy, so its term is added at once
+        pairs[2][0].base_layer.float()
+        pairs[2][1].base_layer.float()
+        xf = x1.float()
+        want_c = pairs[2][1](xf)
+        got_c = pairs[2][0](xf)
+        assert got_c.dtype == torch.float32 and torch.equal(got_c, want_c)
