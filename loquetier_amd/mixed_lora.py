@@ -556,6 +556,13 @@ class MixedLoraLinear(nn.Module):
                 self._group[0].expand_member(self._group[1], result, x, seg_scale, plan,
                                              may_defer=result.dtype == torch_result_dtype)
                 return result.to(torch_result_dtype)
+            if not weights and drop_spec is None and not (
+                    torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):
+                # nothing to differentiate: the operator is called directly, without autograd's bookkeeping
+                kernel.smlm_lora_forward(result, x, self.wa_ptrs, self.wb_ptrs, plan, self.rank,
+                                         seg_scale=seg_scale, beta=1.0, adapter_rank=self.adapter_rank,
+                                         workspace=ctx.workspace(self.device), packed_ranks=self.packed)
+                return result.to(torch_result_dtype)
             step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed)
             if weights and blen.tlen > 0:
                 step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
