@@ -201,3 +201,49 @@ def test_deferred_group_cut_short(K, gpu_device):
         want_c = pairs[2][1](xf)
         got_c = pairs[2][0](xf)
         assert got_c.dtype == torch.float32 and torch.equal(got_c, want_c)
+
+
+@pytest.mark.parametrize("deferred", [False, True])
+def test_grouped_layers_under_graph_capture(K, gpu_device, deferred):
+    """A serving step of grouped layers captured once and replayed with new inputs: every replay gives
+    what ungrouped layers give eagerly (the group's bookkeeping is host-side and done at capture time)."""
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    d, tdt = gpu_device, torch.float16
+    h_in, widths, r, NA = 2048, [1024, 256, 256], 16, 5
+    req_ids, req_len = [int(i) for i in np.random.default_rng(6).integers(0, NA, 48)], [1] * 48
+    T = sum(req_len)
+    ctx, pairs = build(d, tdt, widths, h_in, r, NA, 14)
+    ProjectionGroup([p[0] for p in pairs], deferred=deferred)
+    gen = torch.Generator().manual_seed(15)
+    x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+    outs = [torch.empty(T, w, dtype=tdt, device=d) for w in widths]
+    cap = torch.cuda.Stream()
+    from loquetier_amd.kernel_utils import BatchLenInfo
+    from loquetier_amd.segments import build_segments
+    lora_ids, lora_len, segment = build_segments(req_ids, req_len, d)   # staged on the device before the capture
+    lora_ids = torch.tensor(lora_ids, dtype=torch.int32, device=d) if not isinstance(lora_ids, torch.Tensor) else lora_ids
+    blen = BatchLenInfo([], [], T, [], d)
+
+    def update():
+        ctx.update(blen=blen, lora_ids=lora_ids, lora_len=lora_len, segment=segment, train_idx=[])
+
+    def step():
+        update()
+        got = [p[0](x) for p in pairs]   # (a deferred group's outputs are complete after the last member's call)
+        for o, t in zip(outs, got):
+            o.copy_(t)
+    with torch.no_grad():
+        with torch.cuda.stream(cap):
+            step()                             # eager once: sizes the workspaces outside the capture
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=cap):
+            step()
+        for rep in range(3):
+            x.copy_(torch.randn(T, h_in, generator=gen).to(tdt))
+            g.replay()
+            torch.cuda.synchronize()
+            serve_step(ctx, d, req_ids, req_len)
+            want = [p[1](x) for p in pairs]
+            for a, b in zip(outs, want):
+                assert torch.equal(a, b)
