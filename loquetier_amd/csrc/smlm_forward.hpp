@@ -265,7 +265,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         for (int nb = 0; nb < NB; ++nb) acc[nb] = Num<DT>::mfma(wf[nb][u], xu, acc[nb]);
       }
     };
-    if (NW < 16) {
+    {
       // two load batches in turn: one is on its way while the other is multiplied
       u32x4 xa[U], wa[NB][U], xb[U], wb[NB][U];
       load_batch(kbeg, xa, wa);
@@ -277,13 +277,6 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
         if (!more) break;
         if (k + 64 * U < kend) load_batch(k + 64 * U, xa, wa);
         multiply(k + 32 * U, xb, wb);
-      }
-    } else {  // sixteen waves and more share the VGPR file: one batch at a time
-#pragma unroll 1
-      for (int k = kbeg; k < kend; k += 32 * U) {
-        u32x4 xf[U], wf[NB][U];
-        load_batch(k, xf, wf);
-        multiply(k, xf, wf);
       }
     }
 

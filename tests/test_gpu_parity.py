@@ -388,13 +388,13 @@ def test_forward_dyadic_bit_exact_larger(K, oracle, gpu_device, shape, dt):
 
 @pytest.mark.parametrize("dt", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [
-    # T, S, NA, h_in, h_out, r: few rows and a long k -> sixteen-wave shrink with k split over
-    # two workgroups, partial sums folded by the expand kernel
+    # T, S, NA, h_in, h_out, r: few rows and a long k -> eight-wave shrink with k split over
+    # four workgroups, partial sums folded by the expand kernel
     (1, 1, 1, 4096, 512, 16),
     (17, 17, 5, 4096, 1024, 8),
     (256, 256, 32, 4096, 640, 16),
     (200, 23, 9, 11008, 512, 32),     # k not a multiple of the waves' share: ragged last batch
-    (1000, 61, 7, 2048, 1536, 64),    # shortest k that takes the sixteen-wave route at rank 64
+    (1000, 61, 7, 2048, 1536, 64),    # shortest k that takes the eight-wave route at rank 64
     (96, 10, 3, 4104, 264, 24),       # k and rank off the round sizes
     (300, 30, 4, 2040, 512, 16),      # just below the route's minimum k: four-wave shrink
 ], ids=["one-row", "r8", "decode-256", "k11008", "r64-k2048", "odd-sizes", "below-min-k"])
@@ -448,7 +448,7 @@ def test_forward_beyond_the_direct_grid(K, oracle, gpu_device):
 
 
 def test_multi_projection_mixed_routes_equal_single_calls(K, oracle, gpu_device):
-    """Projections of one launch with different k: all long (sixteen-wave route with a different
+    """Projections of one launch with different k: all long (eight-wave route with a different
     k split each) and one short (which sends the whole launch down the four-wave route)."""
     d, dt = gpu_device, "fp16"
     T, r, NA, S = 120, 16, 5, 14
