@@ -499,13 +499,13 @@ class MixedLoraLinear(nn.Module):
 
     def add_adapter(self, adapter: NamedLoraLayer):
         """New adapter must have the rank of the existing ones."""
-        self.update_adapters(self.adapters + [adapter], self.rank)
+        self.adapters.append(adapter)   # (in place, as the reference does: the caller may hold the list)
+        self.update_adapters(self.adapters, self.rank)
 
     def del_adapter(self, adapter_idx: int):
         assert adapter_idx < len(self.adapters)
-        adapters = list(self.adapters)
-        del adapters[adapter_idx]
-        self.update_adapters(adapters, self.rank)
+        del self.adapters[adapter_idx]
+        self.update_adapters(self.adapters, self.rank)
 
     def set_trainable(self, train_idx: List[int]):
         for idx in train_idx:

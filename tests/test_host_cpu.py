@@ -252,3 +252,37 @@ def test_layer_state_dict_saves_one_adapter_under_peft_names():
         assert not [k for k in layer.state_dict() if k.startswith("lora_")]
     # the parameters share the adapters' storage (mixed_lora.py:168-171): an optimizer step moves no address
     assert layer.get_parameter("lora-2-A").data_ptr() == adapters[2].wa.data_ptr()
+
+
+def test_layer_adapter_list_management():
+    """add_adapter / del_adapter / update_adapters (reference mixed_lora.py:106-166): the layer's own
+    list is changed in place and the pointer and scale tables follow it."""
+    import torch
+    from loquetier_amd import mixed_lora as ml
+
+    class Base(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.zeros(8, 16), requires_grad=False)
+
+    def adapter(i, scale):
+        return ml.NamedLoraLayer(f"a{i}", torch.full((8, 16), float(i)), torch.full((8, 8), 10.0 + i),
+                                 torch.nn.Identity(), scale)
+    held = [adapter(0, 2.0), adapter(1, 0.5)]
+    layer = ml.MixedLoraLinear(ml.MixedLoraContext(), Base(), held, 8, torch.float32, is_scaled=False)
+    assert layer.adapters is held and layer.wa_ptrs.tolist() == [a.wa.data_ptr() for a in held]
+    layer.add_adapter(adapter(2, 4.0))
+    assert layer.adapters is held and len(held) == 3
+    assert layer.wa_ptrs.tolist() == [a.wa.data_ptr() for a in held]
+    assert layer.wb_ptrs.tolist() == [a.wb.data_ptr() for a in held]
+    assert layer.scaling.tolist() == [2.0, 0.5, 4.0]
+    layer.del_adapter(0)
+    assert layer.adapters is held and [a.adapter_name for a in held] == ["a1", "a2"]
+    assert layer.wa_ptrs.tolist() == [a.wa.data_ptr() for a in held] and layer.scaling.tolist() == [0.5, 4.0]
+    import pytest
+    with pytest.raises(AssertionError):
+        layer.del_adapter(5)
+    scaled = ml.MixedLoraLinear(ml.MixedLoraContext(), Base(), [adapter(0, 2.0)], 8, torch.float32, is_scaled=True)
+    assert scaled.scaling is None
+    scaled.add_adapter(adapter(1, 3.0))
+    assert scaled.scaling is None and scaled.wb_ptrs.numel() == 2
