@@ -307,6 +307,9 @@ int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipS
   if (block && a.w_kn)
     return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, true>, grid, dim3(kFwdThreads), st, a)
                    : launch(expand_block_kernel<DT, 4, 2, DIRECT, true>, grid, dim3(kFwdThreads), st, a);
+  if (block && nq == 8)
+    return KS == 1 ? launch(expand_block_kernel<DT, 8, 1, DIRECT, false>, grid, dim3(kFwdThreads), st, a)
+                   : launch(expand_block_kernel<DT, 8, 2, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
   if (block)
     return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, false>, grid, dim3(kFwdThreads), st, a)
                    : launch(expand_block_kernel<DT, 4, 2, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
@@ -322,13 +325,33 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   const bool block = !row_major && MT > 1 && KS > 0;  // tile blocks with the weights staged in LDS
   if (a.drop.seg_p && (row_major || nproj != 1 || a.p[0].vsplit > 0 || (block && !a.w_kn))) return SMLM_ERR_ARG;
   if (row_major) nq = 2;
-  if (block) nq = 4;
-  if (block) nq = 4;
+  // Tile blocks: 128 columns a workgroup, or 256 where measured better (rank 64, 8192 rows: 5-13 % at every
+  // width; a row stride that is a multiple of 4 KiB, e.g. h_out = 14336, from 4096 rows on at every rank:
+  // the 64 rows of a tile block then meet in few HBM channels and pieces of 512 bytes spread them over
+  // twice as many).  Elsewhere 256 columns lose 1-12 % (fewer workgroups a CU; h_out = 11008, the
+  // backward's dX, whose weights lie [k][n]).
+  if (block) {
+    int wide = 0;
+    for (int i = 0; i < nproj; ++i) wide = a.p[i].d_out > wide ? a.p[i].d_out : wide;
+    const bool aligned = (wide * 2) % 4096 == 0;
+    const bool wider = !a.w_kn && !a.drop.seg_p &&
+                       ((KS == 2 && a.T >= 8192) || (aligned && wide >= 8192 && a.T >= 4096));
+    nq = wider ? 8 : 4;
+  }
   const int chunk = block ? 32 * nq : kFwdWaves * 32 * nq;  // columns per workgroup
   a.items.nproj = nproj;
   a.items.interleave = 0;
   a.items.row_start[0] = 0;
-  for (int i = 0; i < nproj; ++i) a.items.row_start[i + 1] = a.items.row_start[i] + ceil_div(a.p[i].d_out, chunk);
+  // Workgroups go to the XCDs in turn.  With an odd number of chunk rows a tile unit, the workgroups of one
+  // column chunk visit all eight XCDs from unit to unit and each L2 fetches that chunk of an adapter's weights
+  // for itself; with an even number they stay within four, two or one.  Odd counts get one empty row
+  // (8192 rows at rank 64: h_out = 11136, 87 chunks of 128 columns, 83.4 -> 73.3 us; h_out = 11008, 43 chunks
+  // of 256, 87.8 -> 71.7 us); rounding even counts up further changed nothing that could be told from noise.
+  for (int i = 0; i < nproj; ++i) {
+    int rows = ceil_div(a.p[i].d_out, chunk);
+    if (rows > 1 && (rows & 1)) rows += 1;
+    a.items.row_start[i + 1] = a.items.row_start[i] + rows;
+  }
   const int units = tile_units_max(a.T, S, groups, block ? kBlkTiles : 1);
   const long items = (long)units * a.items.row_start[nproj];
   bool same_rows = true;

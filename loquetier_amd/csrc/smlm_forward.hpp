@@ -785,7 +785,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
 template <int DT, int NQ, int KS, bool DIRECT, bool WKN, bool DROP = false>
 // (five workgroups a CU instead of the four the compiler's own register budget gives: more y
 // lines in flight per CU; worth 2 % on the prefill launch and 6 % on the fine-tune one)
-__global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(DIRECT ? 5 : 1)))
+__global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(DIRECT ? (NQ > 4 ? 3 : 5) : 1)))
 void expand_block_kernel(ExpandArgs a) {
   static_assert(NQ % 2 == 0, "the output is written 64 columns at a time");
   constexpr int kPitch = WKN ? 32 * NQ + 8 : 32 * KS + 8;  // LDS row pitch in 16-bit elements
@@ -808,6 +808,7 @@ void expand_block_kernel(ExpandArgs a) {
     const ExpandProj P = a.p[pj];
     if (!P.y) continue;  // a projection this call leaves out (uniform over the workgroup)
     const int ncol0 = yy * 32 * NQ;
+    if (ncol0 >= P.d_out) continue;  // a chunk row added to round the count up (uniform over the workgroup)
     const int packed = uload(a.plan.blk, tb);
     const int t0 = packed >> 3, cnt = packed & 7;
     if (cnt == 0) continue;  // past the last block (direct mode); uniform over the workgroup

@@ -360,6 +360,28 @@ def test_forward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
 
 
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [
+    # T, S, NA, h_in, h_out, r: the tile-block expand's launch shapes
+    (4096, 37, 5, 128, 8192, 16),    # 4096 rows and a row stride of 16 KiB: 256 columns a workgroup
+    (4100, 21, 3, 64, 10240, 32),    # the same at rank 32, rows past a multiple of 64
+    (8192, 90, 7, 64, 768, 64),      # rank 64 at 8192 rows: 256 columns, three chunk rows rounded up to four
+    (8200, 50, 6, 64, 1032, 48),     # ... and a width that ends inside a chunk (five chunk rows -> six)
+    (1100, 12, 4, 64, 640, 16),      # 128 columns, five chunk rows rounded up to six
+    (1100, 12, 4, 64, 1160, 64),     # 128 columns at rank 64 below 8192 rows, ragged last chunk (ten rows)
+], ids=["r16-wide-aligned", "r32-wide-aligned", "r64-8192-rows", "r48-ragged-width", "odd-chunk-rows", "r64-short"])
+def test_forward_expand_launch_shapes(K, oracle, gpu_device, shape, dt):
+    """The widths, row counts and ranks at which the tile-block expand changes its columns per
+    workgroup or pads its grid: bit-exact against the oracle."""
+    T, S, NA, h_in, h_out, r = shape
+    rng = np.random.default_rng(47)
+    seg = _ragged_segments(rng, T, S)
+    ids = rng.integers(0, NA, S).tolist()
+    x, A, B = make_case(oracle, 207, T, seg, ids, NA, h_in, h_out, r, dt, dy=True)
+    base = dyadic(np.random.default_rng(23), (T, h_out), 16, 8)
+    _fwd_exact(K, oracle, gpu_device, dt, x, A, B, seg, ids, r, base)
+
+
 def _ragged_segments(rng, T, S):
     cuts = np.sort(rng.choice(np.arange(1, T), S - 1, replace=False))
     return [0] + cuts.tolist() + [T]
