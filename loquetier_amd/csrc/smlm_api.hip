@@ -342,14 +342,16 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
   a.items.nproj = nproj;
   a.items.interleave = 0;
   a.items.row_start[0] = 0;
-  // Workgroups go to the XCDs in turn.  With an odd number of chunk rows a tile unit, the workgroups of one
-  // column chunk visit all eight XCDs from unit to unit and each L2 fetches that chunk of an adapter's weights
-  // for itself; with an even number they stay within four, two or one.  Odd counts get one empty row
-  // (8192 rows at rank 64: h_out = 11136, 87 chunks of 128 columns, 83.4 -> 73.3 us; h_out = 11008, 43 chunks
-  // of 256, 87.8 -> 71.7 us); rounding even counts up further changed nothing that could be told from noise.
+  // Workgroups go to the XCDs in turn (workgroup number modulo eight, whatever the XCDs' load).  With an odd
+  // number of chunk rows a tile unit, the workgroups of one column chunk visit all eight XCDs from unit to
+  // unit and each L2 fetches that chunk of an adapter's weights for itself: a launch of one projection gets one
+  // empty row then (8192 rows at rank 64: h_out = 11136, 87 chunks of 128 columns, 83.4 -> 73.3 us; h_out =
+  // 11008, 43 chunks of 256, 87.8 -> 71.7 us).  Launches of several projections are left as they are: empty
+  // workgroups there can fall on the same few XCDs in every unit and leave the others with all the work
+  // (measured on the shrink launch of five and six projections: up to 2.2 x slower).
   for (int i = 0; i < nproj; ++i) {
     int rows = ceil_div(a.p[i].d_out, chunk);
-    if (rows > 1 && (rows & 1)) rows += 1;
+    if (nproj == 1 && rows > 1 && (rows & 1)) rows += 1;
     a.items.row_start[i + 1] = a.items.row_start[i] + rows;
   }
   const int units = tile_units_max(a.T, S, groups, block ? kBlkTiles : 1);
@@ -432,7 +434,13 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
       P.drop_bits = drop->bits + bits_off;
       bits_off += (size_t)drop->rows * (d_in[i] / 8);
     }
-    a.items.row_start[i + 1] = a.items.row_start[i] + c.ksplit * c.zblocks;
+    // (a launch of one projection with an odd number of chunk rows a tile unit gets one empty row, as the
+    // expand launch does and for its reason: 8192 rows at rank 64, h_in = 11008, k split in five: 75.5 ->
+    // 59.6 us; 6144 rows, h_in = 4096, in three: 27.2 -> 25.0; launches of several projections and those that
+    // build their plan keep their grid)
+    int rows = c.ksplit * c.zblocks;
+    if (nproj == 1 && !build && rows > 1 && (rows & 1)) rows += 1;
+    a.items.row_start[i + 1] = a.items.row_start[i] + rows;
     ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit};
     need_reduce = need_reduce || c.ksplit > 1;
   }

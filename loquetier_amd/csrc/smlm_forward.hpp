@@ -224,6 +224,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
     if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tile)) break;
     const ShrinkProj P = a.p[pj];
     const int kz = yy % P.ksplit, zb = yy / P.ksplit;
+    if (zb >= P.zblocks) continue;  // a chunk row added to make the count even (uniform over the workgroup)
     const int wid = uload(a.plan.tile_wid, tile);
     if (wid < 0) continue;  // past the last tile (direct mode); uniform over the workgroup
     const int n0 = zb * 64;
@@ -343,6 +344,7 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
     if (!item_get<DIRECT>(a.items, V, units, &pj, &yy, &tb)) break;
     const ShrinkProj P = a.p[pj];
     const int kz = yy % P.ksplit, zb = yy / P.ksplit;
+    if (zb >= P.zblocks) continue;  // a chunk row added to make the count even (uniform over the workgroup)
     int t0, cnt, wid;
     pick_tiles<kBlkTiles>(a.plan, tb, &t0, &cnt, &wid);
     if (cnt == 0) continue;  // uniform over the workgroup
