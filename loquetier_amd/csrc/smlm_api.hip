@@ -84,7 +84,8 @@ int shrink_waves(int T, int nproj, const int* d_in, int d_out) {
   return all_long ? kDecodeWaves : kFwdWaves;
 }
 
-ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
+// solo: the launch has this one projection (a launch of several fills the chip with their workgroups together)
+ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw, bool solo) {
   ShrinkCfg c;
   c.zblocks = ceil_div(d_out, 64);
   const int cols = d_out >= 64 ? 64 : d_out;
@@ -100,8 +101,11 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   // beyond 256 workgroups the split stops where the partials reach an eighth of the input.
   // Eight-wave workgroups (decode batches: few tiles) split k in four, which quadruples the
   // number of CUs at work; the expand kernel adds the four partials.
+  // (A launch of one projection fills the chip twice over from 4096 rows on: 8192 rows at rank 64, h_in =
+  // 4096, k in four instead of two: 27.6 -> 23.3 us; 4096 rows, h_in = 11008, in eight instead of five: 44.4
+  // -> 35.6 us.  In a launch of several projections the same splits were 2-20 % slower: cfg5 180 -> 190 us.)
   int want = c.NW == kDecodeWaves ? kDecodeSplit : ceil_div(1024, units);
-  const int cheap = d_in / (32 * d_out), fill = ceil_div(256, units);
+  const int cheap = d_in / (32 * d_out), fill = ceil_div((solo && c.MT > 1 && units >= 64) ? 512 : 256, units);
   const int cap = cheap > fill ? cheap : fill;
   if (want > cap) want = cap;
   int max_split = d_in / (c.NW * kq);
@@ -110,13 +114,31 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw) {
   const int ks = want < 1 ? 1 : (want > max_split ? max_split : want);
   c.k_per_wave = round_up(ceil_div(d_in, c.NW * ks), kq);
   c.ksplit = ceil_div(d_in, c.NW * c.k_per_wave);
+  // An odd split (h_in = 14336 falls into seven slices of 2048) gives way to an even one of equal slices that
+  // still fills the chip twice: 8192 rows, h_in = 14336, k in four instead of seven: rank 16 61.6 -> 53.1 us,
+  // rank 64 80.0 -> 67.8 us (six, eight, ten ... fourteen slices: 56-65 and 77-87 us).
+  if (solo && c.MT > 1 && c.ksplit > 1 && (c.ksplit & 1) && d_in % (c.NW * kq) == 0) {
+    const int pieces = d_in / (c.NW * kq);
+    for (int e = c.ksplit - 1; e >= 2; --e)
+      if (e % 2 == 0 && pieces % e == 0 && units * e >= 512) {
+        c.k_per_wave = pieces / e * kq;
+        c.ksplit = e;
+        break;
+      }
+  }
   return c;
 }
 
 // most k-split partials a shrink of this shape can leave behind, whichever wave count it runs with
 int fwd_ksplit_bound(int T, int d_in, int d_out) {
-  const int a = shrink_cfg(T, d_in, d_out, kFwdWaves).ksplit, b = shrink_cfg(T, d_in, d_out, kDecodeWaves).ksplit;
-  return a > b ? a : b;
+  int most = 1;
+  for (int solo = 0; solo < 2; ++solo) {
+    const int a = shrink_cfg(T, d_in, d_out, kFwdWaves, solo != 0).ksplit;
+    const int b = shrink_cfg(T, d_in, d_out, kDecodeWaves, solo != 0).ksplit;
+    most = a > most ? a : most;
+    most = b > most ? b : most;
+  }
+  return most;
 }
 
 int expand_nq(int T, int d_out) {
@@ -420,7 +442,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   size_t bits_off = 0;
   const int nw = row_major ? kFwdWaves : shrink_waves(T, nproj, d_in, d_out);
   for (int i = 0; i < nproj; ++i) {
-    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw);
+    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw, nproj == 1);
     if (i == 0) c0 = c;
     ShrinkProj& P = a.p[i];
     P.x = reinterpret_cast<const uint16_t*>(x[i]);
@@ -496,8 +518,8 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
     off = align_up(off + bytes, 256);
     return o;
   };
-  L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves);
-  L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves);
+  L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves, true);
+  L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves, true);
   const int ks_dv = fwd_ksplit_bound(n_rows, h_out, r), ks_v = fwd_ksplit_bound(n_rows, h_in, r);
   const int ks = ks_dv > ks_v ? ks_dv : ks_v;
   L.pitch = (long)plan_nt_max(n_rows, P) * kTileRows;
@@ -783,7 +805,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   {
     char* w = reinterpret_cast<char*>(workspace);
     for (int i = 0; i < n_proj; ++i) {
-      vsplit[i] = shrink_cfg(T, h_in[i], r, nw).ksplit;
+      vsplit[i] = shrink_cfg(T, h_in[i], r, nw, n_proj == 1).ksplit;
       expand_folds = expand_folds && vsplit[i] <= kMaxExpandFold;
       partial[i] = reinterpret_cast<float*>(w);
       w += align_up((size_t)fwd_ksplit_bound(T, h_in[i], r) * T * r * 4, 256);

@@ -369,10 +369,13 @@ def test_forward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     (8200, 50, 6, 64, 1032, 48),     # ... and a width that ends inside a chunk (five chunk rows -> six)
     (1100, 12, 4, 64, 640, 16),      # 128 columns, five chunk rows rounded up to six
     (1100, 12, 4, 64, 1160, 64),     # 128 columns at rank 64 below 8192 rows, ragged last chunk (ten rows)
-], ids=["r16-wide-aligned", "r32-wide-aligned", "r64-8192-rows", "r48-ragged-width", "odd-chunk-rows", "r64-short"])
+    (4100, 15, 3, 11008, 128, 64),   # the shrink of one projection from 4096 rows on: k split in eight, ragged last slice
+    (6200, 9, 2, 4096, 64, 64),      # ... k split in three: one empty chunk row
+], ids=["r16-wide-aligned", "r32-wide-aligned", "r64-8192-rows", "r48-ragged-width", "odd-chunk-rows", "r64-short",
+        "k-split-eight", "k-split-three"])
 def test_forward_expand_launch_shapes(K, oracle, gpu_device, shape, dt):
-    """The widths, row counts and ranks at which the tile-block expand changes its columns per
-    workgroup or pads its grid: bit-exact against the oracle."""
+    """The widths, row counts and ranks at which the tile-block launches change their columns per
+    workgroup, their k split or pad their grid: bit-exact against the oracle."""
     T, S, NA, h_in, h_out, r = shape
     rng = np.random.default_rng(47)
     seg = _ragged_segments(rng, T, S)
