@@ -133,7 +133,15 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
         mats = [buf[o: o + shape[0] * shape[1]].view(shape) for o, shape in shapes]
         NA = len(mats) // 2
         da, db = mats[:NA], mats[NA:]
-        tabs = step.grad_offsets + buf.data_ptr()               # device arithmetic, no copy from the host
+        # addresses of the gradients: device arithmetic, no copy from the host; torch's allocator hands the
+        # same block out step after step, so the table of an address is kept
+        tabs = None if step.grad_tabs is None else step.grad_tabs.get(buf.data_ptr())
+        if tabs is None:
+            tabs = step.grad_offsets + buf.data_ptr()
+            if step.grad_tabs is not None:
+                if len(step.grad_tabs) >= 64:
+                    step.grad_tabs.clear()
+                step.grad_tabs[buf.data_ptr()] = tabs
         if tl > 0:
             g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
             kernel.smlm_lora_backward(grad_x, tabs[:NA], tabs[NA:], g, x_train, v_train, step.a_tab, step.b_tab,

@@ -298,6 +298,7 @@ class LayerStep:
     b_tab: Optional[torch.Tensor] = None
     grad_offsets: Optional[torch.Tensor] = None    # byte offsets of dA_0.., dB_0.. inside one gradient buffer
     grad_shapes: Optional[list] = None             # [(offset in elements, shape)] in the same order
+    grad_tabs: Optional[dict] = None               # gradient buffer address -> device table of the gradients' addresses
     memo: Any = None                               # the context's per-step memo (MixedLoraContext.memo)
     packed: bool = False                           # the adapters are stored at their true ranks
 
@@ -469,7 +470,7 @@ class MixedLoraLinear(nn.Module):
                     off += (w.numel() + 7) // 8 * 8   # every matrix 16-byte aligned
             tabs = dict(a_tab=self.wa_ptrs[idx].contiguous(), b_tab=self.wb_ptrs[idx].contiguous(),
                         grad_offsets=torch.tensor(offsets, dtype=torch.int64, device=self.device),
-                        grad_shapes=shapes, grad_numel=off)
+                        grad_shapes=shapes, grad_numel=off, grad_tabs={})
             self._train_tabs[key] = tabs
         return tabs
 
@@ -570,6 +571,7 @@ class MixedLoraLinear(nn.Module):
                 tabs = self._train_tables(ctx.train_order())
                 step.a_tab, step.b_tab = tabs["a_tab"], tabs["b_tab"]
                 step.grad_offsets, step.grad_shapes = tabs["grad_offsets"], (tabs["grad_shapes"], tabs["grad_numel"])
+                step.grad_tabs = tabs["grad_tabs"]
             result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale, plan, self.rank,
                                           blen.tlen, blen.train_partition, drop_spec,
                                           self._rank_args(train_idx), step, *weights)
