@@ -1032,8 +1032,10 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   // ranks above 64 are covered 64 at a time along the grid's z axis
   dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA, ceil_div(r, 64));
   const int nbj = r > 64 ? 4 : ceil_div(r, 16);
-  // four waves splitting the rows of an adapter pay off when adapters have many rows each
-  const bool split = n_rows / NA >= 256;
+  // four waves splitting the rows of an adapter pay off when adapters have many rows each (whole backward,
+  // 16 adapters at rank 16 / 64: 1024 rows each 124.7 -> 118.7 / 180.7 -> 175.3 us, 512 rows even, 256 rows
+  // 43.5 -> 44.6 / 62.1 -> 67.3 us, 64 rows 25.7 -> 30.8 / 33.7 -> 46.5 us)
+  const bool split = n_rows / NA >= 512;
   return dtype == SMLM_DTYPE_F16 ? launch_wgrad<SMLM_DTYPE_F16>(nbj, split, grid, st, wa)
                                  : launch_wgrad<SMLM_DTYPE_BF16>(nbj, split, grid, st, wa);
 }
