@@ -95,6 +95,13 @@ def adapter_sorted(w):
     return w
 
 
+def single_tiles(T: int, r: int) -> bool:
+    """Whether the forward of a batch of T rows at rank r runs on single 16-row tiles (the decode route)
+    or on tile blocks: the library's rule, loquetier_amd/csrc/smlm_api.hip (tiles_per_wave); only used
+    here to say in the output how the step's plan is built."""
+    return T < (2560 if r <= 16 else 1280 if r <= 32 else 1024 if r <= 48 else 512 if r <= 64 else 1024)
+
+
 def algorithmic_bytes(w, h_in, h_out, accumulate=True):
     """Forward bytes of one projection: x and y once (y read too when accumulating),
     A and B of each distinct active adapter once, v written and read once at I/O width."""
@@ -605,7 +612,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
     expand_us = stage_us(2)
     shrink_us = stage_us(1)
     # decode batches: the shrink launch that also builds the plan (what the step's first forward launches)
-    self_planned = T < 1024 and not args.plan_launch and not P
+    self_planned = single_tiles(T, r) and not args.plan_launch and not P
     if self_planned:
         bufs = [st["plan_buf"] for st in sets]
 
@@ -711,7 +718,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
     # whether the library builds this batch's plan inside the forward's shrink launch (the limits of
     # the route, include/smlm.h: segments, possible tiles)
     in_launch = not args.plan_launch and not (args.dropout and P) and (
-        S <= 1024 if T < 1024 else (S <= 512 and T // 16 + S + 1 <= 1024))
+        S <= 1024 if single_tiles(T, r) else (S <= 512 and T // 16 + S + 1 <= 1024))
     out = {
         "metric": METRIC, "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),

@@ -274,15 +274,17 @@ typedef struct smlm_dropout {
  *                  for every later call on the stream) and uses it.  The reference sets its
  *                  problems up inside every call as well (precompute_smlm_forward_args,
  *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  With
- *                  n_weights <= 1024, no dropout and either T < 1024, S <= 1024 and every
- *                  h_in >= 2048, or T >= 1024, S <= 512 and T / 16 + S < 1024, this costs no
+ *                  n_weights <= 1024, no dropout and either a batch of few rows (below 2560 rows
+ *                  at rank <= 16, 1280 at rank <= 32, 1024 at rank <= 48, 512 at rank <= 64,
+ *                  1024 above: the single-tile kernels), S <= 1024 and every h_in >= 2048, or a
+ *                  larger batch with S <= 512 and T / 16 + S < 1024, this costs no
  *                  launch: the shrink's workgroups derive their own tiles from the two arrays
  *                  while a few more workgroups of the same launch write the plan; other batches
  *                  get the plan launch first.  Adapter ids must lie below n_weights (negative:
  *                  no adapter, see the tile plan above); stages must include SMLM_STAGE_SHRINK.
  *                  smlm_lora_bwd_ex takes the pair (part_indptr, part_adapter) the same way and
- *                  builds its plan inside the dV launch when n_rows >= 1024, P <= 512, v is given
- *                  and there is no dropout.
+ *                  builds its plan inside the dV launch when r <= 64, P <= 512,
+ *                  n_rows / 16 + P < 1024, v is given and there is no dropout.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;

@@ -40,7 +40,18 @@ int launch(void (*kernel)(A), dim3 grid, dim3 block, hipStream_t st, const A& a)
 
 // ---- launch shapes: functions of (T, d_in, d_out) only, never of the
 // segmentation, so re-segmenting a batch cannot change a bit of any row. ----
-inline int tiles_per_wave(int T) { return T >= 1024 ? kBlkTiles : 1; }
+// Tiles per work item: single 16-row tiles for batches of few rows, tile blocks (up to kBlkTiles tiles of one
+// adapter, their weights staged once in LDS) for larger ones.  Where the forward changes over depends on the
+// rank -- the tile-block kernels save weight traffic in proportion to it (4096 -> 4096, one projection, single
+// tiles / tile blocks in us: rank 16 at 2000 rows 18.4 / 20.8, at 3072 rows 26.0 / 24.5; rank 32 at 1024 rows
+// 15.6 / 17.8, at 1536 rows 21.7 / 19.2; rank 64 at 512 rows 17.7 / 17.1, at 1000 rows 22.9 / 18.8).
+inline int tiles_per_wave(int T, int r) {
+  const int from = r <= 16 ? 2560 : (r <= 32 ? 1280 : (r <= 48 ? 1024 : (r <= 64 ? 512 : 1024)));
+  return T >= from ? kBlkTiles : 1;
+}
+// The backward runs on tile blocks at every size up to rank 64: its single-tile route needs transposed copies
+// of the weights first (64 rows at rank 64: 25.0 / 18.8 us; 1024 rows at rank 16: 28.3 / 25.3 us).
+inline int bwd_tiles_per_wave(int n_rows, int r) { return (r <= 64 || n_rows >= 1024) ? kBlkTiles : 1; }
 
 // Upper bound of the number of work units along the tile axis.  `groups` bounds
 // the number of distinct plan keys (adapters): every group ends in at most one
@@ -77,20 +88,20 @@ constexpr int kMaxExpandFold = kMaxVsplit;  // most partials the expand kernel f
 
 // waves per shrink workgroup, one choice for all projections of a launch: small
 // batches whose every projection has a long enough k use eight waves and split k in four
-int shrink_waves(int T, int nproj, const int* d_in, int d_out) {
+int shrink_waves(int mt, int nproj, const int* d_in, int d_out) {
   const int kq = 32 * (d_out > 32 ? 2 : 4);  // k per wave and load batch of the decode kernels
-  bool all_long = tiles_per_wave(T) == 1;
+  bool all_long = mt == 1;
   for (int i = 0; i < nproj; ++i) all_long = all_long && d_in[i] >= 16 * kq;
   return all_long ? kDecodeWaves : kFwdWaves;
 }
 
 // solo: the launch has this one projection (a launch of several fills the chip with their workgroups together)
-ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw, bool solo) {
+ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw, bool solo, int mt) {
   ShrinkCfg c;
   c.zblocks = ceil_div(d_out, 64);
   const int cols = d_out >= 64 ? 64 : d_out;
   c.NB = cols <= 16 ? 1 : (cols <= 32 ? 2 : 4);
-  c.MT = tiles_per_wave(T);
+  c.MT = mt;
   // 32-wide k steps per load batch (the tile-block kernel stages four per batch in LDS)
   c.U = c.MT > 1 ? 4 : (c.NB == 4 ? 2 : 4);
   const int kq = 32 * c.U;
@@ -133,10 +144,12 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw, bool solo) {
 int fwd_ksplit_bound(int T, int d_in, int d_out) {
   int most = 1;
   for (int solo = 0; solo < 2; ++solo) {
-    const int a = shrink_cfg(T, d_in, d_out, kFwdWaves, solo != 0).ksplit;
-    const int b = shrink_cfg(T, d_in, d_out, kDecodeWaves, solo != 0).ksplit;
+    const int a = shrink_cfg(T, d_in, d_out, kFwdWaves, solo != 0, 1).ksplit;
+    const int b = shrink_cfg(T, d_in, d_out, kDecodeWaves, solo != 0, 1).ksplit;
+    const int c = shrink_cfg(T, d_in, d_out, kFwdWaves, solo != 0, kBlkTiles).ksplit;
     most = a > most ? a : most;
     most = b > most ? b : most;
+    most = c > most ? c : most;
   }
   return most;
 }
@@ -241,8 +254,7 @@ int launch_self_planned_block(int NB, int S, dim3 grid, hipStream_t st, const Se
 // batches this route takes: few enough segments for the plan-building workgroups of the launch
 // (one segment per thread: 512 or 1024 in the decode shrink, 256 or 512 in the tile-block shrink),
 // adapter ids that index a table of at most kSelfPlanWeights entries
-bool self_planned_ok(int T, int S, int n_weights, int nt_max) {
-  const int mt = tiles_per_wave(T);
+bool self_planned_ok(int T, int S, int n_weights, int nt_max, int mt) {
   const int segs = mt > 1 ? (S <= kFwdThreads ? kFwdThreads : kSelfPlanBlkSegs)
                           : (S <= kSelfPlanThreads ? kSelfPlanThreads : kSelfPlanSegs);
   return S <= segs && nt_max <= 4 * segs && n_weights >= 1 && n_weights <= kSelfPlanWeights &&
@@ -421,7 +433,7 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
-               const float* seg_scale, hipStream_t st, bool fold = true, bool w_kn = false,
+               const float* seg_scale, int mt, hipStream_t st, bool fold = true, bool w_kn = false,
                const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr, int packed = 0,
                const PlanSortArgs* build = nullptr) {
   if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
@@ -440,9 +452,9 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   bool need_reduce = false;
   ShrinkCfg c0{};
   size_t bits_off = 0;
-  const int nw = row_major ? kFwdWaves : shrink_waves(T, nproj, d_in, d_out);
+  const int nw = row_major ? kFwdWaves : shrink_waves(mt, nproj, d_in, d_out);
   for (int i = 0; i < nproj; ++i) {
-    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw, nproj == 1);
+    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw, nproj == 1, mt);
     if (i == 0) c0 = c;
     ShrinkProj& P = a.p[i];
     P.x = reinterpret_cast<const uint16_t*>(x[i]);
@@ -518,8 +530,9 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
     off = align_up(off + bytes, 256);
     return o;
   };
-  L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves, true);
-  L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves, true);
+  const int mt = bwd_tiles_per_wave(n_rows, r);
+  L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves, true, mt);
+  L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves, true, mt);
   const int ks_dv = fwd_ksplit_bound(n_rows, h_out, r), ks_v = fwd_ksplit_bound(n_rows, h_in, r);
   const int ks = ks_dv > ks_v ? ks_dv : ks_v;
   L.pitch = (long)plan_nt_max(n_rows, P) * kTileRows;
@@ -647,12 +660,12 @@ SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs
     P.v = reinterpret_cast<const uint16_t*>(x);
     P.w_ptrs = w_ptrs;
     P.d_in = d_in; P.d_out = d_out; P.ldw = w_ld;
-    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T), S, n_weights,
+    return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T, d_in), S, n_weights,
                          1, d_in, st, a);
   }
   float* partial = reinterpret_cast<float*>(workspace);
   return run_shrink(dtype, w_row_major != 0, pv, T, S, n_weights, 1, &x, &w_ptrs, &partial, &y, &d_in,
-                    d_out, &w_ld, beta, seg_scale, st);
+                    d_out, &w_ld, beta, seg_scale, tiles_per_wave(T, d_out), st);
 }
 
 SMLM_API int smlm_gemm_workspace_size(int T, int S, int d_in, int d_out, size_t* bytes) {
@@ -800,12 +813,13 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   float* partial[kMaxProj];
   void* v16[kMaxProj];
   int vsplit[kMaxProj];
-  const int nw = shrink_waves(T, n_proj, h_in, r);
-  bool expand_folds = nw == kDecodeWaves && tiles_per_wave(T) == 1;
+  const int mt = tiles_per_wave(T, r);
+  const int nw = shrink_waves(mt, n_proj, h_in, r);
+  bool expand_folds = nw == kDecodeWaves && mt == 1;
   {
     char* w = reinterpret_cast<char*>(workspace);
     for (int i = 0; i < n_proj; ++i) {
-      vsplit[i] = shrink_cfg(T, h_in[i], r, nw, n_proj == 1).ksplit;
+      vsplit[i] = shrink_cfg(T, h_in[i], r, nw, n_proj == 1, mt).ksplit;
       expand_folds = expand_folds && vsplit[i] <= kMaxExpandFold;
       partial[i] = reinterpret_cast<float*>(w);
       w += align_up((size_t)fwd_ksplit_bound(T, h_in[i], r) * T * r * 4, 256);
@@ -819,13 +833,13 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   bool even_splits = true;  // (the decode route pairs k slices up beyond 512 segments)
   for (int i = 0; i < n_proj; ++i) even_splits = even_splits && (vsplit[i] % 2 == 0);
   // (both routes pair k slices up in one workgroup beyond 512 / 256 segments)
-  const bool self_planned = build_s && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max) &&
-                            (tiles_per_wave(T) > 1 ? (S <= kFwdThreads || even_splits)
+  const bool self_planned = build_s && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max, mt) &&
+                            (mt > 1 ? (S <= kFwdThreads || even_splits)
                                                    : (expand_folds && (S <= kSelfPlanThreads || even_splits)));
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, S, st))) return rc;
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                    0.0f, nullptr, st, !expand_folds, false, &drop, w_rank, packed,
+                    0.0f, nullptr, mt, st, !expand_folds, false, &drop, w_rank, packed,
                     self_planned ? &build : nullptr);
     if (rc) return rc;
   }
@@ -855,8 +869,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
     }
   }
   if (n_exp == 0) return SMLM_OK;
-  return launch_expand(dtype, false, expand_nq(T, exp_h_out), tiles_per_wave(T), S, n_weights, n_exp, r,
-                       st, ea);
+  return launch_expand(dtype, false, expand_nq(T, exp_h_out), mt, S, n_weights, n_exp, r, st, ea);
 }
 
 SMLM_API int smlm_lora_fwd_workspace_size(int T, int S, int h_in, int h_out, int r, size_t* bytes) {
@@ -935,16 +948,17 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   const int32_t* build_k = opts ? opts->build_seg_adapter : nullptr;
   if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, P, next_pow2(P)};
-  const bool self_planned = build_s && v && !drop.seg_p && tiles_per_wave(n_rows) > 1 && r <= 64 &&
-                            self_planned_ok(n_rows, P, NA, pv.nt_max) &&
+  const int mt = bwd_tiles_per_wave(n_rows, r);
+  const bool self_planned = build_s && v && !drop.seg_p && mt > 1 && r <= 64 &&
+                            self_planned_ok(n_rows, P, NA, pv.nt_max, mt) &&
                             (P <= kFwdThreads || L.cfg_dv.ksplit % 2 == 0);  // (k slices in pairs beyond 256 partitions)
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, P, st))) return rc;
 
   // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The
-  // tile-block kernels (1024 rows and more) read the weights as they lie in memory; smaller
-  // batches work on transposed copies At [h_in, r], Bt [r, h_out] made here.
-  // (ranks above 64 take the one-tile expand kernel's general k loop, which reads [n][k] weights)
-  const bool in_place = tiles_per_wave(n_rows) > 1 && r <= 64;
+  // tile-block kernels read the weights as they lie in memory; ranks above 64 take the one-tile
+  // expand kernel's general k loop, which reads [n][k] weights: transposed copies At [h_in, r],
+  // Bt [r, h_out] made here.
+  const bool in_place = mt > 1 && r <= 64;
   if (!in_place) {
     TransposeArgs ta{};
     ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
@@ -973,7 +987,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
     DropArgs vdrop = drop;
     vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
-                         0.0f, nullptr, st, true, false, &vdrop, w_rank)))  // v of the dropped x, as the forward made it
+                         0.0f, nullptr, mt, st, true, false, &vdrop, w_rank)))  // v of the dropped x, as the forward made it
       return rc;
     vv = reinterpret_cast<const uint16_t*>(v16);
   }
@@ -982,7 +996,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   const void* const* btp = in_place ? b_ptrs : bt_ptrs;
   const int b_ld = in_place ? r : h_out;
   if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
-                       0.0f, nullptr, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
+                       0.0f, nullptr, mt, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
                        self_planned ? &build : nullptr)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
 
@@ -1005,8 +1019,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   }
   ea.w_kn = in_place ? 1 : 0;
   ea.drop = drop;  // dX is the gradient with respect to x before its dropout
-  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), tiles_per_wave(n_rows), P, NA, 1, r, st,
-                          ea)))
+  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), mt, P, NA, 1, r, st, ea)))
     return rc;
 
   // 5. dA_a, dB_a for every adapter (zeros when it has no rows)

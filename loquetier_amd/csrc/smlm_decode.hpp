@@ -321,7 +321,7 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
   }
 }
 
-// ---- batches of 1024 rows and more: the tile-block shrink_block_kernel ------------------------
+// ---- larger batches: the tile-block shrink_block_kernel ------------------------
 // WKN: the weights are stored [k][n], as B is for the backward's dV = dY B.
 // THREADS = 256: a workgroup is the four waves of shrink_block_kernel and takes one k slice of its
 // tile block.  THREADS = 512 (more than 256 segments; finder and plan builders hold a segment per

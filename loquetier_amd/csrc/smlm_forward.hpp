@@ -206,7 +206,7 @@ struct ShrinkArgs {
   DropArgs drop;              // DROP kernels: dropout of the training rows of x
 };
 
-// Shrink for single tiles (batches below 1024 rows).  Work item -> (projection, k
+// Shrink for single tiles (batches of few rows).  Work item -> (projection, k
 // slice, 64-column block, tile).  The NW waves of a workgroup take consecutive k
 // ranges; their accumulators are summed through LDS in wave order and written
 // either as an fp32 partial (k split over workgroups, or a consumer that folds)
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
   }
 }
 
-// Shrink for tile blocks (batches of 1024 rows and more).  Work item -> (projection, k
+// Shrink for tile blocks (larger batches, and the backward).  Work item -> (projection, k
 // slice, 64-column block, tile block) as above, but here wave w owns tile w of the block
 // and all four waves walk the whole k slice together: each 32*U-wide batch of the weight
 // rows is staged once in LDS (two buffers in turn, one barrier a batch) and shared by the

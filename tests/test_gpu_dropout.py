@@ -158,7 +158,7 @@ BWD_CASES = [
     ("shared-adapter", [0, 40, 70, 100], [1, 0, 1], 2, 128, 256, 16, [0.5, 0.0]),   # adapter 0 trains without dropout
     ("empty-part", [0, 17, 17, 50], [0, 1, 2], 3, 256, 128, 32, [0.5, 0.5, 0.5]),
     ("rank64", [0, 33, 90], [0, 1], 2, 192, 320, 64, [0.5, 0.5]),
-    ("in-place", [0, 500, 520, 1300], [2, 0, 2], 3, 256, 192, 16, [0.5, 0.0, 0.5]),  # 1024 rows and more: no transposes
+    ("in-place", [0, 500, 520, 1300], [2, 0, 2], 3, 256, 192, 16, [0.5, 0.0, 0.5]),  # tile blocks: no transposes
     ("many-rows", [0, 1100, 2300], [0, 1], 2, 320, 128, 32, [0.5, 0.5]),             # four-wave weight gradient
     ("long-k", [0, 30, 75], [1, 0], 2, 4096, 2048, 16, [0.5, 0.5]),
 ]

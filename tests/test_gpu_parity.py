@@ -367,7 +367,7 @@ def test_forward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     (4100, 21, 3, 64, 10240, 32),    # the same at rank 32, rows past a multiple of 64
     (8192, 90, 7, 64, 768, 64),      # rank 64 at 8192 rows: 256 columns, three chunk rows rounded up to four
     (8200, 50, 6, 64, 1032, 48),     # ... and a width that ends inside a chunk (five chunk rows -> six)
-    (1100, 12, 4, 64, 640, 16),      # 128 columns, five chunk rows rounded up to six
+    (2600, 12, 4, 64, 640, 16),      # 128 columns, five chunk rows rounded up to six
     (1100, 12, 4, 64, 1160, 64),     # 128 columns at rank 64 below 8192 rows, ragged last chunk (ten rows)
     (4100, 15, 3, 11008, 128, 64),   # the shrink of one projection from 4096 rows on: k split in eight, ragged last slice
     (6200, 9, 2, 4096, 64, 64),      # ... k split in three: one empty chunk row
@@ -392,9 +392,9 @@ def _ragged_segments(rng, T, S):
 
 @pytest.mark.parametrize("dt", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [
-    # T, S, NA, h_in, h_out, r: tile blocks of four (T >= 1024), ragged groups
+    # T, S, NA, h_in, h_out, r: tile blocks of four (larger batches: from 512 rows at rank 64 to 2560 at rank 16), ragged groups
     (1500, 40, 7, 512, 768, 32),
-    (2048, 300, 5, 256, 264, 16),
+    (2600, 300, 5, 256, 264, 16),
     (1100, 3, 3, 128, 1024, 64),
     # more than 1024 segments: two-launch plan with the sort in LDS
     (3000, 1500, 37, 128, 160, 8),

@@ -54,8 +54,8 @@ CASES = [
     ("rank128", list(range(0, 100, 2)), decode_ids(49, 5, 9), 5, 98, 128, [(4096, 256)]),
     ("rank72-tile-blocks", [0, 600, 1200, 1210], [1, 0, 1], 2, 1210, 72, [(512, 128)]),
     ("short-k-falls-back", list(range(41)), decode_ids(40, 4, 8), 4, 40, 16, [(512, 256)]),   # four-wave shrink: plan launch first
-    # 1024 rows and more: the tile-block shrink finds its tile blocks (up to 256 segments)
-    ("tile-blocks", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 16, [(2048, 320)]),
+    # larger batches (from 512 rows at rank 64, 2560 at rank 16): the tile-block shrink finds its tile blocks (up to 256 segments)
+    ("tile-blocks", [0, 700, 1100, 1101, 1500], [0, 1, 3, 2], 4, 1500, 64, [(2048, 320)]),
     ("tile-blocks-finetune-serve", [0, 1024, 2048, 3072, 4096] + list(range(4097, 4225)),
      [0, 1, 2, 3] + [4 + i % 32 for i in range(128)], 36, 4224, 16, [(4096, 512)]),
     ("tile-blocks-prefill-mlp", [0, 512, 1024, 1536, 2048] + list(range(2049, 2113)), [i % 16 for i in range(68)], 16, 2112,
@@ -63,11 +63,11 @@ CASES = [
     ("tile-blocks-256-segments", [5 * i for i in range(257)], [(i * 7) % 300 for i in range(256)], 300, 1300, 64,
      [(512, 128)]),
     ("tile-blocks-257-segments-odd-split-falls-back", [5 * i for i in range(258)], [(i * 7) % 300 for i in range(257)], 300,
-     1300, 8, [(512, 128)]),
+     1300, 64, [(512, 128)]),
     # beyond 256 segments: two groups of four waves a workgroup (the k splits must be even)
-    ("tile-blocks-300-segments", [5 * i for i in range(301)], [(i * 7) % 300 for i in range(300)], 300, 1510, 16,
+    ("tile-blocks-300-segments", [5 * i for i in range(301)], [(i * 7) % 300 for i in range(300)], 300, 1510, 64,
      [(2048, 128), (4096, 64)]),
-    ("tile-blocks-300-segments-ragged-k", [5 * i for i in range(301)], [(i * 7) % 30 for i in range(300)], 30, 1510, 16,
+    ("tile-blocks-300-segments-ragged-k", [5 * i for i in range(301)], [(i * 7) % 30 for i in range(300)], 30, 1510, 64,
      [(3400, 72)]),   # four k slices of 1024, the last one 328 long
     ("tile-blocks-512-segments", [3 * i for i in range(513)], [(i * 5) % 37 for i in range(512)], 37, 1540, 32,
      [(2048, 192)]),
@@ -162,7 +162,8 @@ def test_deferred_plan_is_built_by_other_users_first(K, gpu_device):
 
 @pytest.mark.parametrize("seed", range(12, 20))
 def test_random_tile_block_batches(K, gpu_device, seed):
-    """The same for batches of 1024 rows and more (tile blocks of up to 64 rows of one adapter)."""
+    """The same for larger batches (tile blocks of up to 64 rows of one adapter; a batch of 1024 to
+    2560 rows takes them or the single tiles according to its rank)."""
     rng = np.random.default_rng(800 + seed)
     d, tdt = gpu_device, [torch.float16, torch.bfloat16][seed % 2]
     NA = int(rng.choice([2, 9, 64, 100, 300, 1024]))
@@ -170,13 +171,14 @@ def test_random_tile_block_batches(K, gpu_device, seed):
     lens = rng.integers(0, 12, S) if S < 257 else rng.integers(0, 5, S)
     big = rng.random(S) < 0.08
     lens[big] = rng.integers(100, 700, int(big.sum()))
-    if lens.sum() < 1024:
-        lens[0] += 1100
+    r = int(rng.choice([8, 16, 32, 64]))
+    rows = {8: 2560, 16: 2560, 32: 1280, 64: 512}[r]   # where the forward changes over to tile blocks at this rank
+    if lens.sum() < rows:
+        lens[0] += rows + 76
     seg = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     ids = rng.integers(0, NA, S).astype(np.int32)
     ids[rng.random(S) < 0.03] = -1
     T = int(seg[-1]) + int(rng.integers(0, 40))
-    r = int(rng.choice([8, 16, 32, 64]))
     h_in, h_out = int(rng.choice([256, 1024, 2048])), int(rng.choice([64, 136]))
     gen = torch.Generator().manual_seed(int(seed))
     used = sorted(set(int(i) for i in ids if i >= 0))
@@ -291,7 +293,8 @@ BWD_CASES = [
     ("rank64-many-parts", [0] + [37 * i + 900 for i in range(1, 200)], [i % 5 for i in range(199)], 5, 320, 128, 64, True),
     ("300-partitions", [0] + [7 * i + 100 for i in range(1, 301)], [i % 9 for i in range(300)], 9, 256, 2048, 16, True),
     ("v-recomputed-falls-back", [0, 700, 1400], [0, 1], 2, 256, 128, 32, False),
-    ("single-tiles-fall-back", [0, 35, 90], [0, 1], 2, 192, 320, 16, True),
+    ("few-rows", [0, 35, 90], [0, 1], 2, 192, 320, 16, True),
+    ("rank72-single-tiles-fall-back", [0, 35, 90], [0, 1], 2, 192, 320, 72, True),
 ]
 
 
@@ -299,7 +302,7 @@ BWD_CASES = [
 @pytest.mark.parametrize("case", BWD_CASES, ids=[c[0] for c in BWD_CASES])
 def test_backward_deferred_plan_equals_built_plan(K, gpu_device, case, dt):
     """The backward builds a deferred plan too -- inside its dV shrink when that is the first launch to
-    need it (1024 rows and more, v given, no dropout), with the plan launch otherwise."""
+    need it (ranks up to 64, v given, no dropout), with the plan launch otherwise."""
     name, tp, part_ad, NA, h_in, h_out, r, with_v = case
     d, tdt = gpu_device, TDT[dt]
     n_rows = tp[-1]
