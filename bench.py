@@ -99,7 +99,7 @@ def single_tiles(T: int, r: int) -> bool:
     """Whether the forward of a batch of T rows at rank r runs on single 16-row tiles (the decode route)
     or on tile blocks: the library's rule, loquetier_amd/csrc/smlm_api.hip (tiles_per_wave); only used
     here to say in the output how the step's plan is built."""
-    return T < (2560 if r <= 16 else 1280 if r <= 32 else 1024 if r <= 48 else 512 if r <= 64 else 1024)
+    return T < (2048 if r <= 16 else 768 if r <= 32 else 512 if r <= 48 else 128 if r <= 64 else 1024)
 
 
 def algorithmic_bytes(w, h_in, h_out, accumulate=True):

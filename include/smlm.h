@@ -274,9 +274,9 @@ typedef struct smlm_dropout {
  *                  for every later call on the stream) and uses it.  The reference sets its
  *                  problems up inside every call as well (precompute_smlm_forward_args,
  *                  kernel_src/csrc/smlm_forward/smlm_forward_cutlass.cuh:31-46,76-79).  With
- *                  n_weights <= 1024, no dropout and either a batch of few rows (below 2560 rows
- *                  at rank <= 16, 1280 at rank <= 32, 1024 at rank <= 48, 512 at rank <= 64,
- *                  1024 above: the single-tile kernels), S <= 1024 and every h_in >= 2048, or a
+ *                  n_weights <= 1024, no dropout and either a batch of few rows (the single-tile
+ *                  kernels: below 2048 rows at rank <= 16, 768 at rank <= 32, 512 at rank <= 48,
+ *                  128 at rank <= 64, 1024 above), S <= 1024 and every h_in >= 2048, or a
  *                  larger batch with S <= 512 and T / 16 + S < 1024, this costs no
  *                  launch: the shrink's workgroups derive their own tiles from the two arrays
  *                  while a few more workgroups of the same launch write the plan; other batches

@@ -42,11 +42,15 @@ int launch(void (*kernel)(A), dim3 grid, dim3 block, hipStream_t st, const A& a)
 // segmentation, so re-segmenting a batch cannot change a bit of any row. ----
 // Tiles per work item: single 16-row tiles for batches of few rows, tile blocks (up to kBlkTiles tiles of one
 // adapter, their weights staged once in LDS) for larger ones.  Where the forward changes over depends on the
-// rank -- the tile-block kernels save weight traffic in proportion to it (4096 -> 4096, one projection, single
-// tiles / tile blocks in us: rank 16 at 2000 rows 18.4 / 20.8, at 3072 rows 26.0 / 24.5; rank 32 at 1024 rows
-// 15.6 / 17.8, at 1536 rows 21.7 / 19.2; rank 64 at 512 rows 17.7 / 17.1, at 1000 rows 22.9 / 18.8).
+// rank -- the tile-block kernels save weight traffic in proportion to it.  Single tiles / tile blocks in us, one
+// projection 4096 -> 4096: rank 16 at 2000 rows 18.4 / 20.8, at 3072 rows 26.0 / 24.5; rank 32 at 1024 rows
+// 15.6 / 17.8, at 1536 rows 21.7 / 19.2; rank 64 at 256 rows 17.0 / 16.3, at 1000 rows 22.9 / 18.8.  A launch of
+// several projections, whose workgroups fill the chip together, would change over earlier (q/k/v/o: rank 16 at
+// 1024 rows 30.9 / 30.9, at 2048 rows 53.1 / 47.5; rank 32 at 384 rows 24.5 / 25.3, at 768 rows 34.6 / 30.7;
+// rank 64 at 128 rows 27.6 / 24.7); the rule lies between the two and does not look at the number of
+// projections, so that a launch of several gives the bits that launches of one give.
 inline int tiles_per_wave(int T, int r) {
-  const int from = r <= 16 ? 2560 : (r <= 32 ? 1280 : (r <= 48 ? 1024 : (r <= 64 ? 512 : 1024)));
+  const int from = r <= 16 ? 2048 : (r <= 32 ? 768 : (r <= 48 ? 512 : (r <= 64 ? 128 : 1024)));
   return T >= from ? kBlkTiles : 1;
 }
 // The backward runs on tile blocks at every size up to rank 64: its single-tile route needs transposed copies
@@ -95,7 +99,9 @@ int shrink_waves(int mt, int nproj, const int* d_in, int d_out) {
   return all_long ? kDecodeWaves : kFwdWaves;
 }
 
-// solo: the launch has this one projection (a launch of several fills the chip with their workgroups together)
+// solo: the product is only ever launched by itself (the backward's dV and v products) and may take the
+// splits that suit a launch of one projection; the forward's projections keep one rule
+// whether they are launched alone or together, so that either way gives the same bits
 ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw, bool solo, int mt) {
   ShrinkCfg c;
   c.zblocks = ceil_div(d_out, 64);
@@ -435,7 +441,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
                const float* seg_scale, int mt, hipStream_t st, bool fold = true, bool w_kn = false,
                const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr, int packed = 0,
-               const PlanSortArgs* build = nullptr) {
+               const PlanSortArgs* build = nullptr, bool solo = false) {
   if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
   ShrinkArgs a{};
   if (drop) a.drop = *drop;
@@ -454,7 +460,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   size_t bits_off = 0;
   const int nw = row_major ? kFwdWaves : shrink_waves(mt, nproj, d_in, d_out);
   for (int i = 0; i < nproj; ++i) {
-    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw, nproj == 1, mt);
+    const ShrinkCfg c = shrink_cfg(T, d_in[i], d_out, nw, solo, mt);
     if (i == 0) c0 = c;
     ShrinkProj& P = a.p[i];
     P.x = reinterpret_cast<const uint16_t*>(x[i]);
@@ -819,7 +825,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   {
     char* w = reinterpret_cast<char*>(workspace);
     for (int i = 0; i < n_proj; ++i) {
-      vsplit[i] = shrink_cfg(T, h_in[i], r, nw, n_proj == 1, mt).ksplit;
+      vsplit[i] = shrink_cfg(T, h_in[i], r, nw, false, mt).ksplit;
       expand_folds = expand_folds && vsplit[i] <= kMaxExpandFold;
       partial[i] = reinterpret_cast<float*>(w);
       w += align_up((size_t)fwd_ksplit_bound(T, h_in[i], r) * T * r * 4, 256);
@@ -987,7 +993,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
     DropArgs vdrop = drop;
     vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
-                         0.0f, nullptr, mt, st, true, false, &vdrop, w_rank)))  // v of the dropped x, as the forward made it
+                         0.0f, nullptr, mt, st, true, false, &vdrop, w_rank, 0, nullptr, true)))  // v of the dropped x, as the forward made it
       return rc;
     vv = reinterpret_cast<const uint16_t*>(v16);
   }
@@ -997,7 +1003,7 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   const int b_ld = in_place ? r : h_out;
   if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
                        0.0f, nullptr, mt, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
-                       self_planned ? &build : nullptr)))
+                       self_planned ? &build : nullptr, true)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5

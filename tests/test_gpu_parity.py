@@ -369,10 +369,10 @@ def test_forward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     (8200, 50, 6, 64, 1032, 48),     # ... and a width that ends inside a chunk (five chunk rows -> six)
     (2600, 12, 4, 64, 640, 16),      # 128 columns, five chunk rows rounded up to six
     (1100, 12, 4, 64, 1160, 64),     # 128 columns at rank 64 below 8192 rows, ragged last chunk (ten rows)
-    (4100, 15, 3, 11008, 128, 64),   # the shrink of one projection from 4096 rows on: k split in eight, ragged last slice
+    (4100, 15, 3, 11008, 128, 64),   # k = 11008 split in five, ragged last slice: one empty chunk row
     (6200, 9, 2, 4096, 64, 64),      # ... k split in three: one empty chunk row
 ], ids=["r16-wide-aligned", "r32-wide-aligned", "r64-8192-rows", "r48-ragged-width", "odd-chunk-rows", "r64-short",
-        "k-split-eight", "k-split-three"])
+        "k-split-five", "k-split-three"])
 def test_forward_expand_launch_shapes(K, oracle, gpu_device, shape, dt):
     """The widths, row counts and ranks at which the tile-block launches change their columns per
     workgroup, their k split or pad their grid: bit-exact against the oracle."""
@@ -613,6 +613,23 @@ def test_backward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     x, A, B = make_case(oracle, 204, n_rows, None, None, NA, h_in, h_out, r, dt, dy=True)
     g = dyadic(np.random.default_rng(21), (n_rows, h_out), 16, 8)
     _bwd_exact(K, oracle, gpu_device, dt, x, A, B, g, tp, part_ad, r)
+
+
+@pytest.mark.parametrize("case", [
+    # n_rows, partitions, NA, h_in, h_out, r: shapes at which the backward's products, always launched alone,
+    # take the k splits of a lone projection
+    (4100, 5, 3, 64, 11008, 64),     # dV over k = 11008 from 4096 rows on: split in eight instead of five
+    (8200, 3, 2, 4096, 64, 64),      # v recomputed over k = 4096 at 8192 rows: split in four instead of two
+    (8192, 4, 2, 64, 14336, 16),     # dV over k = 14336 = 7 x 2048: split in four instead of seven
+], ids=["dv-k11008", "v-k4096-8192-rows", "dv-k14336"])
+def test_backward_lone_product_splits(K, oracle, gpu_device, case):
+    n_rows, P, NA, h_in, h_out, r = case
+    rng = np.random.default_rng(61)
+    tp = _ragged_segments(rng, n_rows, P)
+    part_ad = [int(i) % NA for i in range(P)]
+    x, A, B = make_case(oracle, 209, n_rows, None, None, NA, h_in, h_out, r, "bf16", dy=True)
+    g = dyadic(np.random.default_rng(24), (n_rows, h_out), 16, 8)
+    _bwd_exact(K, oracle, gpu_device, "bf16", x, A, B, g, tp, part_ad, r)
 
 
 def test_backward_is_deterministic(K, oracle, gpu_device):
