@@ -129,7 +129,10 @@ ShrinkCfg shrink_cfg(int T, int d_in, int d_out, int nw, bool solo, int mt) {
   if (max_split < 1) max_split = 1;
   if (max_split > kMaxKsplit) max_split = kMaxKsplit;
   const int ks = want < 1 ? 1 : (want > max_split ? max_split : want);
-  c.k_per_wave = round_up(ceil_div(d_in, c.NW * ks), kq);
+  // (the single-tile kernels' waves take a k range each: whole load batches a wave; a tile block's four
+  // waves walk one slice together, which is cut to whole load batches, so its slices come out nearly equal:
+  // k = 11008 in eight is seven slices of 1408 and one of 1152 instead of seven of 1536 and one of 256)
+  c.k_per_wave = round_up(ceil_div(d_in, c.NW * ks), c.MT > 1 ? kq / c.NW : kq);
   c.ksplit = ceil_div(d_in, c.NW * c.k_per_wave);
   // An odd split (h_in = 14336 falls into seven slices of 2048) gives way to an even one of equal slices that
   // still fills the chip twice: 8192 rows, h_in = 14336, k in four instead of seven: rank 16 61.6 -> 53.1 us,
