@@ -503,6 +503,22 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                                   v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f,
                                   adapter_rank=rank_f, packed_ranks=packed)
 
+    def bwd(st):
+        # every projection's backward in one set of launches (--bwd-per-projection: a call per projection)
+        pr, bplan = st["proj"], st["bplan"]
+        if args.bwd_per_projection:
+            for i, d in enumerate(pr):
+                K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
+                                     d["ta_tab"], d["tb_tab"], bplan, r, part_scale,
+                                     dropout=drop_b[i] if drop_b else None, adapter_rank=rank_b,
+                                     packed_ranks=packed)
+            return
+        K.smlm_lora_backward_multi([d["dx"] for d in pr], [d["da_tab"] for d in pr], [d["db_tab"] for d in pr],
+                                   [d["g"] for d in pr], [d["x"] for d in pr], [d["v"] for d in pr],
+                                   [d["ta_tab"] for d in pr], [d["tb_tab"] for d in pr], bplan, r, part_scale,
+                                   dropout=drop_b[0] if drop_b else None, adapter_rank=rank_b,
+                                   packed_ranks=packed)
+
     def step(st, build_plan=True):
         if build_plan:
             # deferred: the forward call builds the plan itself -- decode batches inside their
@@ -513,12 +529,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
             if build_plan or "bplan" not in st:
                 st["bplan"] = K.SegmentPlan(part_indptr, part_ad, n_train, buf=st["bplan_buf"],
                                             defer=not args.plan_launch)
-            bplan = st["bplan"]
-            for i, d in enumerate(st["proj"]):
-                K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
-                                     d["ta_tab"], d["tb_tab"], bplan, r, part_scale,
-                                     dropout=drop_b[i] if drop_b else None, adapter_rank=rank_b,
-                                     packed_ranks=packed)
+            bwd(st)
 
     # eager once on the capture stream (sizes its workspace outside any capture)
     cap_stream = torch.cuda.Stream()
@@ -770,6 +781,8 @@ def main():
     ap.add_argument("--padded-storage", action="store_true",
                     help="workloads with adapters below the padded rank: pass the true ranks but keep the "
                          "adapters zero-padded in memory (default: stored at their own rank, packed)")
+    ap.add_argument("--bwd-per-projection", action="store_true",
+                    help="workloads with a backward: one backward call per projection instead of one for all")
     ap.add_argument("--dropout", type=float, default=0.0,
                     help="dropout probability of the training adapters (workloads with a backward): the "
                          "kernels regenerate the mask in the forward and the backward; default 0 = off")

@@ -322,6 +322,30 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
                               const float* part_scale, const smlm_lora_opts* opts, void* stream);
 
 /*
+ * The backward of up to 8 projections of one batch in one set of launches (one dV product, one
+ * fold, one dX product, one weight-gradient launch for all of them): the projections share the
+ * partition plan, the adapters' indices, the rank and the scale, as q/k/v/o or gate/up/down of
+ * a layer do.  dx, da_ptrs, db_ptrs, dy, x, v, a_ptrs, b_ptrs, h_in, h_out are HOST arrays of
+ * n_proj entries, each entry what smlm_lora_bwd_ex takes for one projection; v is NULL or
+ * names the saved intermediate of every projection.  Results equal n_proj calls of
+ * smlm_lora_bwd_ex bit for bit (the kernels and their launch shapes per projection are the same).
+ * With dropout, projection i uses the stream offset + i and the caller's keep bits of the
+ * projections lie end to end, as smlm_lora_fwd_multi_ex leaves them.  No counterpart in the
+ * reference, whose backward is a Python loop per layer and partition
+ * (src/loquetier_src/kernel_utils.py:128-147).
+ */
+SMLM_API int smlm_lora_bwd_multi_workspace_size(int n_proj, int n_rows, int P, int NA, const int* h_in,
+                                                const int* h_out, int r, size_t* bytes);
+SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* const* da_ptrs,
+                                    void* const* const* db_ptrs, const void* const* dy,
+                                    const void* const* x, const void* const* v,
+                                    const void* const* const* a_ptrs, const void* const* const* b_ptrs,
+                                    const void* plan, void* workspace, size_t workspace_bytes,
+                                    int n_rows, int P, int NA, const int* h_in, const int* h_out, int r,
+                                    int dtype, const float* part_scale, const smlm_lora_opts* opts,
+                                    void* stream);
+
+/*
  * RMSNorm forward.  Replaces dispatch_rms_norm / rms_norm<T>
  * (kernel_src/csrc/loquetier_ops.cc:326-358,
  * kernel_src/csrc/rms_norm/rms_norm_cutlass.cu:81-186):

@@ -62,6 +62,9 @@ SIGNATURES = {
                            _i, _vp, _vp]),
     "smlm_lora_bwd_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i,
                                    _i, _i, _vp, _popts, _vp]),
+    "smlm_lora_bwd_multi_workspace_size": (_i, [_i, _i, _i, _i, _pi, _pi, _i, _psz]),
+    "smlm_lora_bwd_multi_ex": (_i, [_i, _pvp, _pvp, _pvp, _pvp, _pvp, _pvp, _pvp, _pvp, _vp, _vp, _sz, _i, _i,
+                                    _i, _pi, _pi, _i, _i, _vp, _popts, _vp]),
     "smlm_rms_norm_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "smlm_rms_norm_bwd_workspace_size": (_i, [_i, _i, _psz]),
     "smlm_rms_norm_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),

@@ -333,7 +333,7 @@ int launch_expand_dt(bool row_major, bool block, int nq, int KS, dim3 grid, hipS
                      const ExpandArgs& a) {
   if (row_major)
     return launch(expand_wave_kernel<DT, 2, 0, true, DIRECT, false>, grid, dim3(kFwdThreads), st, a);
-  if (a.drop.seg_p) {  // the backward's dX with the dropout of x undone: one projection, no fold
+  if (a.drop.seg_p) {  // the backward's dX with the dropout of x undone: no fold
     const dim3 bl(kFwdThreads);
     if (block)  // launch_expand admits only [k][n] weights here
       return KS == 1 ? launch(expand_block_kernel<DT, 4, 1, DIRECT, true, true>, grid, bl, st, a)
@@ -366,7 +366,7 @@ int launch_expand(int dtype, bool row_major, int nq, int MT, int S, int groups, 
                   hipStream_t st, ExpandArgs& a) {
   const int KS = max_d_in <= 32 ? 1 : (max_d_in <= 64 ? 2 : 0);
   const bool block = !row_major && MT > 1 && KS > 0;  // tile blocks with the weights staged in LDS
-  if (a.drop.seg_p && (row_major || nproj != 1 || a.p[0].vsplit > 0 || (block && !a.w_kn))) return SMLM_ERR_ARG;
+  if (a.drop.seg_p && (row_major || a.p[0].vsplit > 0 || (block && !a.w_kn))) return SMLM_ERR_ARG;
   if (row_major) nq = 2;
   // Tile blocks: 128 columns a workgroup, or 256 where measured better (rank 64, 8192 rows: 5-13 % at every
   // width; a row stride that is a multiple of 4 KiB, e.g. h_out = 14336, from 4096 rows on at every rank:
@@ -525,13 +525,17 @@ int launch_wgrad(int nbj, bool split, dim3 grid, hipStream_t st, const WgradArgs
   return launch(wgrad_kernel<DT, 4, 1>, grid, dim3(64), st, wa);
 }
 
+struct BwdProjLayout {
+  size_t at, bt, at_ptrs, bt_ptrs, partial, dv16, v16, pt_a, pt_b, bits;
+};
 struct BwdLayout {
-  size_t at, bt, at_ptrs, bt_ptrs, partial, dv16, v16, pt_a, pt_b, bits, total;
+  BwdProjLayout p[kMaxProj];
+  size_t total;
   long pitch;
-  ShrinkCfg cfg_dv, cfg_v;
 };
 
-BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
+// the projections' areas lie end to end, each laid out as a backward of that projection alone
+BwdLayout bwd_layout(int n_proj, int n_rows, int P, int NA, const int* h_in, const int* h_out, int r) {
   BwdLayout L;
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -539,22 +543,22 @@ BwdLayout bwd_layout(int n_rows, int P, int NA, int h_in, int h_out, int r) {
     off = align_up(off + bytes, 256);
     return o;
   };
-  const int mt = bwd_tiles_per_wave(n_rows, r);
-  L.cfg_dv = shrink_cfg(n_rows, h_out, r, kFwdWaves, true, mt);
-  L.cfg_v = shrink_cfg(n_rows, h_in, r, kFwdWaves, true, mt);
-  const int ks_dv = fwd_ksplit_bound(n_rows, h_out, r), ks_v = fwd_ksplit_bound(n_rows, h_in, r);
-  const int ks = ks_dv > ks_v ? ks_dv : ks_v;
   L.pitch = (long)plan_nt_max(n_rows, P) * kTileRows;
-  L.at = take((size_t)NA * h_in * r * 2);
-  L.bt = take((size_t)NA * h_out * r * 2);
-  L.at_ptrs = take((size_t)NA * 8);
-  L.bt_ptrs = take((size_t)NA * 8);
-  L.partial = take((size_t)ks * n_rows * r * 4);
-  L.dv16 = take((size_t)n_rows * r * 2);
-  L.v16 = take((size_t)n_rows * r * 2);
-  L.pt_a = take((size_t)r * L.pitch * 2);
-  L.pt_b = take((size_t)r * L.pitch * 2);
-  L.bits = take((size_t)n_rows * (h_in / 8));  // keep bits of x's dropout mask when the caller has none
+  for (int i = 0; i < n_proj; ++i) {
+    BwdProjLayout& Q = L.p[i];
+    const int ks_dv = fwd_ksplit_bound(n_rows, h_out[i], r), ks_v = fwd_ksplit_bound(n_rows, h_in[i], r);
+    const int ks = ks_dv > ks_v ? ks_dv : ks_v;
+    Q.at = take((size_t)NA * h_in[i] * r * 2);
+    Q.bt = take((size_t)NA * h_out[i] * r * 2);
+    Q.at_ptrs = take((size_t)NA * 8);
+    Q.bt_ptrs = take((size_t)NA * 8);
+    Q.partial = take((size_t)ks * n_rows * r * 4);
+    Q.dv16 = take((size_t)n_rows * r * 2);
+    Q.v16 = take((size_t)n_rows * r * 2);
+    Q.pt_a = take((size_t)r * L.pitch * 2);
+    Q.pt_b = take((size_t)r * L.pitch * 2);
+    Q.bits = take((size_t)n_rows * (h_in[i] / 8));  // keep bits of x's dropout mask when the caller has none
+  }
   L.total = off;
   return L;
 }
@@ -896,12 +900,19 @@ SMLM_API int smlm_lora_fwd(void* y, const void* x, void* v_out, const void* cons
                              SMLM_STAGE_SHRINK | SMLM_STAGE_EXPAND, stream);
 }
 
+SMLM_API int smlm_lora_bwd_multi_workspace_size(int n_proj, int n_rows, int P, int NA, const int* h_in,
+                                                const int* h_out, int r, size_t* bytes) {
+  if (n_proj < 1 || n_proj > kMaxProj || n_rows < 0 || P < 0 || NA < 0 || !h_in || !h_out || r <= 0 || !bytes)
+    return SMLM_ERR_ARG;
+  for (int i = 0; i < n_proj; ++i)
+    if (h_in[i] <= 0 || h_out[i] <= 0) return SMLM_ERR_ARG;
+  *bytes = bwd_layout(n_proj, n_rows > 0 ? n_rows : 1, P, NA > 0 ? NA : 1, h_in, h_out, r).total;
+  return SMLM_OK;
+}
+
 SMLM_API int smlm_lora_bwd_workspace_size(int n_rows, int P, int NA, int h_in, int h_out, int r,
                                           size_t* bytes) {
-  if (n_rows < 0 || P < 0 || NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0 || !bytes)
-    return SMLM_ERR_ARG;
-  *bytes = bwd_layout(n_rows > 0 ? n_rows : 1, P, NA > 0 ? NA : 1, h_in, h_out, r).total;
-  return SMLM_OK;
+  return smlm_lora_bwd_multi_workspace_size(1, n_rows, P, NA, &h_in, &h_out, r, bytes);
 }
 
 SMLM_API int smlm_lora_bwd(void* dx, void* const* da_ptrs, void* const* db_ptrs, const void* dy,
@@ -919,35 +930,44 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
                               const void* plan, void* workspace, size_t workspace_bytes,
                               int n_rows, int P, int NA, int h_in, int h_out, int r, int dtype,
                               const float* part_scale, const smlm_lora_opts* opts, void* stream) {
+  return smlm_lora_bwd_multi_ex(1, &dx, &da_ptrs, &db_ptrs, &dy, &x, v ? &v : nullptr, &a_ptrs, &b_ptrs, plan,
+                                workspace, workspace_bytes, n_rows, P, NA, &h_in, &h_out, r, dtype, part_scale,
+                                opts, stream);
+}
+
+SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* const* da_ptrs,
+                                    void* const* const* db_ptrs, const void* const* dy,
+                                    const void* const* x, const void* const* v,
+                                    const void* const* const* a_ptrs, const void* const* const* b_ptrs,
+                                    const void* plan, void* workspace, size_t workspace_bytes,
+                                    int n_rows, int P, int NA, const int* h_in, const int* h_out, int r,
+                                    int dtype, const float* part_scale, const smlm_lora_opts* opts,
+                                    void* stream) {
   int rc = check_common(n_rows, P, dtype);
   if (rc) return rc;
   DropArgs drop;
   if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
-  if (NA < 0 || h_in <= 0 || h_out <= 0 || r <= 0) return SMLM_ERR_ARG;
-  if ((h_in & 7) || (h_out & 7) || (r & 7)) return SMLM_ERR_ALIGN;
+  if (n_proj < 1 || n_proj > kMaxProj || NA < 0 || r <= 0 || !h_in || !h_out) return SMLM_ERR_ARG;
+  if (r & 7) return SMLM_ERR_ALIGN;
   if (NA == 0 || n_rows == 0 || P == 0) return SMLM_ERR_ARG;
-  if (!da_ptrs || !db_ptrs || !a_ptrs || !b_ptrs || !workspace) return SMLM_ERR_ARG;
-  if (!dx || !dy || !x || !plan) return SMLM_ERR_ARG;
-  if (!aligned16(dx) || !aligned16(dy) || !aligned16(x) || !aligned16(v) || !aligned16(workspace) ||
-      !aligned16(plan))
-    return SMLM_ERR_ALIGN;
-  const BwdLayout L = bwd_layout(n_rows, P, NA, h_in, h_out, r);
+  if (!dx || !da_ptrs || !db_ptrs || !dy || !x || !a_ptrs || !b_ptrs || !workspace || !plan) return SMLM_ERR_ARG;
+  if (!aligned16(workspace) || !aligned16(plan)) return SMLM_ERR_ALIGN;
+  bool have_v = v != nullptr && v[0] != nullptr;
+  for (int i = 0; i < n_proj; ++i) {
+    if (h_in[i] <= 0 || h_out[i] <= 0) return SMLM_ERR_ARG;
+    if ((h_in[i] & 7) || (h_out[i] & 7)) return SMLM_ERR_ALIGN;
+    if (!da_ptrs[i] || !db_ptrs[i] || !a_ptrs[i] || !b_ptrs[i] || !dx[i] || !dy[i] || !x[i]) return SMLM_ERR_ARG;
+    if (have_v != (v != nullptr && v[i] != nullptr)) return SMLM_ERR_ARG;  // v of every projection or of none
+    if (!aligned16(dx[i]) || !aligned16(dy[i]) || !aligned16(x[i]) || (have_v && !aligned16(v[i])))
+      return SMLM_ERR_ALIGN;
+  }
+  const BwdLayout L = bwd_layout(n_proj, n_rows, P, NA, h_in, h_out, r);
   if (workspace_bytes < L.total) return SMLM_ERR_WORKSPACE;
 
   hipStream_t st = (hipStream_t)stream;
   char* ws = reinterpret_cast<char*>(workspace);
-  uint16_t* at = reinterpret_cast<uint16_t*>(ws + L.at);
-  uint16_t* bt = reinterpret_cast<uint16_t*>(ws + L.bt);
-  const void** at_ptrs = reinterpret_cast<const void**>(ws + L.at_ptrs);
-  const void** bt_ptrs = reinterpret_cast<const void**>(ws + L.bt_ptrs);
-  float* partial = reinterpret_cast<float*>(ws + L.partial);
-  void* dv16 = ws + L.dv16;
-  void* v16 = ws + L.v16;
-  uint16_t* pt_a = reinterpret_cast<uint16_t*>(ws + L.pt_a);
-  uint16_t* pt_b = reinterpret_cast<uint16_t*>(ws + L.pt_b);
-
   PlanView pv{};
   plan_carve(const_cast<void*>(plan), n_rows, P, &pv);
 
@@ -958,9 +978,10 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, P, next_pow2(P)};
   const int mt = bwd_tiles_per_wave(n_rows, r);
-  const bool self_planned = build_s && v && !drop.seg_p && mt > 1 && r <= 64 &&
-                            self_planned_ok(n_rows, P, NA, pv.nt_max, mt) &&
-                            (P <= kFwdThreads || L.cfg_dv.ksplit % 2 == 0);  // (k slices in pairs beyond 256 partitions)
+  bool even_dv = true;  // (k slices in pairs beyond 256 partitions)
+  for (int i = 0; i < n_proj; ++i) even_dv = even_dv && shrink_cfg(n_rows, h_out[i], r, kFwdWaves, true, mt).ksplit % 2 == 0;
+  const bool self_planned = build_s && have_v && !drop.seg_p && mt > 1 && r <= 64 &&
+                            self_planned_ok(n_rows, P, NA, pv.nt_max, mt) && (P <= kFwdThreads || even_dv);
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, P, st))) return rc;
 
   // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The
@@ -969,42 +990,71 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   // Bt [r, h_out] made here.
   const bool in_place = mt > 1 && r <= 64;
   if (!in_place) {
-    TransposeArgs ta{};
-    ta.set[0] = TransposeSet{a_ptrs, at, at_ptrs, (long)h_in * r, r, h_in};
-    ta.set[1] = TransposeSet{b_ptrs, bt, bt_ptrs, (long)h_out * r, h_out, r};
-    ta.NA = NA;
-    ta.w_rank = w_rank;
-    ta.packed = packed;
-    const int gx = ceil_div(h_in > h_out ? h_in : h_out, 64), gy = ceil_div(r, 64);
-    if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
-  }
-
-  // The keep bits of x's dropout mask: the forward's when the caller kept them, else made here
-  // (same stream, same bits) so that the kernels below apply a stored mask either way.
-  if (drop.seg_p) {
-    drop.bits_pitch = h_in / 8;
-    if (!drop.bits) {
-      drop.bits = reinterpret_cast<uint8_t*>(ws + L.bits);
-      const DropBitsArgs ba{pv.hdr, pv.tile_row, pv.tile_rseg, drop};
-      if ((rc = launch(drop_bits_kernel, dim3((unsigned)pv.nt_max), dim3(256), st, ba))) return rc;
+    for (int i = 0; i < n_proj; ++i) {
+      TransposeArgs ta{};
+      ta.set[0] = TransposeSet{a_ptrs[i], reinterpret_cast<uint16_t*>(ws + L.p[i].at),
+                               reinterpret_cast<const void**>(ws + L.p[i].at_ptrs), (long)h_in[i] * r, r, h_in[i]};
+      ta.set[1] = TransposeSet{b_ptrs[i], reinterpret_cast<uint16_t*>(ws + L.p[i].bt),
+                               reinterpret_cast<const void**>(ws + L.p[i].bt_ptrs), (long)h_out[i] * r, h_out[i], r};
+      ta.NA = NA;
+      ta.w_rank = w_rank;
+      ta.packed = packed;
+      const int gx = ceil_div(h_in[i] > h_out[i] ? h_in[i] : h_out[i], 64), gy = ceil_div(r, 64);
+      if ((rc = launch(transpose_kernel, dim3(gx, gy, 2 * NA), dim3(256), st, ta))) return rc;
     }
   }
 
+  // The keep bits of x's dropout mask (projection i: the stream offset + i; the caller's bits of the
+  // projections lie end to end): the forward's when the caller kept them, else made here (same stream,
+  // same bits) so that the kernels below apply a stored mask either way.
+  const uint8_t* bits[kMaxProj] = {};
+  if (drop.seg_p) {
+    size_t bits_off = 0;
+    for (int i = 0; i < n_proj; ++i) {
+      if (drop.bits) {
+        bits[i] = drop.bits + bits_off;
+        bits_off += (size_t)drop.rows * (h_in[i] / 8);
+      } else {
+        DropArgs di = drop;
+        const uint64_t off = (((uint64_t)drop.o1 << 32) | drop.o0) + (uint32_t)i;
+        di.o0 = (uint32_t)off; di.o1 = (uint32_t)(off >> 32);
+        di.bits = reinterpret_cast<uint8_t*>(ws + L.p[i].bits);
+        di.bits_pitch = h_in[i] / 8;
+        bits[i] = di.bits;
+        const DropBitsArgs ba{pv.hdr, pv.tile_row, pv.tile_rseg, di};
+        if ((rc = launch(drop_bits_kernel, dim3((unsigned)pv.nt_max), dim3(256), st, ba))) return rc;
+      }
+    }
+  }
+
+  float* partial[kMaxProj];
+  void* dv16[kMaxProj];
+  void* v16[kMaxProj];
+  const void* vv[kMaxProj];
+  for (int i = 0; i < n_proj; ++i) {
+    partial[i] = reinterpret_cast<float*>(ws + L.p[i].partial);
+    dv16[i] = ws + L.p[i].dv16;
+    v16[i] = ws + L.p[i].v16;
+    vv[i] = have_v ? v[i] : v16[i];
+  }
+
   // 2. v = round16(x A^T) unless the forward saved it
-  const uint16_t* vv = reinterpret_cast<const uint16_t*>(v);
-  if (!vv) {
+  if (!have_v) {
     DropArgs vdrop = drop;
     vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
-    if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &x, &a_ptrs, &partial, &v16, &h_in, r, &h_in,
+    if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
                          0.0f, nullptr, mt, st, true, false, &vdrop, w_rank, 0, nullptr, true)))  // v of the dropped x, as the forward made it
       return rc;
-    vv = reinterpret_cast<const uint16_t*>(v16);
   }
 
   // 3. dV = round16(dY B)
-  const void* const* btp = in_place ? b_ptrs : bt_ptrs;
-  const int b_ld = in_place ? r : h_out;
-  if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, 1, &dy, &btp, &partial, &dv16, &h_out, r, &b_ld,
+  const void* const* btp[kMaxProj];
+  int b_ld[kMaxProj];
+  for (int i = 0; i < n_proj; ++i) {
+    btp[i] = in_place ? b_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].bt_ptrs);
+    b_ld[i] = in_place ? r : h_out[i];
+  }
+  if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, dy, btp, partial, dv16, h_out, r, b_ld,
                        0.0f, nullptr, mt, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
                        self_planned ? &build : nullptr, true)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
@@ -1014,21 +1064,25 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   ea.plan = tile_args(pv);
   ea.plan.w_rank = w_rank;
   ea.seg_scale = part_scale;
-  ea.pt_a = pt_a;
-  ea.pt_b = pt_b;
-  ea.v2 = vv;
   ea.beta = 0.0f;
   ea.T = n_rows; ea.nt_max = pv.nt_max;
-  {
-    ExpandProj& E = ea.p[0];
-    E.y = reinterpret_cast<uint16_t*>(dx);
-    E.v = reinterpret_cast<const uint16_t*>(dv16);
-    E.w_ptrs = in_place ? a_ptrs : at_ptrs;
-    E.d_in = r; E.d_out = h_in; E.ldw = in_place ? h_in : r;
+  int widest = 0;
+  for (int i = 0; i < n_proj; ++i) {
+    ExpandProj& E = ea.p[i];
+    E.y = reinterpret_cast<uint16_t*>(dx[i]);
+    E.v = reinterpret_cast<const uint16_t*>(dv16[i]);
+    E.w_ptrs = in_place ? a_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].at_ptrs);
+    E.d_in = r; E.d_out = h_in[i]; E.ldw = in_place ? h_in[i] : r;
+    E.pt_a = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_a);
+    E.pt_b = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_b);
+    E.v2 = reinterpret_cast<const uint16_t*>(vv[i]);
+    E.drop_bits = bits[i];
+    E.drop_pitch = h_in[i] / 8;
+    if (h_in[i] > widest) widest = h_in[i];
   }
   ea.w_kn = in_place ? 1 : 0;
   ea.drop = drop;  // dX is the gradient with respect to x before its dropout
-  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, h_in), mt, P, NA, 1, r, st, ea)))
+  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, widest), mt, P, NA, n_proj, r, st, ea)))
     return rc;
 
   // 5. dA_a, dB_a for every adapter (zeros when it has no rows)
@@ -1037,22 +1091,32 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
   wa.grp_tile = pv.grp_tile;
   wa.grp_id = pv.grp_id;
   wa.tile_row = pv.tile_row;
-  wa.q_a = reinterpret_cast<const uint16_t*>(x);
-  wa.q_b = reinterpret_cast<const uint16_t*>(dy);
-  wa.pt_a = pt_a;
-  wa.pt_b = pt_b;
-  wa.da_ptrs = da_ptrs;
-  wa.db_ptrs = db_ptrs;
+  wa.nproj = n_proj;
+  int chunks = 0;
+  for (int i = 0; i < n_proj; ++i) {
+    WgradProj& Q = wa.p[i];
+    Q.q_a = reinterpret_cast<const uint16_t*>(x[i]);
+    Q.q_b = reinterpret_cast<const uint16_t*>(dy[i]);
+    Q.pt_a = reinterpret_cast<const uint16_t*>(ws + L.p[i].pt_a);
+    Q.pt_b = reinterpret_cast<const uint16_t*>(ws + L.p[i].pt_b);
+    Q.da_ptrs = da_ptrs[i];
+    Q.db_ptrs = db_ptrs[i];
+    Q.h_in = h_in[i]; Q.h_out = h_out[i];
+    Q.chunks_a = ceil_div(h_in[i], kWgCols);
+    Q.chunk0 = chunks;
+    Q.drop_bits = bits[i];
+    Q.drop_pitch = h_in[i] / 8;
+    chunks += Q.chunks_a + ceil_div(h_out[i], kWgCols);
+  }
   wa.pitch = L.pitch;
-  wa.h_in = h_in; wa.h_out = h_out; wa.r = r;
-  wa.chunks_a = ceil_div(h_in, kWgCols);
+  wa.r = r;
   wa.n_parts = P;
   wa.grp_seg = pv.grp_seg;
   wa.w_rank = w_rank;
   wa.packed = packed;
   wa.drop = drop;  // dA against the dropped x
   // ranks above 64 are covered 64 at a time along the grid's z axis
-  dim3 grid(wa.chunks_a + ceil_div(h_out, kWgCols), NA, ceil_div(r, 64));
+  dim3 grid(chunks, NA, ceil_div(r, 64));
   const int nbj = r > 64 ? 4 : ceil_div(r, 16);
   // four waves splitting the rows of an adapter pay off when adapters have many rows each (whole backward,
   // 16 adapters at rank 16 / 64: 1024 rows each 124.7 -> 118.7 / 180.7 -> 175.3 us, 512 rows even, 256 rows

@@ -78,24 +78,36 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   }
 }
 
-struct WgradArgs {
-  const int32_t* hdr;
-  const int32_t* grp_tile;
-  const int32_t* grp_id;
-  const int32_t* tile_row;
+constexpr int kWgMaxProj = 8;  // projections one weight-gradient launch can serve (as the forward's launches)
+
+struct WgradProj {
   const uint16_t* q_a;   // x  [n_rows, h_in]   -> dA
   const uint16_t* q_b;   // dY [n_rows, h_out]  -> dB
   const uint16_t* pt_a;  // scale*dV by slot, transposed [r, pitch]
   const uint16_t* pt_b;  // scale*v  by slot, transposed [r, pitch]
   void* const* da_ptrs;  // [NA] -> [r, h_in]
   void* const* db_ptrs;  // [NA] -> [h_out, r]
+  int h_in, h_out, chunks_a;  // chunks_a = ceil(h_in/64): the projection's first chunks_a chunks work on dA
+  int chunk0;                 // first chunk (blockIdx.x) of this projection; its chunks lie end to end
+  const uint8_t* drop_bits;   // DROP kernels: keep bits of this projection's mask of x, [rows, drop_pitch]
+  long drop_pitch;
+};
+
+struct WgradArgs {
+  const int32_t* hdr;
+  const int32_t* grp_tile;
+  const int32_t* grp_id;
+  const int32_t* tile_row;
+  WgradProj p[kWgMaxProj];
+  int nproj;
   long pitch;
-  int h_in, h_out, r, chunks_a;  // chunks_a = ceil(h_in/64): blockIdx.x below it works on dA
+  int r;
   int n_parts;             // partitions the plan was laid out for (>= 1): its group tables hold n_parts + 1 entries
   const int32_t* w_rank;   // optional [NA]: true rank of each adapter (rows of dV / v past it are zero padding)
   int packed;              // with w_rank: dA_a [r_a, h_in] and dB_a [h_out, r_a] are stored at the true rank
   const int32_t* grp_seg;  // DROP kernels: first segment of every group (its adapter's dropout probability)
-  DropArgs drop;           // DROP kernels: dA is taken against the dropped x, regenerated while x is staged
+  DropArgs drop;           // DROP kernels: dA is taken against the dropped x (probabilities and row count; the
+                           //   keep bits are each projection's own)
 };
 
 constexpr int kWgCols = 64;     // columns of x / dY per workgroup
@@ -110,7 +122,7 @@ __device__ __forceinline__ int wg_lds_row(int s) {
   return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1);
 }
 
-// grid: (ceil(h_in/64) + ceil(h_out/64), NA, ceil(r/64)), block 64*NW.  A workgroup owns 64
+// grid: (sum over the projections of ceil(h_in/64) + ceil(h_out/64), NA, ceil(r/64)), block 64*NW.  A workgroup owns 64
 // columns (and up to 64 ranks) of one adapter's dA or dB and walks all of that adapter's tiles, 64
 // gathered rows (four tiles, two MFMA k steps) per wave and loop step.  With
 // NW = 4 (adapters with many rows each) the waves take steps round-robin and
@@ -123,11 +135,11 @@ __device__ __forceinline__ int wg_lds_row(int s) {
 // memory while the current step is multiplied.
 //
 // DROP (dA only): the forward multiplied the dropped x, so dA = dV^T dropout(x).  The keep
-// bits (one byte per eight columns, a.drop.bits) travel with the rows and are applied while the
+// bits (one byte per eight columns, the projection's drop_bits) travel with the rows and are applied while the
 // rows are staged; every row of the workgroup belongs to one adapter, whose probability is read
 // once from the group's first segment.
 template <int DT, int NBJ, int NW, bool IS_A, bool DROP = false>
-__device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
+__device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& P, int chunk, char* smem) {
   constexpr int kWgWaves = NW;
   constexpr int kStageElems = kWgSlots * kWgPitch;
   constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
@@ -135,11 +147,11 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
   const int ad = blockIdx.y;
   const int j0 = 64 * blockIdx.z;  // first rank of this workgroup (ranks above 64: 64 per z)
   constexpr bool is_a = IS_A;
-  const int n0 = (is_a ? blockIdx.x : blockIdx.x - a.chunks_a) * kWgCols;
-  const int h = is_a ? a.h_in : a.h_out;
-  const uint16_t* Q = is_a ? a.q_a : a.q_b;
-  const uint16_t* PT = is_a ? a.pt_a : a.pt_b;
-  uint16_t* out = reinterpret_cast<uint16_t*>(is_a ? a.da_ptrs[ad] : a.db_ptrs[ad]);
+  const int n0 = (is_a ? chunk : chunk - P.chunks_a) * kWgCols;
+  const int h = is_a ? P.h_in : P.h_out;
+  const uint16_t* Q = is_a ? P.q_a : P.q_b;
+  const uint16_t* PT = is_a ? P.pt_a : P.pt_b;
+  uint16_t* out = reinterpret_cast<uint16_t*>(is_a ? P.da_ptrs[ad] : P.db_ptrs[ad]);
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
@@ -214,7 +226,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, char* smem) {
       val[u] = ldg16_or_nt(Q + (long)row[u] * h + n0 + lcol, ok, zeros);
       if (DROP) {  // rows at or past drop.rows keep everything: their byte is never applied
         const bool dropped = ok && row[u] < a.drop.rows;
-        keep[u] = *(const SMLM_GLOBAL uint8_t*)(dropped ? a.drop.bits + (long)row[u] * a.drop.bits_pitch + ((n0 + lcol) >> 3)
+        keep[u] = *(const SMLM_GLOBAL uint8_t*)(dropped ? P.drop_bits + (long)row[u] * P.drop_pitch + ((n0 + lcol) >> 3)
                                                         : zero_bytes) | (dropped ? 0u : 0x100u);
       }
     }
@@ -390,10 +402,15 @@ __global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
   constexpr int kStageBytes = NW * kWgSlots * kWgPitch * 2;
   constexpr int kTailBytes = (NW > 1 ? NW * 4 * kWaveSize * 16 : 0) + 16 * (64 + 4) * 4;  // red + store staging
   __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kTailBytes ? kStageBytes : kTailBytes];
-  if ((int)blockIdx.x < a.chunks_a)  // uniform over the workgroup
-    wgrad_body<DT, NBJ, NW, true, DROP>(a, smem);
+  int pj = 0;
+#pragma unroll
+  for (int i = 1; i < kWgMaxProj; ++i) pj += (i < a.nproj && (int)blockIdx.x >= a.p[i].chunk0) ? 1 : 0;
+  const WgradProj& P = a.p[pj];
+  const int chunk = (int)blockIdx.x - P.chunk0;
+  if (chunk < P.chunks_a)  // uniform over the workgroup
+    wgrad_body<DT, NBJ, NW, true, DROP>(a, P, chunk, smem);
   else
-    wgrad_body<DT, NBJ, NW, false>(a, smem);
+    wgrad_body<DT, NBJ, NW, false>(a, P, chunk, smem);
 }
 
 }  // namespace smlm

@@ -536,6 +536,11 @@ struct ExpandProj {
   const float* vpart;         // VFOLD wave kernels: v arrives as vsplit (1..4) fp32 k-split partials
   int vsplit;                 //   [vsplit, T, d_in], summed here in split order and rounded
   int d_in, d_out, ldw;
+  uint16_t* pt_a;             // optional [d_in, nt_max*16]: scale*v by tile slot, transposed
+  uint16_t* pt_b;             // optional: same treatment of v2 (a second [T, d_in] matrix)
+  const uint16_t* v2;
+  const uint8_t* drop_bits;   // DROP kernels: keep bits of this projection's mask, [rows, drop_pitch]
+  long drop_pitch;
 };
 
 constexpr int kMaxVsplit = 4;  // most k-split partials of v the wave kernel folds itself
@@ -544,14 +549,12 @@ struct ExpandArgs {
   TileArgs plan;
   ExpandProj p[kMaxProj];
   const float* seg_scale;
-  uint16_t* pt_a;            // optional [d_in, nt_max*16]: scale*v by tile slot, transposed
-  uint16_t* pt_b;            // optional: same treatment of v2 (a second [T, d_in] matrix)
-  const uint16_t* v2;
   float beta;
   int T, nt_max;
   ItemSpace items;           // chunk rows of projection p: its column chunks
   int w_kn;                  // tile-block kernel only: weights are stored [k][n]
   DropArgs drop;             // DROP kernels (the backward's dX): the mask and factor applied to the stored values
+                             //   (probabilities and row count; the keep bits are each projection's own)
 };
 
 // by-products one wave per tile writes while it holds the token fragment: the
@@ -562,17 +565,17 @@ __device__ __forceinline__ void write_side(const ExpandArgs& a, const ExpandProj
                                            int kk, u32x4 vf, float scale) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
   if (P.v_out && row >= 0) stg16(P.v_out + (long)row * P.d_in + kk, vf);
-  if (a.pt_a) {
+  if (P.pt_a) {
     const long pitch = (long)a.nt_max * kTileRows;
     u32x4 v2f = zero;
-    if (a.pt_b && row >= 0) v2f = ldg16(a.v2 + (long)row * P.d_in + kk);
+    if (P.pt_b && row >= 0) v2f = ldg16(P.v2 + (long)row * P.d_in + kk);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      a.pt_a[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(vf[e]));
-      a.pt_a[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(vf[e]));
-      if (a.pt_b) {
-        a.pt_b[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(v2f[e]));
-        a.pt_b[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(v2f[e]));
+      P.pt_a[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(vf[e]));
+      P.pt_a[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(vf[e]));
+      if (P.pt_b) {
+        P.pt_b[(kk + 2 * e) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::lo(v2f[e]));
+        P.pt_b[(kk + 2 * e + 1) * pitch + slot] = (uint16_t)Num<DT>::bits(scale * Num<DT>::hi(v2f[e]));
       }
     }
   }
@@ -599,15 +602,15 @@ struct LineLane {
 // keep bits of the pieces a lane will store (DROP kernels): requested with the other loads of
 // the item; rows that are not dropped read a zero byte that is never applied
 template <int NQ>
-__device__ __forceinline__ void load_keep_bits(LineLane& L, const DropArgs& d, int ncol0, int d_out,
-                                               const uint16_t* zeros) {
+__device__ __forceinline__ void load_keep_bits(LineLane& L, const DropArgs& d, const uint8_t* bits, long bits_pitch,
+                                               int ncol0, int d_out, const uint16_t* zeros) {
 #pragma unroll
   for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int h = 0; h < NQ / 2; ++h) {
       const int col = ncol0 + 64 * h + L.ocol;
       const bool ok = L.srow[j] >= 0 && L.srow[j] < d.rows && col < d_out;  // whatever the row's probability
-      L.keep[h][j] = *(const SMLM_GLOBAL uint8_t*)(ok ? d.bits + (long)L.srow[j] * d.bits_pitch + (col >> 3)
+      L.keep[h][j] = *(const SMLM_GLOBAL uint8_t*)(ok ? bits + (long)L.srow[j] * bits_pitch + (col >> 3)
                                                       : reinterpret_cast<const uint8_t*>(zeros));
     }
 }
@@ -724,11 +727,11 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     }
     u32x4 yold[NQ / 2][2];
     load_y_lines<NQ>(yold, L, ncol0, P.d_out, a.beta != 0.0f, zeros);
-    if (DROP) load_keep_bits<NQ>(L, a.drop, ncol0, P.d_out, zeros);
+    if (DROP) load_keep_bits<NQ>(L, a.drop, P.drop_bits, P.drop_pitch, ncol0, P.d_out, zeros);
 #pragma unroll
     for (int j = 0; j < 2; ++j) L.scale[j] = sseg[j] >= 0 ? a.seg_scale[sseg[j]] : 1.0f;
 
-    const float scale = (side && a.pt_a && rseg >= 0) ? a.seg_scale[rseg] : 1.0f;  // for the by-products
+    const float scale = (side && P.pt_a && rseg >= 0) ? a.seg_scale[rseg] : 1.0f;  // for the by-products
 
     f32x4 acc[NQ][2];
 #pragma unroll
@@ -834,7 +837,7 @@ void expand_block_kernel(ExpandArgs a) {
       L.yrow[j] = P.y + (long)(L.srow[j] < 0 ? 0 : L.srow[j]) * P.d_out + ncol0 + L.ocol;
       if (DROP) L.drop[j] = drop_row(a.drop, L.srow[j], a.plan.tile_rseg, tslot + L.orow + 8 * j);
     }
-    const int rseg = (a.pt_a && a.seg_scale && active) ? a.plan.tile_rseg[slot] : -1;
+    const int rseg = (P.pt_a && a.seg_scale && active) ? a.plan.tile_rseg[slot] : -1;
     const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.plan.hdr + kHdrZeros);
 
     // Every load of the item is issued before anything waits for one (predicated-off loads
@@ -859,7 +862,7 @@ void expand_block_kernel(ExpandArgs a) {
     const bool read_y = a.beta != 0.0f;
     u32x4 yold[NQ / 2][2];
     load_y_lines<NQ>(yold, L, ncol0, P.d_out, read_y, zeros);
-    if (DROP) load_keep_bits<NQ>(L, a.drop, ncol0, P.d_out, zeros);
+    if (DROP) load_keep_bits<NQ>(L, a.drop, P.drop_bits, P.drop_pitch, ncol0, P.d_out, zeros);
     u32x4 vf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {

@@ -470,40 +470,83 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
     forward's stream with seg_p per partition; x is the tensor before dropout."""
-    for t, n in ((dx, "dx"), (dy, "dy"), (x, "x"), (da_ptrs, "da_ptrs"), (db_ptrs, "db_ptrs"),
-                 (a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs")):
-        _check_input(t, n)
+    smlm_lora_backward_multi([dx], [da_ptrs], [db_ptrs], [dy], [x], None if v is None else [v], [a_ptrs],
+                             [b_ptrs], plan, rank, part_scale=part_scale, dropout=dropout,
+                             adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks)
+
+
+_BWD_MULTI_SIZES: Dict[Tuple, int] = {}
+
+
+def _bwd_multi_workspace_size(n_rows: int, P: int, NA: int, widths_in: Tuple[int, ...],
+                              widths_out: Tuple[int, ...], rank: int) -> int:
+    key = (n_rows, P, NA, widths_in, widths_out, rank)
+    n = _BWD_MULTI_SIZES.get(key)
+    if n is None:
+        need = C.c_size_t(0)
+        CI = C.c_int * len(widths_in)
+        _lib.check(_lib.load().smlm_lora_bwd_multi_workspace_size(len(widths_in), n_rows, P, NA, CI(*widths_in),
+                                                                  CI(*widths_out), rank, C.byref(need)),
+                   "smlm_lora_bwd_multi_workspace_size")
+        n = _BWD_MULTI_SIZES[key] = need.value
+    return n
+
+
+def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int,
+                             part_scale: Optional[torch.Tensor] = None,
+                             dropout: Optional[DropoutSpec] = None,
+                             adapter_rank: Optional[torch.Tensor] = None,
+                             workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
+    """The backward of several projections of one batch (q/k/v/o, gate/up/down) in one set of
+    launches; lists of equal length, one entry per projection, each what smlm_lora_backward
+    takes.  vs: None, or the saved intermediate of every projection.  The results equal
+    per-projection calls bit for bit.  dropout: projection i uses the stream offset + i and
+    the keep bits of the projections lie end to end (as smlm_lora_forward_multi leaves them)."""
+    n = len(dxs)
+    lists = (da_ptrs, db_ptrs, dys, xs, a_ptrs, b_ptrs) + (() if vs is None else (vs,))
+    if not (1 <= n <= 8) or any(len(l) != n for l in lists):
+        raise RuntimeError("between 1 and 8 projections, all lists of one length")
     if plan.kind != _lib.SMLM_KEY_I32:
         raise RuntimeError("the backward plan must be built from int32 adapter ids")
     n_rows = plan.T
-    if dy.size(0) < n_rows or x.size(0) < n_rows or dx.size(0) < n_rows:
-        raise RuntimeError("dy, x and dx need at least plan.T rows")
-    if dx.dtype != dy.dtype or x.dtype != dy.dtype or (v is not None and v.dtype != dy.dtype):
-        raise RuntimeError("dx, dy, x, v must share one dtype")
-    NA = a_ptrs.size(0)
-    if b_ptrs.size(0) != NA or da_ptrs.size(0) != NA or db_ptrs.size(0) != NA:
-        raise RuntimeError("pointer tables must all have one entry per adapter")
-    if v is not None and (v.size(0) < n_rows or v.size(1) != rank or not v.is_contiguous()):
-        raise RuntimeError("v must be a contiguous [>=n_rows, rank] tensor")
-    code = _dtype_code(dy)
-    h_in, h_out = x.size(1), dy.size(1)
-    dev = dy.device
+    NA = a_ptrs[0].size(0)
+    dtype = dys[0].dtype
+    for i in range(n):
+        for t, name in ((dxs[i], "dx"), (dys[i], "dy"), (xs[i], "x"), (da_ptrs[i], "da_ptrs"),
+                        (db_ptrs[i], "db_ptrs"), (a_ptrs[i], "a_ptrs"), (b_ptrs[i], "b_ptrs")):
+            _check_input(t, name)
+        if dys[i].size(0) < n_rows or xs[i].size(0) < n_rows or dxs[i].size(0) < n_rows:
+            raise RuntimeError("dy, x and dx need at least plan.T rows")
+        v = None if vs is None else vs[i]
+        if dxs[i].dtype != dtype or xs[i].dtype != dtype or dys[i].dtype != dtype or \
+                (v is not None and v.dtype != dtype):
+            raise RuntimeError("dx, dy, x, v must share one dtype")
+        if any(t.size(0) != NA for t in (a_ptrs[i], b_ptrs[i], da_ptrs[i], db_ptrs[i])):
+            raise RuntimeError("pointer tables must all have one entry per adapter")
+        if vs is not None and (v is None or v.size(0) < n_rows or v.size(1) != rank or not v.is_contiguous()):
+            raise RuntimeError("v must be a contiguous [>=n_rows, rank] tensor (of every projection or of none)")
+        if dxs[i].size(1) != xs[i].size(1):
+            raise RuntimeError("dx and x must have the same width")
+    code = _dtype_code(dys[0])
+    widths_in = tuple(t.size(1) for t in xs)
+    widths_out = tuple(t.size(1) for t in dys)
+    dev = dys[0].device
+    VP, CI = C.c_void_p * n, C.c_int * n
     with _on(dev):
-        need = _lib.size_query("smlm_lora_bwd_workspace_size", n_rows, plan.S, NA, h_in, h_out, rank)
-        ws = _workspace(dev, need, workspace)
+        ws = _workspace(dev, _bwd_multi_workspace_size(n_rows, plan.S, NA, widths_in, widths_out, rank), workspace)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
-        opts = _opts(plan, dropout, h_in, adapter_rank, NA, packed_ranks)
+        opts = _opts(plan, dropout, list(widths_in), adapter_rank, NA, packed_ranks)
         if not plan.built:  # a deferred plan: this call builds it (inside its first launch where it can)
             opts = opts or _lib.LoraOpts()
             opts.build_seg_indptr = plan.segment.data_ptr()
             opts.build_seg_adapter = plan.seg_key.data_ptr()
-        rc = _lib.load().smlm_lora_bwd_ex(dx.data_ptr(), da_ptrs.data_ptr(), db_ptrs.data_ptr(),
-                                               dy.data_ptr(), x.data_ptr(), _ptr(v), a_ptrs.data_ptr(),
-                                               b_ptrs.data_ptr(), plan.buf.data_ptr(), ws.data_ptr(),
-                                               ws.numel(), n_rows, plan.S, NA, h_in, h_out, rank, code,
-                                               _ptr(part_scale), None if opts is None else C.byref(opts),
-                                               _stream(dev))
+        arr = lambda ts: VP(*[t.data_ptr() for t in ts])
+        rc = _lib.load().smlm_lora_bwd_multi_ex(
+            n, arr(dxs), arr(da_ptrs), arr(db_ptrs), arr(dys), arr(xs), None if vs is None else arr(vs),
+            arr(a_ptrs), arr(b_ptrs), plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), n_rows, plan.S, NA,
+            CI(*widths_in), CI(*widths_out), rank, code, _ptr(part_scale),
+            None if opts is None else C.byref(opts), _stream(dev))
     _lib.check(rc, "smlm_lora_backward")
     plan.built = True
 
