@@ -34,16 +34,23 @@ METRIC = "SMLM tokens/s + HBM GB/s (% of 8 TB/s), Llama-2-7B shapes, 1 GPU"
 
 def workload(name: str):
     """Shapes and routing of BASELINE.json's configs 2-5 (seeds = config number)."""
-    if name in ("cfg2", "cfg2mod", "cfg2one"):
+    if name in ("cfg2", "cfg2mod", "cfg2one", "cfg2layer"):
         # adapters drawn uniformly (the headline workload) or dealt round-robin, i % 32 (the variant);
         # cfg2one is the headline batch through ONE projection, what a single layer call of the reference issues
         ids = [i % 32 for i in range(256)] if name == "cfg2mod" else np.random.default_rng(2).integers(0, 32, 256).tolist()
         proj = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096)]
-        return dict(name=f"{name}: 256 single-token segments over 32 adapters"
-                         f"{' dealt round-robin' if name == 'cfg2mod' else ''}, r=16, "
-                         f"{'q' if name == 'cfg2one' else 'q/k/v/o'} 4096->4096, "
-                         "fp16, forward", dtype="fp16", r=16, NA=32, seg=list(range(257)), ids=ids,
-                    proj=proj[:1] if name == "cfg2one" else proj, n_train_parts=0)
+        w = dict(name=f"{name}: 256 single-token segments over 32 adapters"
+                      f"{' dealt round-robin' if name == 'cfg2mod' else ''}, r=16, "
+                      f"{'q' if name == 'cfg2one' else 'q/k/v/o'} 4096->4096, "
+                      "fp16, forward", dtype="fp16", r=16, NA=32, seg=list(range(257)), ids=ids,
+                 proj=proj[:1] if name == "cfg2one" else proj, n_train_parts=0)
+        if name == "cfg2layer":
+            # as a decoder layer can issue it: q, k, v read ONE input and go out in one call, o (whose input is the
+            # attention's output) in a call of its own
+            w["name"] = ("cfg2layer: the cfg2 batch as one decoder layer issues it -- q/k/v of one shared input in "
+                         "one call, then o in its own call, fp16, forward")
+            w["calls"], w["shared_x"] = [[0, 1, 2], [3]], {1: 0, 2: 0}
+        return w
     if name == "cfg3":
         return dict(name="cfg3: 4x512 prefill + 64 decode, 16 adapters, r=32, gate/up 4096->11008, "
                          "down 11008->4096, fp16, forward", dtype="fp16", r=32, NA=16,
@@ -65,7 +72,7 @@ def workload(name: str):
         lens[-1] -= sum(lens) - 8192
         seg = np.concatenate([[0], np.cumsum(lens)]).tolist()
         S = len(lens)
-        return dict(name="cfg5: 64 adapters, ranks {8,16,32,64} padded to 64, geometric segments, 8192 "
+        return dict(name="cfg5: 64 adapters of ranks {8,16,32,64}, geometric segments, 8192 "
                          "rows, Llama-3-8B shapes, bf16, fwd + bwd on first quarter of segments",
                     dtype="bf16", r=64, NA=64, seg=seg, ids=[i % 64 for i in range(S)],
                     proj=[("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024),
@@ -102,9 +109,10 @@ def single_tiles(T: int, r: int) -> bool:
     return T < (2048 if r <= 16 else 768 if r <= 32 else 512 if r <= 48 else 128 if r <= 64 else 1024)
 
 
-def algorithmic_bytes(w, h_in, h_out, accumulate=True):
+def algorithmic_bytes(w, h_in, h_out, accumulate=True, own_x=True):
     """Forward bytes of one projection: x and y once (y read too when accumulating),
-    A and B of each distinct active adapter once, v written and read once at I/O width."""
+    A and B of each distinct active adapter once, v written and read once at I/O width.
+    own_x False: the projection reads an input that another projection of the call is charged for."""
     T = w["seg"][-1]
     active = sorted(set(w["ids"]))
     ranks = w.get("true_ranks")
@@ -113,7 +121,7 @@ def algorithmic_bytes(w, h_in, h_out, accumulate=True):
     for i, a in enumerate(w["ids"]):
         n = w["seg"][i + 1] - w["seg"][i]
         vbytes += 2 * n * (ranks[a % 4] if ranks else w["r"]) * 2
-    return (T * h_in + T * h_out * (2 if accumulate else 1)) * 2 + rsum * (h_in + h_out) * 2 + vbytes
+    return (T * h_in * (1 if own_x else 0) + T * h_out * (2 if accumulate else 1)) * 2 + rsum * (h_in + h_out) * 2 + vbytes
 
 
 def backward_bytes(w, h_in, h_out):
@@ -215,7 +223,7 @@ def rmsnorm_bench(args, torch, K):
         "cpu_baseline": cpu}), flush=True)
 
 
-def model_step_bench(args, torch, K):
+def model_step_bench(args, torch, K, finetune=True):
     """The path as the reference drives it (src/loquetier_src/models/mixed_lora.py:173-218, 224 LoRA linears
     per model forward): 32 layers x (q, k, v, o, gate, up, down) of Llama-2-7B through MixedLoraLinear(fused=True)
     with ONE MixedLoraContext.update per step.  The base layers hand back preallocated outputs (their GEMMs
@@ -355,6 +363,8 @@ def model_step_bench(args, torch, K):
     del grouped
     del layers
     torch.cuda.empty_cache()
+    if not finetune:
+        return out
 
     # ---- fine-tune + serve batch, forward + backward through autograd (eager)
     w, ctx, layers, tdt = build("cfg4", [0, 1, 2, 3])
@@ -395,7 +405,103 @@ def model_step_bench(args, torch, K):
         host_us_per_call_backward=round((t1 - t_f) * 1e6 / len(layers), 2),
         eager_us_per_call_incl_gpu=round((t2 - t0) * 1e6 / len(layers), 2),
         event_us_per_call=round(a.elapsed_time(b) * 1e3 / len(layers), 2))
-    print(json.dumps(out), flush=True)
+    return out
+
+
+def reference_surface_bench(args, torch, K):
+    """One LoRA layer call of the decode batch through the surface the reference's own code calls, next to the
+    fused call: (1) the lines of the reference's add_lora.forward (src/loquetier_src/kernel_utils.py:113-119)
+    against this library's `_kernels` module -- three allocations and two smlm_forward_cutlass calls with
+    per-segment pointer tables -- followed by the caller's scale multiply and residual add
+    (models/mixed_lora.py:214-217); (2) the mirror `add_lora.apply` with the same tensors and the same two
+    caller ops; (3) the fused call (scale, residual add and the adapter gather inside the op) over a plan the
+    step's layers share.  GPU time per call from graph replays over rotating buffer sets."""
+    from loquetier_amd.kernel_utils import add_lora
+    dev = torch.device("cuda:0")
+    w = workload("cfg2one")
+    tdt = torch.float16
+    T, S, r, NA = w["seg"][-1], len(w["ids"]), w["r"], w["NA"]
+    _, hi, ho = w["proj"][0]
+    gen = torch.Generator(device="cpu").manual_seed(21)
+    seg_t = torch.tensor(w["seg"], dtype=torch.int32, device=dev)
+    ids_t = torch.tensor(w["ids"], dtype=torch.int32, device=dev)
+    lens_t = torch.ones(S, dtype=torch.int32, device=dev)
+    scaling = torch.full((NA,), 2.0, dtype=tdt, device=dev)
+    R = 16
+    sets = []
+    for _ in range(R):
+        A = (torch.randn(NA, r, hi, generator=gen) * hi ** -0.5).to(dev).to(tdt)
+        B = (torch.randn(NA, ho, r, generator=gen) * r ** -0.5).to(dev).to(tdt)
+        a_tab = torch.tensor([A[a].data_ptr() for a in range(NA)], dtype=torch.int64, device=dev)
+        b_tab = torch.tensor([B[a].data_ptr() for a in range(NA)], dtype=torch.int64, device=dev)
+        sets.append(dict(x=torch.randn(T, hi, generator=gen).to(dev).to(tdt), base=torch.randn(T, ho, generator=gen).to(dev).to(tdt),
+                         A=A, B=B, a_tab=a_tab, b_tab=b_tab, wa_ptr=a_tab[ids_t.long()], wb_ptr=b_tab[ids_t.long()]))
+    plan = K.SegmentPlan(seg_t, ids_t, T)
+    scale_seg = torch.full((S,), 2.0, device=dev)
+
+    def caller_tail(st, lora_res):  # mixed_lora.py:214-217
+        lora_res = lora_res * torch.repeat_interleave(scaling[ids_t.long()], lens_t.long(), output_size=T)[:, None]
+        return st["base"] + lora_res
+
+    def two_call(st):
+        x, s_, wa_ptr, wb_ptr = st["x"], seg_t, st["wa_ptr"], st["wb_ptr"]
+        y = torch.empty((T, ho), dtype=x.dtype, device=x.device)
+        tmp = torch.empty((K.smlm_forward_cutlass_tmp_size(s_.size(0) - 1),), dtype=torch.uint8, device=x.device)
+        v = torch.empty((x.size(0), r), dtype=x.dtype, device=x.device)
+        K.smlm_forward_cutlass(v, x, wa_ptr, s_, tmp, False)
+        K.smlm_forward_cutlass(y, v, wb_ptr, s_, tmp, False)
+        return caller_tail(st, y)
+
+    def mirror(st):
+        return caller_tail(st, add_lora.apply((T, ho), st["x"], st["wa_ptr"], st["wb_ptr"], seg_t, r, 0, []))
+
+    def fused(st):
+        K.smlm_lora_forward(st["base"], st["x"], st["a_tab"], st["b_tab"], plan, r, seg_scale=scale_seg, beta=1.0)
+
+    cap = torch.cuda.Stream()
+
+    def per_call_us(fn):
+        with torch.no_grad(), torch.cuda.stream(cap):
+            for st in sets[:2]:
+                fn(st)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(g, stream=cap):
+            for _ in range(2):
+                for st in sets:
+                    fn(st)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(2):
+            g.replay()
+        a.record()
+        for _ in range(10):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / (10 * 2 * R)
+
+    t_two, t_mirror, t_fused = per_call_us(two_call), per_call_us(mirror), per_call_us(fused)
+    tmp_t = torch.empty(K.smlm_forward_cutlass_tmp_size(S), dtype=torch.uint8, device=dev)
+    for st in sets:
+        st["v"], st["y"] = torch.empty(T, r, dtype=tdt, device=dev), torch.empty(T, ho, dtype=tdt, device=dev)
+
+    def two_call_kernels(st):  # the two GEMM calls alone: no allocation, no caller ops
+        K.smlm_forward_cutlass(st["v"], st["x"], st["wa_ptr"], seg_t, tmp_t, False)
+        K.smlm_forward_cutlass(st["y"], st["v"], st["wb_ptr"], seg_t, tmp_t, False)
+    t_two_k = per_call_us(two_call_kernels)
+    nbytes = algorithmic_bytes(w, hi, ho)
+    return dict(workload=w["name"] + ", one layer call",
+                fused_call_us=round(t_fused, 2),
+                reference_lines_two_calls_us=round(t_two, 2),
+                reference_lines_two_calls_kernels_only_us=round(t_two_k, 2),
+                add_lora_mirror_us=round(t_mirror, 2),
+                ratio_two_calls_vs_fused=round(t_two / t_fused, 2),
+                ratio_kernels_only_vs_fused=round(t_two_k / t_fused, 2),
+                ratio_mirror_vs_fused=round(t_mirror / t_fused, 2),
+                fused_call_hbm_gbps=round(nbytes / (t_fused * 1e-6) / 1e9, 1),
+                note="GPU time per layer call, graph replay over 16 rotating buffer sets; the reference-surface "
+                     "legs include the caller's scale multiply and residual add (two more passes over y) unless "
+                     "marked kernels only; the fused call reuses the step's plan")
 
 
 def load_probe():
@@ -423,7 +529,9 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
     P = w["n_train_parts"]
     n_train = w["seg"][P] if P else 0
 
-    fwd_bytes = sum(algorithmic_bytes(w, hi, ho) for _, hi, ho in w["proj"])
+    shared_x = w.get("shared_x", {})  # projection -> the projection whose input it reads
+    calls = w.get("calls", [list(range(len(w["proj"])))])  # projections issued together, call by call
+    fwd_bytes = sum(algorithmic_bytes(w, hi, ho, own_x=i not in shared_x) for i, (_, hi, ho) in enumerate(w["proj"]))
     bwd_bytes = sum(backward_bytes(w, hi, ho) for _, hi, ho in w["proj"]) if P else 0
     footprint = sum((T * (hi + ho) + NA * r * (hi + ho)) * 2 for _, hi, ho in w["proj"])
     if P:
@@ -445,7 +553,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
     sets = []
     for _ in range(R):
         projs = []
-        for _, hi, ho in w["proj"]:
+        for pi, (_, hi, ho) in enumerate(w["proj"]):
             A = randn(NA, r, hi, std=hi ** -0.5)
             B = randn(NA, ho, r, std=r ** -0.5)
             if ranks:  # true rank below the padded rank: zero the padding (mixed_lora.py:501-521)
@@ -456,7 +564,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
             if packed:  # every adapter stored at its own rank: what prepare_weight(pack=True) produces
                 Aw = [A[a, :ranks[a % 4]].contiguous() for a in range(NA)]
                 Bw = [B[a, :, :ranks[a % 4]].contiguous() for a in range(NA)]
-            d = dict(x=randn(T, hi), y=randn(T, ho), A=Aw, B=Bw,
+            d = dict(x=projs[shared_x[pi]]["x"] if pi in shared_x else randn(T, hi), y=randn(T, ho), A=Aw, B=Bw,
                      a_tab=torch.tensor([w_.data_ptr() for w_ in Aw], dtype=torch.int64, device=dev),
                      b_tab=torch.tensor([w_.data_ptr() for w_ in Bw], dtype=torch.int64, device=dev))
             if P:
@@ -497,16 +605,17 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         drop_b = [K.DropoutSpec(seg_p[:P].contiguous(), n_train, 1, i, bits[starts[i]:]) for i in range(len(widths))]
 
     def fwd(st, stages=3):
-        pr = st["proj"]
-        K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
-                                  [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
-                                  v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f,
-                                  adapter_rank=rank_f, packed_ranks=packed)
+        for call in calls:
+            pr = [st["proj"][i] for i in call]
+            K.smlm_lora_forward_multi([d["y"] for d in pr], [d["x"] for d in pr], [d["a_tab"] for d in pr],
+                                      [d["b_tab"] for d in pr], st["plan"], r, seg_scale=scale_t, beta=1.0,
+                                      v_out=[d["v"] for d in pr] if P else None, stages=stages, dropout=drop_f,
+                                      adapter_rank=rank_f, packed_ranks=packed)
 
-    def bwd(st):
+    def bwd(st, stages=0):
         # every projection's backward in one set of launches (--bwd-per-projection: a call per projection)
         pr, bplan = st["proj"], st["bplan"]
-        if args.bwd_per_projection:
+        if args.bwd_per_projection and not stages:
             for i, d in enumerate(pr):
                 K.smlm_lora_backward(d["dx"], d["da_tab"], d["db_tab"], d["g"], d["x"], d["v"],
                                      d["ta_tab"], d["tb_tab"], bplan, r, part_scale,
@@ -517,7 +626,7 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                                    [d["g"] for d in pr], [d["x"] for d in pr], [d["v"] for d in pr],
                                    [d["ta_tab"] for d in pr], [d["tb_tab"] for d in pr], bplan, r, part_scale,
                                    dropout=drop_b[0] if drop_b else None, adapter_rank=rank_b,
-                                   packed_ranks=packed)
+                                   packed_ranks=packed, stages=stages)
 
     def step(st, build_plan=True):
         if build_plan:
@@ -589,10 +698,14 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
     torch.cuda.synchronize()
 
     timed([(g_round, args.warmup // R)] + ([(g_warm, 1)] if g_warm else []))
-    t0 = time.perf_counter()
-    ms = timed([(g_round, args.steps // R)] + ([(g_rest, 1)] if g_rest else []))
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms_per_step = ms / args.steps
+    # the timed region of exactly K steps, repeated: the median region is the reported one
+    regions, wall = [], []
+    for _ in range(3 if brief else 9):
+        t0 = time.perf_counter()
+        regions.append(timed([(g_round, args.steps // R)] + ([(g_rest, 1)] if g_rest else [])) / args.steps)
+        wall.append((time.perf_counter() - t0) * 1e3)
+    ms_per_step = float(np.median(regions))
+    wall_ms = float(np.median(wall))
     tokens_per_s = T / (ms_per_step * 1e-3)
     step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
 
@@ -637,7 +750,8 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         timed([(g, 2)])
         shrink_plan_us = timed([(g, 10)]) * 1e3 / (10 * reps * R)
     expand_bytes = sum(T * ho * 2 * 2 + rsum * ho * 2 + T * r * 2 for _, hi, ho in w["proj"])
-    shrink_bytes = sum(T * hi * 2 + rsum * hi * 2 + T * r * 2 for _, hi, ho in w["proj"])
+    shrink_bytes = sum((T * hi * 2 if i not in shared_x else 0) + rsum * hi * 2 + T * r * 2
+                       for i, (_, hi, ho) in enumerate(w["proj"]))
     traffic = {}
     tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
@@ -657,6 +771,36 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
                                  shrink_plan_us, shrink_bytes, "shrink_self_planned_bytes_per_launch"))
     # the forward launch furthest below the HBM peak is the one the roofline entry names
     roofline = min(lines, key=lambda l: l["frac"])
+
+    # ---- the backward's launches alone (training workloads), each stage of all projections: the products
+    # (dV = dY B with its fold launch; v comes from the forward), dX = s dV A, the weight gradients.  Each line
+    # counts what that launch has to move by itself -- dY is read by the first and the third -- while the
+    # roll-up below them counts the step's algorithmic bytes (dY once) against the backward's own time.
+    backward = None
+    if P:
+        train_ids = sorted(set(w["ids"][:P]))
+        rsum_t = sum((ranks[a % 4] if ranks else r) for a in train_ids)
+        n = n_train
+
+        def bwd_stage_us(stages):
+            g = capture(lambda: [bwd(st, stages) for _ in range(reps) for st in sets])
+            timed([(g, 2)])
+            return timed([(g, 10)]) * 1e3 / (10 * reps * R)
+        dv_bytes = sum(n * ho * 2 + rsum_t * ho * 2 + n * r * 2 for _, hi, ho in w["proj"])
+        dx_bytes = sum(n * hi * 2 + rsum_t * hi * 2 + n * r * 2 for _, hi, ho in w["proj"])
+        wg_bytes = sum(n * (hi + ho) * 2 + rsum_t * (hi + ho) * 2 + 2 * n * r * 2 for _, hi, ho in w["proj"])
+        dv_us, dx_us, wg_us, all_us = bwd_stage_us(1), bwd_stage_us(2), bwd_stage_us(4), bwd_stage_us(0)
+        lines += [launch_line("backward: dV = dY B over all projections (shrink launch + fold launch)", dv_us,
+                              dv_bytes, "bwd_dv_bytes_per_launch"),
+                  launch_line("backward: dX = s dV A over all projections (expand launch)", dx_us, dx_bytes,
+                              "bwd_dx_bytes_per_launch"),
+                  launch_line("backward: dA, dB of all projections (weight-gradient launch)", wg_us, wg_bytes,
+                              "bwd_wgrad_bytes_per_launch")]
+        gbps = bwd_bytes / (all_us * 1e-6) / 1e9
+        backward = dict(algorithmic_bytes=bwd_bytes, us=round(all_us, 3), achieved=round(gbps, 1), unit="GB/s",
+                        frac=round(gbps / HBM_PEAK_GBPS, 4), launches_per_step=4,
+                        note="all projections in one set of launches (smlm_lora_bwd_multi_ex), plan reused; "
+                             "algorithmic bytes count dY, x once, dX, A/B and dA/dB of the training adapters, v, dV")
 
     # ---- what plain streaming kernels reach at these launch sizes (loquetier_amd/csrc/stream_probe.hip:
     # a read-modify-write moving the expand launch's bytes, a read moving the shrink launch's), cold over
@@ -747,8 +891,11 @@ def run_workload(args, cfg, torch, K, probe, brief=False):
         "step_hbm_gbps": round(step_gbps, 1), "step_frac_of_8TBps": round(step_gbps / HBM_PEAK_GBPS, 4),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
         "ms_per_step_plan_reused": round(reuse_ms, 5),
+        "timed_regions": {"count": len(regions), "steps_each": args.steps, "ms_per_step_median": round(ms_per_step, 5),
+                          "ms_per_step_min": round(min(regions), 5), "ms_per_step_max": round(max(regions), 5)},
         "roofline": roofline,
         "launches": lines,
+        "backward": backward,
         "streaming_reference": streaming,
         "cpu_baseline": cpu,
     }
@@ -764,7 +911,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="all",
                     help="all (default): the headline workload cfg2 in full, then cfg3, cfg4 and cfg5 in brief "
-                         "under 'configs'; or one of cfg2 | cfg2mod | cfg2one | cfg3 | cfg4 | cfg5 | rmsnorm | model-step")
+                         "under 'configs', plus per-projection / layer-issue / reference-surface / model-step legs; or one "
+                         "of cfg2 | cfg2mod | cfg2one | cfg2layer | cfg2ref | cfg3 | cfg4 | cfg5 | rmsnorm | model-step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-rotate", action="store_true", help="one buffer set (cache-hot numbers)")
     ap.add_argument("--step-only", action="store_true", help="skip the single-kernel and CPU legs")
@@ -805,7 +953,11 @@ def main():
     if args.config == "rmsnorm":
         return rmsnorm_bench(args, torch, K)
     if args.config == "model-step":
-        return model_step_bench(args, torch, K)
+        print(json.dumps(model_step_bench(args, torch, K)), flush=True)
+        return
+    if args.config == "cfg2ref":
+        print(json.dumps(reference_surface_bench(args, torch, K)), flush=True)
+        return
     probe = load_probe()
     if args.config != "all":
         print(json.dumps(run_workload(args, args.config, torch, K, probe)), flush=True)
@@ -813,13 +965,28 @@ def main():
     # the headline: BASELINE.json's configs[1]; the other GPU workloads ride along in brief
     out = run_workload(args, "cfg2", torch, K, probe)
     if not args.step_only:
+        keys = ("value", "unit", "ms_per_step", "ms_per_step_plan_reused", "timed_regions", "dtype",
+                "step_algorithmic_bytes", "step_hbm_gbps", "step_frac_of_8TBps", "roofline", "launches", "backward",
+                "cpu_baseline")
+        quiet = argparse.Namespace(**dict(vars(args), no_cpu_baseline=True))
+        # what a model gets out of the headline batch: one projection per call (a layer call of the reference), the
+        # launches one decoder layer can issue (q/k/v of one input together, o alone), the reference's own call
+        # sequence, and the whole layer path (224 MixedLoraLinear calls a model step)
+        for name, cfg in (("per_projection", "cfg2one"), ("layer_issue", "cfg2layer")):
+            o = run_workload(quiet, cfg, torch, K, probe, brief=True)
+            out[name] = {k: o[k] for k in keys if k != "cpu_baseline"}
+            out[name]["workload"] = o["config"]["workload"]
+        out["reference_surface"] = reference_surface_bench(args, torch, K)
+        out["model_step_decode"] = model_step_bench(args, torch, K, finetune=False)["decode_forward"]
         out["configs"] = {}
         for cfg in ("cfg3", "cfg4", "cfg5"):
             o = run_workload(args, cfg, torch, K, probe, brief=True)
-            out["configs"][cfg] = {k: o[k] for k in ("value", "unit", "ms_per_step", "ms_per_step_plan_reused",
-                                                     "dtype", "step_algorithmic_bytes", "step_hbm_gbps",
-                                                     "step_frac_of_8TBps", "roofline", "launches", "cpu_baseline")}
+            out["configs"][cfg] = {k: o[k] for k in keys}
             out["configs"][cfg]["workload"] = o["config"]["workload"]
+        # cfg5 with the adapters kept zero-padded to rank 64 in memory, as the reference keeps them
+        padded = argparse.Namespace(**dict(vars(args), padded_storage=True, step_only=True))
+        out["configs"]["cfg5"]["ms_per_step_adapters_padded_in_memory"] = run_workload(padded, "cfg5", torch, K, probe,
+                                                                                      brief=True)["ms_per_step"]
     print(json.dumps(out), flush=True)
 
 

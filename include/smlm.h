@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SMLM_ABI_VERSION 3
+#define SMLM_ABI_VERSION 4
 
 #if defined(__GNUC__)
 #define SMLM_API __attribute__((visibility("default")))
@@ -49,6 +49,11 @@ extern "C" {
 /* stages of the fused forward (smlm_lora_fwd_multi) */
 #define SMLM_STAGE_SHRINK 1 /* v = x A^T, left in the workspace                */
 #define SMLM_STAGE_EXPAND 2 /* y = beta*y + scale * v B^T from that workspace  */
+
+/* stages of the backward (smlm_lora_opts.bwd_stages) */
+#define SMLM_BWD_PRODUCTS 1 /* plan (when the call builds it), v when not given, dV = dY B  */
+#define SMLM_BWD_DX 2       /* dX = s dV A (and the transposed s dV, s v the next stage reads) */
+#define SMLM_BWD_WGRAD 4    /* dA_a, dB_a                                        */
 
 #define SMLM_OK 0
 #define SMLM_ERR_ARG (-1)       /* null pointer, negative size, bad enum      */
@@ -285,6 +290,11 @@ typedef struct smlm_dropout {
  *                  smlm_lora_bwd_ex takes the pair (part_indptr, part_adapter) the same way and
  *                  builds its plan inside the dV launch when r <= 64, P <= 512,
  *                  n_rows / 16 + P < 1024, v is given and there is no dropout.
+ *   bwd_stages   : (backward entry points) 0 = the whole backward; else a set of SMLM_BWD_* bits: the
+ *                  stages of one backward may be issued as separate calls with the same arguments,
+ *                  workspace and stream, in the order PRODUCTS, DX, WGRAD (each reads what the stage
+ *                  before left in the workspace) -- to time them one by one, or to put other work of
+ *                  the stream between them.  A plan the call is to build is built by the PRODUCTS stage.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;
@@ -292,6 +302,7 @@ typedef struct smlm_lora_opts {
   int packed_ranks;
   const int32_t* build_seg_indptr;
   const int32_t* build_seg_adapter;
+  int bwd_stages;
 } smlm_lora_opts;
 
 /* smlm_lora_fwd_multi with options. */

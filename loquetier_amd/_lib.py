@@ -17,6 +17,7 @@ SMLM_ERR_DTYPE = -2
 SMLM_ERR_SCRATCH = -7
 SMLM_STATIC_SCRATCH_BYTES = 8 << 20
 SMLM_STAGE_SHRINK, SMLM_STAGE_EXPAND = 1, 2
+SMLM_BWD_PRODUCTS, SMLM_BWD_DX, SMLM_BWD_WGRAD = 1, 2, 4
 
 _vp, _i, _sz, _f = C.c_void_p, C.c_int, C.c_size_t, C.c_float
 _psz = C.POINTER(C.c_size_t)
@@ -32,7 +33,7 @@ class Dropout(C.Structure):
 class LoraOpts(C.Structure):
     """struct smlm_lora_opts of include/smlm.h."""
     _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p), ("packed_ranks", C.c_int),
-                ("build_seg_indptr", C.c_void_p), ("build_seg_adapter", C.c_void_p)]
+                ("build_seg_indptr", C.c_void_p), ("build_seg_adapter", C.c_void_p), ("bwd_stages", C.c_int)]
 
 
 _popts = C.POINTER(LoraOpts)

@@ -949,6 +949,8 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   if ((rc = drop_args(opts ? opts->dropout : nullptr, &drop))) return rc;
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
+  const int stages = (opts && opts->bwd_stages) ? opts->bwd_stages : (SMLM_BWD_PRODUCTS | SMLM_BWD_DX | SMLM_BWD_WGRAD);
+  if (stages < 0 || stages > (SMLM_BWD_PRODUCTS | SMLM_BWD_DX | SMLM_BWD_WGRAD)) return SMLM_ERR_ARG;
   if (n_proj < 1 || n_proj > kMaxProj || NA < 0 || r <= 0 || !h_in || !h_out) return SMLM_ERR_ARG;
   if (r & 7) return SMLM_ERR_ALIGN;
   if (NA == 0 || n_rows == 0 || P == 0) return SMLM_ERR_ARG;
@@ -976,12 +978,14 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   const int32_t* build_s = opts ? opts->build_seg_indptr : nullptr;
   const int32_t* build_k = opts ? opts->build_seg_adapter : nullptr;
   if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
+  if (build_s && !(stages & SMLM_BWD_PRODUCTS)) return SMLM_ERR_ARG;  // the plan is built with the first stage
   PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, P, next_pow2(P)};
   const int mt = bwd_tiles_per_wave(n_rows, r);
   bool even_dv = true;  // (k slices in pairs beyond 256 partitions)
   for (int i = 0; i < n_proj; ++i) even_dv = even_dv && shrink_cfg(n_rows, h_out[i], r, kFwdWaves, true, mt).ksplit % 2 == 0;
   const bool self_planned = build_s && have_v && !drop.seg_p && mt > 1 && r <= 64 &&
                             self_planned_ok(n_rows, P, NA, pv.nt_max, mt) && (P <= kFwdThreads || even_dv);
+  const bool products = (stages & SMLM_BWD_PRODUCTS) != 0;
   if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, P, st))) return rc;
 
   // 1. The backward multiplies by B and A where the forward multiplies by A^T and B^T.  The
@@ -989,7 +993,7 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   // expand kernel's general k loop, which reads [n][k] weights: transposed copies At [h_in, r],
   // Bt [r, h_out] made here.
   const bool in_place = mt > 1 && r <= 64;
-  if (!in_place) {
+  if (!in_place && products) {
     for (int i = 0; i < n_proj; ++i) {
       TransposeArgs ta{};
       ta.set[0] = TransposeSet{a_ptrs[i], reinterpret_cast<uint16_t*>(ws + L.p[i].at),
@@ -1022,7 +1026,7 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
         di.bits_pitch = h_in[i] / 8;
         bits[i] = di.bits;
         const DropBitsArgs ba{pv.hdr, pv.tile_row, pv.tile_rseg, di};
-        if ((rc = launch(drop_bits_kernel, dim3((unsigned)pv.nt_max), dim3(256), st, ba))) return rc;
+        if (products && (rc = launch(drop_bits_kernel, dim3((unsigned)pv.nt_max), dim3(256), st, ba))) return rc;
       }
     }
   }
@@ -1039,7 +1043,7 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   }
 
   // 2. v = round16(x A^T) unless the forward saved it
-  if (!have_v) {
+  if (!have_v && products) {
     DropArgs vdrop = drop;
     vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
     if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
@@ -1054,9 +1058,9 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     btp[i] = in_place ? b_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].bt_ptrs);
     b_ld[i] = in_place ? r : h_out[i];
   }
-  if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, dy, btp, partial, dv16, h_out, r, b_ld,
-                       0.0f, nullptr, mt, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
-                       self_planned ? &build : nullptr, true)))
+  if (products && (rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, dy, btp, partial, dv16, h_out, r, b_ld,
+                                   0.0f, nullptr, mt, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
+                                   self_planned ? &build : nullptr, true)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
@@ -1082,8 +1086,9 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   }
   ea.w_kn = in_place ? 1 : 0;
   ea.drop = drop;  // dX is the gradient with respect to x before its dropout
-  if ((rc = launch_expand(dtype, false, expand_nq(n_rows, widest), mt, P, NA, n_proj, r, st, ea)))
+  if ((stages & SMLM_BWD_DX) && (rc = launch_expand(dtype, false, expand_nq(n_rows, widest), mt, P, NA, n_proj, r, st, ea)))
     return rc;
+  if (!(stages & SMLM_BWD_WGRAD)) return SMLM_OK;
 
   // 5. dA_a, dB_a for every adapter (zeros when it has no rows)
   WgradArgs wa{};

@@ -496,12 +496,15 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
                              part_scale: Optional[torch.Tensor] = None,
                              dropout: Optional[DropoutSpec] = None,
                              adapter_rank: Optional[torch.Tensor] = None,
-                             workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
+                             workspace: Optional[Workspace] = None, packed_ranks: bool = False,
+                             stages: int = 0) -> None:
     """The backward of several projections of one batch (q/k/v/o, gate/up/down) in one set of
     launches; lists of equal length, one entry per projection, each what smlm_lora_backward
     takes.  vs: None, or the saved intermediate of every projection.  The results equal
     per-projection calls bit for bit.  dropout: projection i uses the stream offset + i and
-    the keep bits of the projections lie end to end (as smlm_lora_forward_multi leaves them)."""
+    the keep bits of the projections lie end to end (as smlm_lora_forward_multi leaves them).
+    stages: 0 = everything; else SMLM_BWD_* bits (1 products v / dV, 2 dX, 4 weight gradients): the stages
+    may be issued as separate calls with the same arguments, workspace and stream, in that order."""
     n = len(dxs)
     lists = (da_ptrs, db_ptrs, dys, xs, a_ptrs, b_ptrs) + (() if vs is None else (vs,))
     if not (1 <= n <= 8) or any(len(l) != n for l in lists):
@@ -538,9 +541,15 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
         opts = _opts(plan, dropout, list(widths_in), adapter_rank, NA, packed_ranks)
         if not plan.built:  # a deferred plan: this call builds it (inside its first launch where it can)
+            if stages and not (stages & _lib.SMLM_BWD_PRODUCTS):
+                plan.ensure_built()
+            else:
+                opts = opts or _lib.LoraOpts()
+                opts.build_seg_indptr = plan.segment.data_ptr()
+                opts.build_seg_adapter = plan.seg_key.data_ptr()
+        if stages:
             opts = opts or _lib.LoraOpts()
-            opts.build_seg_indptr = plan.segment.data_ptr()
-            opts.build_seg_adapter = plan.seg_key.data_ptr()
+            opts.bwd_stages = int(stages)
         arr = lambda ts: VP(*[t.data_ptr() for t in ts])
         rc = _lib.load().smlm_lora_bwd_multi_ex(
             n, arr(dxs), arr(da_ptrs), arr(db_ptrs), arr(dys), arr(xs), None if vs is None else arr(vs),
