@@ -1097,7 +1097,21 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   wa.grp_id = pv.grp_id;
   wa.tile_row = pv.tile_row;
   wa.nproj = n_proj;
-  int chunks = 0;
+  // four waves splitting the rows of an adapter pay off when adapters have many rows each (whole backward,
+  // 16 adapters at rank 16 / 64: 1024 rows each 124.7 -> 118.7 / 180.7 -> 175.3 us, 512 rows even, 256 rows
+  // 43.5 -> 44.6 / 62.1 -> 67.3 us, 64 rows 25.7 -> 30.8 / 33.7 -> 46.5 us)
+  const bool split = n_rows / NA >= 512;
+  // one-wave workgroups take several neighbouring chunks in turn when there are chunks enough to keep the
+  // chip busy anyway: about 8192 workgroups are left
+  long all_chunks = 0;
+  for (int i = 0; i < n_proj; ++i) all_chunks += ceil_div(h_in[i], kWgCols) + ceil_div(h_out[i], kWgCols);
+  int walk = 1;
+  if (!split) {
+    const long want = all_chunks * NA * ceil_div(r, 64) / 8192;
+    walk = want < 1 ? 1 : (want > 8 ? 8 : (int)want);
+  }
+  wa.walk = walk;
+  int units = 0;
   for (int i = 0; i < n_proj; ++i) {
     WgradProj& Q = wa.p[i];
     Q.q_a = reinterpret_cast<const uint16_t*>(x[i]);
@@ -1108,10 +1122,11 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     Q.db_ptrs = db_ptrs[i];
     Q.h_in = h_in[i]; Q.h_out = h_out[i];
     Q.chunks_a = ceil_div(h_in[i], kWgCols);
-    Q.chunk0 = chunks;
+    Q.units_a = ceil_div(Q.chunks_a, walk);
+    Q.unit0 = units;
     Q.drop_bits = bits[i];
     Q.drop_pitch = h_in[i] / 8;
-    chunks += Q.chunks_a + ceil_div(h_out[i], kWgCols);
+    units += Q.units_a + ceil_div(ceil_div(h_out[i], kWgCols), walk);
   }
   wa.pitch = L.pitch;
   wa.r = r;
@@ -1121,12 +1136,8 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   wa.packed = packed;
   wa.drop = drop;  // dA against the dropped x
   // ranks above 64 are covered 64 at a time along the grid's z axis
-  dim3 grid(chunks, NA, ceil_div(r, 64));
+  dim3 grid(units, NA, ceil_div(r, 64));
   const int nbj = r > 64 ? 4 : ceil_div(r, 16);
-  // four waves splitting the rows of an adapter pay off when adapters have many rows each (whole backward,
-  // 16 adapters at rank 16 / 64: 1024 rows each 124.7 -> 118.7 / 180.7 -> 175.3 us, 512 rows even, 256 rows
-  // 43.5 -> 44.6 / 62.1 -> 67.3 us, 64 rows 25.7 -> 30.8 / 33.7 -> 46.5 us)
-  const bool split = n_rows / NA >= 512;
   return dtype == SMLM_DTYPE_F16 ? launch_wgrad<SMLM_DTYPE_F16>(nbj, split, grid, st, wa)
                                  : launch_wgrad<SMLM_DTYPE_BF16>(nbj, split, grid, st, wa);
 }

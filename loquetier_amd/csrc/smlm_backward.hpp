@@ -87,8 +87,9 @@ struct WgradProj {
   const uint16_t* pt_b;  // scale*v  by slot, transposed [r, pitch]
   void* const* da_ptrs;  // [NA] -> [r, h_in]
   void* const* db_ptrs;  // [NA] -> [h_out, r]
-  int h_in, h_out, chunks_a;  // chunks_a = ceil(h_in/64): the projection's first chunks_a chunks work on dA
-  int chunk0;                 // first chunk (blockIdx.x) of this projection; its chunks lie end to end
+  int h_in, h_out, chunks_a;  // chunks_a = ceil(h_in/64) 64-column chunks of dA (dB: ceil(h_out/64))
+  int units_a;                // units (walk chunks each) of dA: the projection's first units_a units work on dA
+  int unit0;                  // first unit (blockIdx.x) of this projection; the projections' units lie end to end
   const uint8_t* drop_bits;   // DROP kernels: keep bits of this projection's mask of x, [rows, drop_pitch]
   long drop_pitch;
 };
@@ -100,6 +101,7 @@ struct WgradArgs {
   const int32_t* tile_row;
   WgradProj p[kWgMaxProj];
   int nproj;
+  int walk;                // chunks a one-wave workgroup takes in turn (NW = 1 kernels; else 1)
   long pitch;
   int r;
   int n_parts;             // partitions the plan was laid out for (>= 1): its group tables hold n_parts + 1 entries
@@ -122,13 +124,17 @@ __device__ __forceinline__ int wg_lds_row(int s) {
   return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1);
 }
 
-// grid: (sum over the projections of ceil(h_in/64) + ceil(h_out/64), NA, ceil(r/64)), block 64*NW.  A workgroup owns 64
-// columns (and up to 64 ranks) of one adapter's dA or dB and walks all of that adapter's tiles, 64
+// grid: (sum over the projections of their dA and dB units, NA, ceil(r/64)), block 64*NW; a unit is
+// `walk` neighbouring 64-column chunks of one projection's dA or dB.  A workgroup owns the unit's columns (and
+// up to 64 ranks) of one adapter's gradient and walks all of that adapter's tiles once per chunk, 64
 // gathered rows (four tiles, two MFMA k steps) per wave and loop step.  With
-// NW = 4 (adapters with many rows each) the waves take steps round-robin and
+// NW = 4 (adapters with many rows each; walk = 1) the waves take steps round-robin and
 // their accumulators are summed through LDS in wave order; with NW = 1 (many
 // adapters with few rows each) a lone wave does it all and more workgroups fit
-// on a CU.  The token dimension is the contraction, so a wave stages its
+// on a CU -- and it takes several chunks in turn, the first rows of the next chunk on their way while
+// the last of this one are multiplied: an adapter of 32 rows is 4 KB of input per chunk, and a
+// workgroup per chunk is all look-ups (64 adapters, 1152 chunks: 202 us for 590 MB).  The token
+// dimension is the contraction, so a wave stages its
 // [token][column] block of x / dY in its own part of LDS and reads it back
 // token-innermost with the transposing LDS read; no workgroup barrier is needed
 // inside the loop, and the rows of the next step are already on their way from
@@ -139,7 +145,8 @@ __device__ __forceinline__ int wg_lds_row(int s) {
 // rows are staged; every row of the workgroup belongs to one adapter, whose probability is read
 // once from the group's first segment.
 template <int DT, int NBJ, int NW, bool IS_A, bool DROP = false>
-__device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& P, int chunk, char* smem) {
+__device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& P, int chunk_first, int n_chunks,
+                                           char* smem) {
   constexpr int kWgWaves = NW;
   constexpr int kStageElems = kWgSlots * kWgPitch;
   constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
@@ -147,7 +154,6 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
   const int ad = blockIdx.y;
   const int j0 = 64 * blockIdx.z;  // first rank of this workgroup (ranks above 64: 64 per z)
   constexpr bool is_a = IS_A;
-  const int n0 = (is_a ? chunk : chunk - P.chunks_a) * kWgCols;
   const int h = is_a ? P.h_in : P.h_out;
   const uint16_t* Q = is_a ? P.q_a : P.q_b;
   const uint16_t* PT = is_a ? P.pt_a : P.pt_b;
@@ -191,18 +197,11 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
   const int n_steps = (t_end - t_beg + kStepTiles - 1) / kStepTiles;
 
   const uint16_t* zeros = reinterpret_cast<const uint16_t*>(a.hdr + kHdrZeros);
-  f32x4 acc[NBJ][4];
-#pragma unroll
-  for (int jb = 0; jb < NBJ; ++jb)
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) acc[jb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
   uint16_t* st = reinterpret_cast<uint16_t*>(smem) + wave * kStageElems;
   // staging: load u of a lane brings 8 columns (lane & 7) of the slot whose LDS row is
   // 8u + rlow; the two rows a 16-lane group writes together are 4 apart (32 banks)
   const int q8 = lane >> 3, lcol = (lane & 7) * 8;
   const int rlow = (q8 >> 1) + 4 * (q8 & 1);
-  const bool col_ok = n0 + lcol < h;
   // transposed reads: lane i of a 16-lane group names row (8g + 4h + i/4) of the k step,
   // columns 16nb + 4(i%4) .. +3
   const int tr_row = wg_lds_row(8 * g + (c >> 2));  // + 4h -> LDS row + 8h; + 32 per k step
@@ -218,7 +217,8 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
     }
   };
   const uint8_t* zero_bytes = reinterpret_cast<const uint8_t*>(zeros);
-  auto load_data = [&](const int32_t (&row)[8], u32x4 (&val)[8], uint32_t (&keep)[DROP ? 8 : 1]) {
+  auto load_data = [&](const int32_t (&row)[8], int n0, u32x4 (&val)[8], uint32_t (&keep)[DROP ? 8 : 1]) {
+    const bool col_ok = n0 + lcol < h;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const bool ok = row[u] >= 0 && col_ok;
@@ -251,96 +251,17 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
     drop_on = dr.on;
   }
 
-  int32_t row_next[8];
+  // the first step of the first chunk
+  int32_t row_first[8], row_next[8];  // the rows of the wave's first step (every chunk starts with them), of the step ahead
   uint32_t keep[DROP ? 8 : 1];  // bit 8 set: the row is not dropped
   u32x4 val[8], pf[NBJ][2];
-  load_rows(wave, row_next);
-  load_data(row_next, val, keep);
+  load_rows(wave, row_first);
+  load_data(row_first, chunk_first * kWgCols, val, keep);
   load_p(wave, pf);
   load_rows(wave + kWgWaves, row_next);
 
-  for (int step = wave; step < n_steps; step += kWgWaves) {
-    // the next step's rows and token-side operand start their way from memory now
-    u32x4 val_next[8], pf_next[NBJ][2];
-    uint32_t keep_next[DROP ? 8 : 1];
-    load_data(row_next, val_next, keep_next);
-    load_p(step + kWgWaves, pf_next);
-    load_rows(step + 2 * kWgWaves, row_next);
-
-    if (DROP && drop_on) {  // uniform over the workgroup
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        dr.on = (keep[u] & 0x100u) == 0;
-        val[u] = drop8_bits<DT>(val[u], dr, keep[u]);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4*>(st + (8 * u + rlow) * kWgPitch + lcol) = val[u];
-    // the wave's own LDS accesses are served in order; only the compiler must not move
-    // the reads above the writes
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // column-side operands: Q[slots 32ks + 8g .. +7][n0 + 16nb + c], token index innermost;
-    // all sixteen reads are issued before the first multiply waits for them
-    u32x4 qf[2][4];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) {
-        const uint16_t* base = st + (32 * ks + tr_row) * kWgPitch + 16 * nb + tr_col;
-        const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 8 * kWgPitch);
-        qf[ks][nb] = u32x4{q0[0], q0[1], q1[0], q1[1]};
-      }
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-        for (int jb = 0; jb < NBJ; ++jb) {
-          // dA: rows = columns of x, cols = rank -> lane holds 4 consecutive x columns of rank c
-          // dB: rows = rank, cols = columns of dY -> lane holds 4 consecutive ranks of column c
-          acc[jb][nb] = is_a ? Num<DT>::mfma(qf[ks][nb], pf[jb][ks], acc[jb][nb])
-                             : Num<DT>::mfma(pf[jb][ks], qf[ks][nb], acc[jb][nb]);
-        }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int u = 0; u < 8; ++u) val[u] = val_next[u];
-    if (DROP) {
-#pragma unroll
-      for (int u = 0; u < 8; ++u) keep[u] = keep_next[u];
-    }
-#pragma unroll
-    for (int jb = 0; jb < NBJ; ++jb) pf[jb][0] = pf_next[jb][0], pf[jb][1] = pf_next[jb][1];
-  }
-
-  // cross-wave sum in wave order, one rank block at a time; wave 0 ends up with the totals
   f32x4(*red)[4][kWaveSize] = reinterpret_cast<f32x4(*)[4][kWaveSize]>(smem);
-  if (NW > 1) {
-    __syncthreads();  // every wave is done with its staging area, which red overlays
-    for (int jb = 0; jb < NBJ; ++jb) {
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) red[wave][nb][lane] = acc[jb][nb];
-      __syncthreads();
-      if (wave == 0) {
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-          f32x4 part[kWgWaves];
-#pragma unroll
-          for (int w = 0; w < kWgWaves; ++w) part[w] = red[w][nb][lane];
-          f32x4 sum = part[0];
-#pragma unroll
-          for (int w = 1; w < kWgWaves; ++w) sum += part[w];
-          acc[jb][nb] = sum;
-        }
-      }
-      __syncthreads();
-    }
-    if (wave != 0) return;  // no barrier follows
-  }
-
-  // Store.  The MFMA leaves 32-byte pieces per output row; the totals go through LDS once
+  // Store staging.  The MFMA leaves 32-byte pieces per output row; the totals go through LDS once
   // more (an area of their own behind `red`) so that every store instruction writes full
   // rows: lane -> output row lane/8 (+8), eight elements at (lane%8)*8.
   constexpr int kSPitch = 64 + 4;  // floats; conflict-free for the writes below and the reads
@@ -357,60 +278,161 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
     return u32x4{pack2<DT>(lo4[0], lo4[1]), pack2<DT>(lo4[2], lo4[3]), pack2<DT>(hi4[0], hi4[1]),
                  pack2<DT>(hi4[2], hi4[3])};
   };
-  if (is_a) {
-    // dA [r, h]: per rank block, 16 rank rows x 64 columns; lane (c, g) holds rank row c,
-    // columns 16nb + 4g .. +3
+
+#pragma unroll 1
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int n0 = (chunk_first + ci) * kWgCols;
+    const bool more_chunks = ci + 1 < n_chunks;  // uniform over the workgroup
+    f32x4 acc[NBJ][4];
 #pragma unroll
-    for (int jb = 0; jb < NBJ; ++jb) {
+    for (int jb = 0; jb < NBJ; ++jb)
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * nb + 4 * g]) = acc[jb][nb];
+      for (int nb = 0; nb < 4; ++nb) acc[jb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int step = wave; step < n_steps; step += kWgWaves) {
+      // the next step's rows and token-side operand start their way from memory now; after this chunk's
+      // last step that is the first step of the next chunk (the rows are the same, the columns move on)
+      const bool last = step + kWgWaves >= n_steps;
+      const bool wrap = last && more_chunks;
+      u32x4 val_next[8];
+      uint32_t keep_next[DROP ? 8 : 1];
+      if (wrap) load_data(row_first, n0 + kWgCols, val_next, keep_next);
+      else load_data(row_next, n0, val_next, keep_next);
+      load_rows(wrap ? wave + kWgWaves : step + 2 * kWgWaves, row_next);
+
+      if (DROP && drop_on) {  // uniform over the workgroup
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          dr.on = (keep[u] & 0x100u) == 0;
+          val[u] = drop8_bits<DT>(val[u], dr, keep[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4*>(st + (8 * u + rlow) * kWgPitch + lcol) = val[u];
+      // the wave's own LDS accesses are served in order; only the compiler must not move
+      // the reads above the writes
       wave_sync();
-      u32x4 o[2];
+      // column-side operands: Q[slots 32ks + 8g .. +7][n0 + 16nb + c], token index innermost;
+      // all sixteen reads are issued before the first multiply waits for them
+      u32x4 qf[2][4];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) o[i] = read_and_pack(orow + 8 * i);
-      wave_sync();
+      for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int j = j0 + 16 * jb + orow + 8 * i, n = n0 + ocol;
-        if (j < (a.packed ? rlim : a.r) && n < h) stg16_nt(out + (long)j * h + n, o[i]);
+        for (int nb = 0; nb < 4; ++nb) {
+          const uint16_t* base = st + (32 * ks + tr_row) * kWgPitch + 16 * nb + tr_col;
+          const u32x2 q0 = lds_read_tr16(base), q1 = lds_read_tr16(base + 8 * kWgPitch);
+          qf[ks][nb] = u32x4{q0[0], q0[1], q1[0], q1[1]};
+        }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+          for (int jb = 0; jb < NBJ; ++jb) {
+            // dA: rows = columns of x, cols = rank -> lane holds 4 consecutive x columns of rank c
+            // dB: rows = rank, cols = columns of dY -> lane holds 4 consecutive ranks of column c
+            acc[jb][nb] = is_a ? Num<DT>::mfma(qf[ks][nb], pf[jb][ks], acc[jb][nb])
+                               : Num<DT>::mfma(pf[jb][ks], qf[ks][nb], acc[jb][nb]);
+          }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      // the token-side operand of the next step, into the registers the multiplies above are done with (it
+      // arrives behind the rows requested before it, which the next step waits for first); a wave whose
+      // only step this is keeps what it has, chunk after chunk
+      if (!last) load_p(step + kWgWaves, pf);
+      else if (wrap && wave + kWgWaves < n_steps) load_p(wave, pf);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) val[u] = val_next[u];
+      if (DROP) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) keep[u] = keep_next[u];
       }
     }
-  } else {
-    // dB [h, r]: per 16 columns of dY (output rows), all ranks; lane (c, g) holds output row
-    // 16nb + c, ranks 16jb + 4g .. +3
+    // cross-wave sum in wave order, one rank block at a time; wave 0 ends up with the totals
+    if (NW > 1) {
+      __syncthreads();  // every wave is done with its staging area, which red overlays
+      for (int jb = 0; jb < NBJ; ++jb) {
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+        for (int nb = 0; nb < 4; ++nb) red[wave][nb][lane] = acc[jb][nb];
+        __syncthreads();
+        if (wave == 0) {
 #pragma unroll
-      for (int jb = 0; jb < NBJ; ++jb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * jb + 4 * g]) = acc[jb][nb];
-      wave_sync();
-      u32x4 o[2];
+          for (int nb = 0; nb < 4; ++nb) {
+            f32x4 part[kWgWaves];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) o[i] = read_and_pack(orow + 8 * i);
-      wave_sync();
+            for (int w = 0; w < kWgWaves; ++w) part[w] = red[w][nb][lane];
+            f32x4 sum = part[0];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int n = n0 + 16 * nb + orow + 8 * i;
-        const int ldb = a.packed ? rlim : a.r;  // columns of dB as it is stored
-        if (j0 + ocol < ldb && n < h) stg16_nt(out + (long)n * ldb + j0 + ocol, o[i]);
+            for (int w = 1; w < kWgWaves; ++w) sum += part[w];
+            acc[jb][nb] = sum;
+          }
+        }
+        __syncthreads();
+      }
+      if (wave != 0) return;  // no barrier follows (several waves never walk more than one chunk)
+    }
+
+    if (is_a) {
+      // dA [r, h]: per rank block, 16 rank rows x 64 columns; lane (c, g) holds rank row c,
+      // columns 16nb + 4g .. +3
+#pragma unroll
+      for (int jb = 0; jb < NBJ; ++jb) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * nb + 4 * g]) = acc[jb][nb];
+        wave_sync();
+        u32x4 o[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) o[i] = read_and_pack(orow + 8 * i);
+        wave_sync();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int j = j0 + 16 * jb + orow + 8 * i, n = n0 + ocol;
+          if (j < (a.packed ? rlim : a.r) && n < h) stg16_nt(out + (long)j * h + n, o[i]);
+        }
+      }
+    } else {
+      // dB [h, r]: per 16 columns of dY (output rows), all ranks; lane (c, g) holds output row
+      // 16nb + c, ranks 16jb + 4g .. +3
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+#pragma unroll
+        for (int jb = 0; jb < NBJ; ++jb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * jb + 4 * g]) = acc[jb][nb];
+        wave_sync();
+        u32x4 o[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) o[i] = read_and_pack(orow + 8 * i);
+        wave_sync();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int n = n0 + 16 * nb + orow + 8 * i;
+          const int ldb = a.packed ? rlim : a.r;  // columns of dB as it is stored
+          if (j0 + ocol < ldb && n < h) stg16_nt(out + (long)n * ldb + j0 + ocol, o[i]);
+        }
       }
     }
   }
 }
 
 template <int DT, int NBJ, int NW, bool DROP = false>
-__global__ __launch_bounds__(NW * kWaveSize) void wgrad_kernel(WgradArgs a) {
+// (two waves a SIMD at every rank: the one-wave kernels hide their latencies through occupancy)
+__global__ __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(2))) void wgrad_kernel(WgradArgs a) {
   constexpr int kStageBytes = NW * kWgSlots * kWgPitch * 2;
   constexpr int kTailBytes = (NW > 1 ? NW * 4 * kWaveSize * 16 : 0) + 16 * (64 + 4) * 4;  // red + store staging
   __shared__ __attribute__((aligned(16))) char smem[kStageBytes > kTailBytes ? kStageBytes : kTailBytes];
   int pj = 0;
 #pragma unroll
-  for (int i = 1; i < kWgMaxProj; ++i) pj += (i < a.nproj && (int)blockIdx.x >= a.p[i].chunk0) ? 1 : 0;
+  for (int i = 1; i < kWgMaxProj; ++i) pj += (i < a.nproj && (int)blockIdx.x >= a.p[i].unit0) ? 1 : 0;
   const WgradProj& P = a.p[pj];
-  const int chunk = (int)blockIdx.x - P.chunk0;
-  if (chunk < P.chunks_a)  // uniform over the workgroup
-    wgrad_body<DT, NBJ, NW, true, DROP>(a, P, chunk, smem);
-  else
-    wgrad_body<DT, NBJ, NW, false>(a, P, chunk, smem);
+  const int unit = (int)blockIdx.x - P.unit0;
+  const int walk = NW > 1 ? 1 : a.walk;
+  if (unit < P.units_a) {  // uniform over the workgroup
+    const int first = unit * walk, left = P.chunks_a - first;
+    wgrad_body<DT, NBJ, NW, true, DROP>(a, P, first, left < walk ? left : walk, smem);
+  } else {
+    const int chunks_b = (P.h_out + kWgCols - 1) / kWgCols;
+    const int first = (unit - P.units_a) * walk, left = chunks_b - first;
+    wgrad_body<DT, NBJ, NW, false>(a, P, first, left < walk ? left : walk, smem);
+  }
 }
 
 }  // namespace smlm
