@@ -93,7 +93,10 @@ SMLM_API int smlm_tmp_size(int num_problems, size_t* bytes);
  * plan makes them read w_ptrs[i] for segment i (one entry per segment).
  * Segments that share a key must share their weights.  A negative SMLM_KEY_I32 key marks a
  * segment that no adapter serves (a request without LoRA in a mixed batch): the forward entry
- * points leave its rows of y alone (its rows of v are undefined).
+ * points leave its rows of y alone (its rows of v are undefined).  A key at or above the
+ * n_weights the GEMM entry points are told (when they are told one: n_weights > 0) is treated
+ * the same way -- the tables are never read past their end; the backward leaves the rows of such
+ * a partition's dx as they were and sums nothing for it.
  */
 SMLM_API int smlm_plan_size(int T, int S, size_t* bytes);
 SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr,

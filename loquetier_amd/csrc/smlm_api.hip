@@ -170,8 +170,10 @@ int expand_nq(int T, int d_out) {
   return d_out >= 512 ? 4 : 2;
 }
 
-TileArgs tile_args(const PlanView& pv) {
-  return TileArgs{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
+TileArgs tile_args(const PlanView& pv, int n_weights) {
+  TileArgs t{pv.hdr, pv.tile_row, pv.tile_rseg, pv.tile_wid, pv.blk};
+  t.n_weights = n_weights;  // 0: unknown
+  return t;
 }
 
 // grid of a launch: (chunk row, tile unit, projection), or (chunk row over all projections,
@@ -449,7 +451,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   ShrinkArgs a{};
   if (drop) a.drop = *drop;
   a.w_kn = w_kn ? 1 : 0;
-  a.plan = tile_args(pv);
+  a.plan = tile_args(pv, groups);
   a.plan.w_rank = w_rank;  // the output columns are the rank
   a.plan.packed = packed;
   a.seg_scale = seg_scale;
@@ -664,7 +666,7 @@ SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs
 
   if (d_in < d_out) {  // the reference's "expand" branch (smlm_forward_cutlass.cuh:82)
     ExpandArgs a{};
-    a.plan = tile_args(pv);
+    a.plan = tile_args(pv, n_weights);
     a.seg_scale = seg_scale;
     a.beta = beta;
     a.T = T; a.nt_max = pv.nt_max;
@@ -859,7 +861,7 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   if (!(stages & SMLM_STAGE_EXPAND)) return SMLM_OK;
 
   ExpandArgs ea{};
-  ea.plan = tile_args(pv);
+  ea.plan = tile_args(pv, n_weights);
   ea.plan.w_rank = w_rank;
   ea.plan.packed = packed;
   ea.seg_scale = seg_scale;
@@ -1065,7 +1067,7 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
   ExpandArgs ea{};
-  ea.plan = tile_args(pv);
+  ea.plan = tile_args(pv, NA);
   ea.plan.w_rank = w_rank;
   ea.seg_scale = part_scale;
   ea.beta = 0.0f;

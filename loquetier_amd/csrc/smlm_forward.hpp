@@ -40,7 +40,15 @@ struct TileArgs {
   const int32_t* w_rank;     // optional, indexed like the weight tables: true rank of each adapter
   int packed;                // with w_rank: the weights are STORED at their true rank (rounded up to 8),
                              //   A_a [r_a, h_in], B_a [h_out, r_a], instead of zero-padded to the launch's rank
+  int n_weights;             // entries of the caller's weight tables (0: unknown): a tile whose index is not
+                             //   below it is left alone, like a tile of a negative adapter id
 };
+
+// whether tile index `wid` of a plan names an entry of the caller's weight tables (negative: a segment no
+// adapter serves; at or past the table length: an id the caller's tables do not hold -- never dereferenced)
+__device__ __forceinline__ bool wid_ok(const TileArgs& p, int wid) {
+  return wid >= 0 && (p.n_weights <= 0 || wid < p.n_weights);
+}
 
 // Adapters of different ranks live zero-padded to one rank (the reference pads every adapter
 // of a layer to the layer's maximum, src/loquetier_src/models/mixed_lora.py:501-521).  With the
@@ -148,13 +156,13 @@ __device__ __forceinline__ void pick_tiles(const TileArgs& p, int tb, int* t0, i
   if (MT == 1) {
     *t0 = tb;
     *wid = uload(p.tile_wid, tb);
-    *cnt = *wid < 0 ? 0 : 1;
+    *cnt = wid_ok(p, *wid) ? 1 : 0;
   } else {
     const int packed = uload(p.blk, tb);
     *t0 = packed >> 3;
     *cnt = packed & 7;
     *wid = *cnt ? uload(p.tile_wid, *t0) : -1;
-    if (*wid < 0) *cnt = 0;  // a negative adapter id: rows that no adapter serves
+    if (!wid_ok(p, *wid)) *cnt = 0;  // a negative adapter id (rows that no adapter serves) or one past the tables
   }
 }
 
@@ -226,7 +234,7 @@ __global__ __launch_bounds__(NW * kWaveSize) void shrink_kernel(ShrinkArgs a) {
     const int kz = yy % P.ksplit, zb = yy / P.ksplit;
     if (zb >= P.zblocks) continue;  // a chunk row added to make the count even (uniform over the workgroup)
     const int wid = uload(a.plan.tile_wid, tile);
-    if (wid < 0) continue;  // past the last tile (direct mode); uniform over the workgroup
+    if (!wid_ok(a.plan, wid)) continue;  // past the last tile (direct mode), or no such adapter; uniform over the workgroup
     const int n0 = zb * 64;
     const int slot = tile * kTileRows + c;
     const int row = a.plan.tile_row[slot];
@@ -482,7 +490,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
     const int pj = V / units, tile = V - pj * units;
     const ReduceProj P = a.p[pj];
     if (P.ksplit <= 1) continue;
-    if (uload(a.plan.tile_wid, tile) < 0) continue;  // past the last tile (direct mode)
+    if (!wid_ok(a.plan, uload(a.plan.tile_wid, tile))) continue;  // past the last tile (direct mode), or no such adapter
     const int row = a.plan.tile_row[tile * kTileRows + c];
     if (row < 0) continue;
     const float scale = a.seg_scale ? a.seg_scale[a.plan.tile_rseg[tile * kTileRows + c]] : 1.0f;
@@ -701,7 +709,7 @@ __global__ __launch_bounds__(kFwdThreads) void expand_wave_kernel(ExpandArgs a) 
     const int ncol0 = (yy * kFwdWaves + wave) * 32 * NQ;
     if (ncol0 >= P.d_out) continue;
     const int wid = uload(a.plan.tile_wid, tile);
-    if (wid < 0) continue;  // past the last tile (direct mode)
+    if (!wid_ok(a.plan, wid)) continue;  // past the last tile (direct mode), or no such adapter
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
     const int ldw = ROWMAJOR ? P.ldw : rank_ld(a.plan, P.ldw, klim);
@@ -818,7 +826,7 @@ void expand_block_kernel(ExpandArgs a) {
     const int t0 = packed >> 3, cnt = packed & 7;
     if (cnt == 0) continue;  // past the last block (direct mode); uniform over the workgroup
     const int wid = uload(a.plan.tile_wid, t0);
-    if (wid < 0) continue;  // a negative adapter id: rows that no adapter serves
+    if (!wid_ok(a.plan, wid)) continue;  // a negative adapter id (rows that no adapter serves) or one past the tables
     const uint16_t* W = uload_ptr(P.w_ptrs, wid);
     const int klim = rank_limit(a.plan, wid, P.d_in);  // k at or past it: zero padding of v and the weights
     const int ldw = WKN ? P.ldw : rank_ld(a.plan, P.ldw, klim);  // [k][n] weights (A) have whole rows per rank

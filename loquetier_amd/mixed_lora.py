@@ -43,6 +43,7 @@ class MixedLoraContext:
         self._step: dict = {}          # per-step memo, dropped by update()
         self._workspaces: dict = {}    # device -> kernel.Workspace, kept across steps
         self._dropout_calls = 0        # host-side counter: every dropout call gets its own mask stream
+        self._dropout_salt: Optional[int] = None  # drawn from torch's CPU generator at the first dropout call
 
     def update(self, blen: Optional[BatchLenInfo] = None, lora_ids: Optional[List[int]] = None,
                lora_len: Optional[torch.Tensor] = None, segment: Optional[torch.Tensor] = None,
@@ -102,10 +103,38 @@ class MixedLoraContext:
         return ws
 
     def next_dropout_offset(self) -> int:
-        """Offset of the next dropout mask stream: a host-side counter, so drawing it waits for nothing
-        (eight projections' worth of offsets apart)."""
+        """Offset of the next dropout mask stream: a per-context salt plus a host-side counter (eight
+        projections' worth of offsets apart), so drawing it waits for nothing on the device.  The salt
+        is drawn ONCE, at the context's first dropout call, from torch's CPU generator: two contexts of
+        one process get different masks, and `torch.manual_seed(s)` followed by the same sequence of
+        calls on a fresh context repeats a run.  A run that is resumed, or re-seeded without a fresh
+        context, continues the sequence where `dropout_state()` says; hand that to
+        `set_dropout_state` to repeat from there."""
+        if self._dropout_salt is None:
+            self._dropout_salt = int(torch.randint(0, 1 << 40, (1,), dtype=torch.int64).item()) << 20
         self._dropout_calls += 1
-        return self._dropout_calls * 8
+        return self._dropout_salt + self._dropout_calls * 8
+
+    def dropout_state(self):
+        """(salt, calls made): what a trainer checkpoints beside torch's seed to repeat the masks."""
+        return self._dropout_salt, self._dropout_calls
+
+    def set_dropout_state(self, state) -> None:
+        self._dropout_salt, self._dropout_calls = (None if state[0] is None else int(state[0])), int(state[1])
+
+    def check_adapter_ids(self, n_adapters: int) -> None:
+        """Adapter ids handed over as a host list must index the layer's adapters (negative: a segment no
+        adapter serves).  Ids that only exist on the device cannot be looked at without waiting for it: the
+        kernels skip segments whose id is not below the table length.  Checked once per step and table length."""
+        if isinstance(self._lora_ids, torch.Tensor) or self._lora_ids is None:
+            return
+
+        def check():
+            top = max((int(i) for i in self._lora_ids), default=-1)
+            if top >= n_adapters:
+                raise IndexError(f"adapter id {top} in lora_ids, but the layer holds {n_adapters} adapters")
+            return True
+        self.memo(("ids_ok", n_adapters), check)
 
     def seg_adapter(self, device: torch.device) -> torch.Tensor:
         """Adapter id of every segment as a device tensor.  `lora_ids` may already be one (int32,
@@ -344,6 +373,7 @@ class ProjectionGroup:
             ra, rb = l.adapter_rank, first.adapter_rank
             if (ra is None) != (rb is None) or (ra is not None and not torch.equal(ra, rb)):
                 raise ValueError("the layers of a group must hold adapters of the same true ranks")
+        self.suspended = False  # set while the members' adapter sets disagree (one of them was changed alone)
         for i, l in enumerate(self.layers):
             l._group = (self, i)
 
@@ -373,14 +403,28 @@ class ProjectionGroup:
             self._expand(ys, scale, state["plan"])
             waiting = rest
 
+    @staticmethod
+    def input_key(src: torch.Tensor):
+        """What identifies the input of a pass: the tensor the caller handed to the layer (before any
+        cast or copy the layer makes of it), its layout and -- where torch keeps one -- its version
+        counter.  Inference tensors (torch.inference_mode) have no version counter; they cannot be
+        modified in place outside inference mode either, so address and layout are all there is."""
+        try:
+            version = None if src.is_inference() else src._version
+        except RuntimeError:
+            version = None
+        return (src.data_ptr(), version, tuple(src.shape), tuple(src.stride()), src.dtype)
+
     def expand_member(self, i: int, result: torch.Tensor, x: torch.Tensor, seg_scale, plan,
-                      may_defer: bool = False) -> None:
+                      may_defer: bool = False, src: Optional[torch.Tensor] = None) -> None:
         """result += scale * v_i B^T for member i, shrinking x for the whole group first when this is
         the first member to see x.  may_defer: the caller hands `result` itself on to its own caller,
-        so a deferred group may add to it later."""
+        so a deferred group may add to it later.  src: the tensor the layer was called with, of which
+        x is the contiguous copy in the layer's dtype (None: x itself); the pass is keyed on src, so
+        members that are handed one strided or differently typed tensor still share one shrink."""
         first, n = self.layers[0], len(self.layers)
         ctx = first.root_context
-        key = (x.data_ptr(), x._version, tuple(x.shape), x.dtype)
+        key = self.input_key(x if src is None else src)
         state = ctx._step.get("open_group")
         if state is None or state["group"] is not self or state["key"] != key or i not in state["pending"]:
             if state is not None:
@@ -390,9 +434,9 @@ class ProjectionGroup:
                                            adapter_rank=first.adapter_rank,
                                            workspace=ctx.group_workspace(first.device),
                                            packed_ranks=first.packed, dims=self.dims())
-            # (x is kept so that its address cannot be handed to another tensor while the pass is open)
+            # (the tensors are kept so that their addresses cannot be handed to others while the pass is open)
             state = ctx._step["open_group"] = {"group": self, "key": key, "pending": set(range(n)), "x": x,
-                                               "plan": plan, "waiting": []}
+                                               "src": src, "plan": plan, "waiting": []}
         state["pending"].discard(i)
         if self.deferred and may_defer:
             state["waiting"].append((i, result, seg_scale))
@@ -425,28 +469,48 @@ class MixedLoraLinear(nn.Module):
     def _ptrs(self, tensors) -> torch.Tensor:
         return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, device=self.device)
 
+    def _true_ranks(self, adapters: List[NamedLoraLayer], rank: int):
+        """(packed, true rank of every adapter); raises when the set cannot be served.  Touches nothing."""
+        # adapters stored at their own rank (prepare_weight(pack=True)): every one must be, consistently
+        packed = any(a.wa.size(0) < rank or a.wb.size(1) < rank for a in adapters)
+        ranks = []
+        for a in adapters:
+            stored = a.wa.size(0)
+            q = min(int(a.true_rank), rank) if a.true_rank is not None else min(stored, rank)
+            if packed and not (stored == a.wb.size(1) == min(rank, (q + 7) // 8 * 8)):
+                raise RuntimeError(f"adapter {a.adapter_name}: packed storage needs A [r8, h_in] and B [h_out, r8] "
+                                   f"with r8 = true rank rounded up to 8; got {tuple(a.wa.shape)}, {tuple(a.wb.shape)}")
+            ranks.append(q)
+        if packed and not self.fused:
+            raise RuntimeError("adapters stored at their true rank need the fused path")
+        return packed, ranks
+
     def update_adapters(self, adapters: List[NamedLoraLayer], rank: int):
+        # everything that can refuse the set comes first: a refused set leaves the layer as it was
+        packed, ranks = self._true_ranks(adapters, rank)
+        adapter_rank = (torch.tensor(ranks, dtype=torch.int32, device=self.device)
+                        if packed or any(q < rank for q in ranks) else None)
+        if self._group is not None:  # the members of a projection group hold adapters of the same true ranks
+            for other in self._group[0].layers:
+                if other is self:
+                    continue
+                ra = other.adapter_rank
+                if other.packed != packed or (ra is None) != (adapter_rank is None) or (
+                        ra is not None and not torch.equal(ra, adapter_rank)):
+                    # the siblings may be about to get the same change: the group stops sharing until they agree
+                    self._group[0].suspended = True
+                    break
+            else:
+                self._group[0].suspended = False
         self.adapters = adapters
         self.rank = rank
+        self.packed = packed
+        self.adapter_rank = adapter_rank
         self.wa_ptrs = self._ptrs([a.wa for a in adapters])
         self.wb_ptrs = self._ptrs([a.wb for a in adapters])
         if not self.is_scaled:
             self.scaling = torch.tensor([a.scaling for a in adapters], dtype=self.dtype,
                                         device=self.device)
-        # adapters stored at their own rank (prepare_weight(pack=True)): every one must be, consistently
-        self.packed = any(a.wa.size(0) < rank or a.wb.size(1) < rank for a in adapters)
-        ranks = []
-        for a in adapters:
-            stored = a.wa.size(0)
-            q = min(int(a.true_rank), rank) if a.true_rank is not None else min(stored, rank)
-            if self.packed and not (stored == a.wb.size(1) == min(rank, (q + 7) // 8 * 8)):
-                raise RuntimeError(f"adapter {a.adapter_name}: packed storage needs A [r8, h_in] and B [h_out, r8] "
-                                   f"with r8 = true rank rounded up to 8; got {tuple(a.wa.shape)}, {tuple(a.wb.shape)}")
-            ranks.append(q)
-        if self.packed and not self.fused:
-            raise RuntimeError("adapters stored at their true rank need the fused path")
-        self.adapter_rank = (torch.tensor(ranks, dtype=torch.int32, device=self.device)
-                             if self.packed or any(q < rank for q in ranks) else None)
         self._train_rank_key, self._train_rank = None, None
         self._scaling_f32 = None if self.is_scaled else self.scaling.float()
         self._scaling_key = None if self.is_scaled else tuple(float(a.scaling) for a in adapters)
@@ -499,12 +563,15 @@ class MixedLoraLinear(nn.Module):
         return self.adapter_rank, self._train_rank
 
     def add_adapter(self, adapter: NamedLoraLayer):
-        """New adapter must have the rank of the existing ones."""
+        """New adapter must have the rank of the existing ones.  A set that the layer cannot serve raises
+        and leaves the layer and its list as they were."""
+        self._true_ranks(self.adapters + [adapter], self.rank)
         self.adapters.append(adapter)   # (in place, as the reference does: the caller may hold the list)
         self.update_adapters(self.adapters, self.rank)
 
     def del_adapter(self, adapter_idx: int):
         assert adapter_idx < len(self.adapters)
+        self._true_ranks(self.adapters[:adapter_idx] + self.adapters[adapter_idx + 1:], self.rank)
         del self.adapters[adapter_idx]
         self.update_adapters(self.adapters, self.rank)
 
@@ -521,6 +588,7 @@ class MixedLoraLinear(nn.Module):
         lora_ids = ctx.lora_ids
         train_idx = ctx.train_idx
 
+        x_arg = x  # the tensor the caller handed over (a projection group recognises its input by it)
         x = x.to(self.dtype)
         drop_spec = None
         if blen.tlen > 0 and self.fused:
@@ -550,12 +618,13 @@ class MixedLoraLinear(nn.Module):
             result = result.to(self.dtype).contiguous()
             if not x.is_contiguous():
                 x = x.contiguous()
+            ctx.check_adapter_ids(len(self.adapters))
             plan = ctx.plan(self.device, x.size(0))
-            if self._group is not None and blen.tlen == 0 and not weights and not (
+            if self._group is not None and not self._group[0].suspended and blen.tlen == 0 and not weights and not (
                     torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):
                 # a serving step: the group's members share one shrink launch
                 self._group[0].expand_member(self._group[1], result, x, seg_scale, plan,
-                                             may_defer=result.dtype == torch_result_dtype)
+                                             may_defer=result.dtype == torch_result_dtype, src=x_arg)
                 return result.to(torch_result_dtype)
             if not weights and drop_spec is None and not (
                     torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):

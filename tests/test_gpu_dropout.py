@@ -287,9 +287,13 @@ def test_mixed_lora_linear_layer_with_dropout(K, oracle, gpu_device):
     blen = BatchLenInfo([(1, 24), (1, 16)], [9], 3, [], d)
     ctx.update(blen=blen, lora_ids=lora_ids, lora_len=lora_len, segment=segment, train_idx=[1, 3])
     torch.manual_seed(777)
-    offset = 8  # the first dropout call of a fresh context (MixedLoraContext.next_dropout_offset)
     xd = dev_t(xs, dt, d).requires_grad_(True)
     out = layer(xd)
+    # the first dropout call of a fresh context: its salt (drawn from torch's CPU generator at that call,
+    # after the seed above was set) plus eight (MixedLoraContext.next_dropout_offset)
+    salt, calls = ctx.dropout_state()
+    assert calls == 1 and salt is not None
+    offset = salt + 8
     # rows 0..23 drop with 0.5, rows 24..39 with 0.25, the prefill rows of adapter 3 and the decode
     # rows (adapter 2 has p = 0.9 but never trains here) are not dropped
     rp = np.zeros(T, np.float32)

@@ -247,3 +247,50 @@ def test_grouped_layers_under_graph_capture(K, gpu_device, deferred):
             want = [p[1](x) for p in pairs]
             for a, b in zip(outs, want):
                 assert torch.equal(a, b)
+
+
+def test_group_under_inference_mode_and_with_a_strided_input(K, gpu_device, monkeypatch):
+    """A serving loop under torch.inference_mode (tensors without a version counter) and an input that is a
+    strided view (the layer works on a contiguous copy): the members still share ONE shrink launch and
+    the results equal the ungrouped layers'."""
+    from loquetier_amd import mixed_lora as ml
+    d, tdt = gpu_device, torch.float16
+    h_in, r, NA = 2048, 16, 4
+    ctx, pairs = build(d, tdt, [256, 512, 256], h_in, r, NA, 8)
+    ml.ProjectionGroup([p[0] for p in pairs])
+    req_ids, req_len = [1, 0, 3, 2, 1, 0, 0], [1, 1, 1, 1, 1, 1, 9]
+    T = sum(req_len)
+    shrinks = []
+    real = ml.kernel.smlm_lora_forward_multi
+
+    def counting(*a, **kw):
+        if kw.get("stages") == 1:
+            shrinks.append(1)
+        return real(*a, **kw)
+    monkeypatch.setattr(ml.kernel, "smlm_lora_forward_multi", counting)
+    gen = torch.Generator().manual_seed(12)
+    with torch.inference_mode():
+        serve_step(ctx, d, req_ids, req_len)
+        x = torch.randn(T, h_in, generator=gen).to(tdt).to(d)
+        got = [p[0](x) for p in pairs]
+        assert len(shrinks) == 1
+        for g_, p in zip(got, pairs):
+            assert torch.equal(g_, p[1](x))
+        # a strided view: every member is handed the same view object, each makes its own contiguous copy
+        wide = torch.randn(T, 2 * h_in, generator=gen).to(tdt).to(d)
+        view = wide[:, ::2]
+        assert not view.is_contiguous()
+        del shrinks[:]
+        got = [p[0](view) for p in pairs]
+        assert len(shrinks) == 1
+        for g_, p in zip(got, pairs):
+            assert torch.equal(g_, p[1](view.contiguous()))
+    # and outside inference mode, with no_grad, a strided view of an ordinary tensor
+    with torch.no_grad():
+        serve_step(ctx, d, req_ids, req_len)
+        wide = torch.randn(T, 2 * h_in, generator=gen).to(tdt).to(d)
+        del shrinks[:]
+        got = [p[0](wide[:, 1::2]) for p in pairs]     # equal views made anew for every call
+        assert len(shrinks) == 1
+        for g_, p in zip(got, pairs):
+            assert torch.equal(g_, p[1](wide[:, 1::2].contiguous()))

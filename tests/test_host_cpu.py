@@ -286,3 +286,93 @@ def test_layer_adapter_list_management():
     assert scaled.scaling is None
     scaled.add_adapter(adapter(1, 3.0))
     assert scaled.scaling is None and scaled.wb_ptrs.numel() == 2
+
+
+def _cpu_layer(ml, n_adapters=2, rank=8, fused=True):
+    class Base(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.zeros(8, 16), requires_grad=False)
+    ads = [ml.NamedLoraLayer(f"a{i}", torch.full((rank, 16), float(i)), torch.full((8, rank), 10.0 + i),
+                             torch.nn.Identity(), 2.0) for i in range(n_adapters)]
+    ctx = ml.MixedLoraContext()
+    return ctx, ml.MixedLoraLinear(ctx, Base(), ads, rank, torch.float32, is_scaled=False, fused=fused)
+
+
+def test_host_adapter_ids_must_index_the_layers_adapters():
+    """A host list of adapter ids with an id at or past the number of adapters is refused before any
+    launch (the kernels, which are also told the table length, would skip such segments); negative ids
+    (segments no adapter serves) and ids that live on the device pass."""
+    from loquetier_amd import mixed_lora as ml
+    ctx, layer = _cpu_layer(ml, n_adapters=3)
+    ctx.update(lora_ids=[0, 2, -1, 1])
+    ctx.check_adapter_ids(3)
+    with pytest.raises(IndexError, match="adapter id 2"):
+        ctx.check_adapter_ids(2)
+    ctx.update(lora_ids=[0, 3])
+    with pytest.raises(IndexError):
+        ctx.check_adapter_ids(len(layer.adapters))
+    ctx.update(lora_ids=torch.tensor([0, 7], dtype=torch.int32))  # device-side ids: not read back
+    ctx.check_adapter_ids(3)
+    ctx.update(lora_ids=[])
+    ctx.check_adapter_ids(1)
+
+
+def test_projection_group_input_key():
+    """The key a projection group recognises its input by: no version counter is read from inference
+    tensors (they have none), a strided tensor is keyed by its own address and strides, and an in-place
+    change of an ordinary tensor changes the key."""
+    from loquetier_amd.mixed_lora import ProjectionGroup
+    x = torch.zeros(6, 8)
+    k0 = ProjectionGroup.input_key(x)
+    assert k0 == ProjectionGroup.input_key(x)
+    x.add_(1.0)
+    assert ProjectionGroup.input_key(x) != k0
+    with torch.inference_mode():
+        y = torch.zeros(6, 8)
+        ky = ProjectionGroup.input_key(y)     # would raise if it asked for y._version
+        assert ky[1] is None and ky == ProjectionGroup.input_key(y)
+    s1, s2 = x[:, ::2], x[:, 1::2]
+    assert not s1.is_contiguous()
+    assert ProjectionGroup.input_key(s1) == ProjectionGroup.input_key(x[:, ::2])
+    assert ProjectionGroup.input_key(s1) != ProjectionGroup.input_key(s2)
+    assert ProjectionGroup.input_key(s1) != ProjectionGroup.input_key(s1.contiguous())
+
+
+def test_dropout_offsets_differ_between_contexts_and_can_be_restored():
+    from loquetier_amd import mixed_lora as ml
+    torch.manual_seed(1234)
+    a, b = ml.MixedLoraContext(), ml.MixedLoraContext()
+    oa, ob = [a.next_dropout_offset() for _ in range(3)], [b.next_dropout_offset() for _ in range(3)]
+    assert oa[1] - oa[0] == 8 and oa[2] - oa[1] == 8          # eight projections' worth apart
+    assert not set(range(oa[0], oa[2] + 8)) & set(range(ob[0], ob[2] + 8))  # two contexts: different streams
+    torch.manual_seed(1234)                                    # a fresh context after re-seeding repeats the run
+    c = ml.MixedLoraContext()
+    assert [c.next_dropout_offset() for _ in range(3)] == oa
+    state = a.dropout_state()
+    nxt = a.next_dropout_offset()
+    d = ml.MixedLoraContext()
+    d.set_dropout_state(state)                                 # a resumed run continues the sequence
+    assert d.next_dropout_offset() == nxt
+    assert 0 <= nxt < 2 ** 63
+
+
+def test_refused_adapter_set_leaves_the_layer_unchanged():
+    """add_adapter with an adapter the layer cannot serve raises and changes neither the caller's list
+    nor the layer's tables (an unfused layer cannot take an adapter stored below the layer's rank)."""
+    from loquetier_amd import mixed_lora as ml
+    ctx, layer = _cpu_layer(ml, n_adapters=2, rank=16, fused=False)
+    held, ptrs = layer.adapters, layer.wa_ptrs.tolist()
+    bad = ml.NamedLoraLayer("short", torch.zeros(8, 16), torch.zeros(8, 8), torch.nn.Identity(), 1.0)
+    with pytest.raises(RuntimeError, match="fused path"):
+        layer.add_adapter(bad)
+    assert layer.adapters is held and len(held) == 2 and layer.wa_ptrs.tolist() == ptrs
+    assert layer.scaling.numel() == 2 and layer.adapter_rank is None and not layer.packed
+    # a fused layer takes no adapter whose A and B are stored at different ranks
+    ctx2, fused = _cpu_layer(ml, n_adapters=2, rank=16, fused=True)
+    odd = ml.NamedLoraLayer("odd", torch.zeros(8, 16), torch.zeros(8, 16), torch.nn.Identity(), 1.0)
+    with pytest.raises(RuntimeError, match="packed storage"):
+        fused.add_adapter(odd)
+    assert len(fused.adapters) == 2 and fused.wa_ptrs.numel() == 2 and not fused.packed
+    fused.add_adapter(bad)  # stored at its own rank beside padded ones: served (packed_ranks)
+    assert len(fused.adapters) == 3 and fused.packed and fused.adapter_rank.tolist() == [16, 16, 8]
