@@ -298,6 +298,13 @@ typedef struct smlm_dropout {
  *                  workspace and stream, in the order PRODUCTS, DX, WGRAD (each reads what the stage
  *                  before left in the workspace) -- to time them one by one, or to put other work of
  *                  the stream between them.  A plan the call is to build is built by the PRODUCTS stage.
+ *   w_row_major  : (backward entry points) non-zero: the weights are in the layout the reference calls
+ *                  is_row_major = True -- A_a [h_in, r], B_a [r, h_out] row-major -- the layout its Python
+ *                  backward is written for (src/loquetier_src/kernel_utils.py:139-145):
+ *                    mid = dY B^T   dX = s mid A^T   dA_a = sum x^T (s mid)   dB_a = sum (s x A)^T dY
+ *                  with dA_a [h_in, r] and dB_a [r, h_out] in the weights' own shapes.  Same kernels, no
+ *                  copies; not together with dropout or packed_ranks.  (The forward in this layout is
+ *                  smlm_gemm / smlm_gemm_planned with w_row_major = 1.)
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;
@@ -306,6 +313,7 @@ typedef struct smlm_lora_opts {
   const int32_t* build_seg_indptr;
   const int32_t* build_seg_adapter;
   int bwd_stages;
+  int w_row_major;
 } smlm_lora_opts;
 
 /* smlm_lora_fwd_multi with options. */

@@ -675,11 +675,21 @@ SMLM_API int smlm_gemm_planned(void* y, const void* x, const void* const* w_ptrs
     P.v = reinterpret_cast<const uint16_t*>(x);
     P.w_ptrs = w_ptrs;
     P.d_in = d_in; P.d_out = d_out; P.ldw = w_ld;
+    // Row-major weights (element (k, n) at w[k * w_ld + n]) are the [k][n] layout the tile-block kernels read
+    // as it lies (as the backward's dX = dV A does): up to a contraction of 64 they run at every size, as
+    // they do for the backward; longer ones keep the one-tile kernel's strided reads.
+    if (w_row_major && d_in <= 64) {
+      a.w_kn = 1;
+      return launch_expand(dtype, false, expand_nq(T, d_out), kBlkTiles, S, n_weights, 1, d_in, st, a);
+    }
     return launch_expand(dtype, w_row_major != 0, expand_nq(T, d_out), tiles_per_wave(T, d_in), S, n_weights,
                          1, d_in, st, a);
   }
   float* partial = reinterpret_cast<float*>(workspace);
-  return run_shrink(dtype, w_row_major != 0, pv, T, S, n_weights, 1, &x, &w_ptrs, &partial, &y, &d_in,
+  if (w_row_major)  // the tile-block shrink stages [k][n] weights as they lie (as the backward's dV = dY B does)
+    return run_shrink(dtype, false, pv, T, S, n_weights, 1, &x, &w_ptrs, &partial, &y, &d_in, d_out, &w_ld, beta,
+                      seg_scale, kBlkTiles, st, true, true);
+  return run_shrink(dtype, false, pv, T, S, n_weights, 1, &x, &w_ptrs, &partial, &y, &d_in,
                     d_out, &w_ld, beta, seg_scale, tiles_per_wave(T, d_out), st);
 }
 
@@ -952,6 +962,9 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
   const int stages = (opts && opts->bwd_stages) ? opts->bwd_stages : (SMLM_BWD_PRODUCTS | SMLM_BWD_DX | SMLM_BWD_WGRAD);
+  // the other weight layout (the reference's is_row_major = True): A_a [h_in, r], B_a [r, h_out], and so are dA_a, dB_a
+  const bool rm = opts && opts->w_row_major;
+  if (rm && (drop.seg_p || packed)) return SMLM_ERR_ARG;
   if (stages < 0 || stages > (SMLM_BWD_PRODUCTS | SMLM_BWD_DX | SMLM_BWD_WGRAD)) return SMLM_ERR_ARG;
   if (n_proj < 1 || n_proj > kMaxProj || NA < 0 || r <= 0 || !h_in || !h_out) return SMLM_ERR_ARG;
   if (r & 7) return SMLM_ERR_ALIGN;
@@ -994,7 +1007,9 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   // tile-block kernels read the weights as they lie in memory; ranks above 64 take the one-tile
   // expand kernel's general k loop, which reads [n][k] weights: transposed copies At [h_in, r],
   // Bt [r, h_out] made here.
-  const bool in_place = mt > 1 && r <= 64;
+  // (The row-major layout needs no copies at any rank: dV = dY B^T and dX = dV A^T read B [r, h_out] and
+  // A [h_in, r] the way the forward reads A [r, h_in] and B [h_out, r], and v = x A reads A as [k][n].)
+  const bool in_place = rm || (mt > 1 && r <= 64);
   if (!in_place && products) {
     for (int i = 0; i < n_proj; ++i) {
       TransposeArgs ta{};
@@ -1048,8 +1063,14 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   if (!have_v && products) {
     DropArgs vdrop = drop;
     vdrop.bits = nullptr;  // the shrink kernels run the generator themselves; nothing to store here
-    if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
-                         0.0f, nullptr, mt, st, true, false, &vdrop, w_rank, 0, nullptr, true)))  // v of the dropped x, as the forward made it
+    if (rm) {  // A [h_in, r] is [k][n]: the tile-block shrink at every size
+      int a_ld[kMaxProj];
+      for (int i = 0; i < n_proj; ++i) a_ld[i] = r;
+      if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, x, a_ptrs, partial, v16, h_in, r, a_ld, 0.0f,
+                           nullptr, kBlkTiles, st, true, true, nullptr, w_rank, 0, nullptr, true)))
+        return rc;
+    } else if ((rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
+                                0.0f, nullptr, mt, st, true, false, &vdrop, w_rank, 0, nullptr, true)))  // v of the dropped x, as the forward made it
       return rc;
   }
 
@@ -1058,10 +1079,10 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   int b_ld[kMaxProj];
   for (int i = 0; i < n_proj; ++i) {
     btp[i] = in_place ? b_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].bt_ptrs);
-    b_ld[i] = in_place ? r : h_out[i];
+    b_ld[i] = (in_place && !rm) ? r : h_out[i];  // B [h_out, r] read as [k][n]; B [r, h_out] and the copies as [n][k]
   }
   if (products && (rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, dy, btp, partial, dv16, h_out, r, b_ld,
-                                   0.0f, nullptr, mt, st, true, in_place, nullptr, w_rank, in_place ? packed : 0,
+                                   0.0f, nullptr, mt, st, true, in_place && !rm, nullptr, w_rank, in_place ? packed : 0,
                                    self_planned ? &build : nullptr, true)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
 
@@ -1078,7 +1099,7 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     E.y = reinterpret_cast<uint16_t*>(dx[i]);
     E.v = reinterpret_cast<const uint16_t*>(dv16[i]);
     E.w_ptrs = in_place ? a_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].at_ptrs);
-    E.d_in = r; E.d_out = h_in[i]; E.ldw = in_place ? h_in[i] : r;
+    E.d_in = r; E.d_out = h_in[i]; E.ldw = (in_place && !rm) ? h_in[i] : r;  // A [r, h_in] as [k][n]; A [h_in, r] as [n][k]
     E.pt_a = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_a);
     E.pt_b = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_b);
     E.v2 = reinterpret_cast<const uint16_t*>(vv[i]);
@@ -1086,7 +1107,7 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     E.drop_pitch = h_in[i] / 8;
     if (h_in[i] > widest) widest = h_in[i];
   }
-  ea.w_kn = in_place ? 1 : 0;
+  ea.w_kn = (in_place && !rm) ? 1 : 0;
   ea.drop = drop;  // dX is the gradient with respect to x before its dropout
   if ((stages & SMLM_BWD_DX) && (rc = launch_expand(dtype, false, expand_nq(n_rows, widest), mt, P, NA, n_proj, r, st, ea)))
     return rc;
@@ -1123,12 +1144,23 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     Q.da_ptrs = da_ptrs[i];
     Q.db_ptrs = db_ptrs[i];
     Q.h_in = h_in[i]; Q.h_out = h_out[i];
-    Q.chunks_a = ceil_div(h_in[i], kWgCols);
+    if (rm) {
+      // dB [r, h_out] = sum (s v)^T dY has the shape the kernel's first product writes ([rank, columns]) and
+      // dA [h_in, r] = sum x^T (s dV) the shape of its second ([columns, rank]): the two change places
+      Q.q_a = reinterpret_cast<const uint16_t*>(dy[i]);
+      Q.q_b = reinterpret_cast<const uint16_t*>(x[i]);
+      Q.pt_a = reinterpret_cast<const uint16_t*>(ws + L.p[i].pt_b);
+      Q.pt_b = reinterpret_cast<const uint16_t*>(ws + L.p[i].pt_a);
+      Q.da_ptrs = db_ptrs[i];
+      Q.db_ptrs = da_ptrs[i];
+      Q.h_in = h_out[i]; Q.h_out = h_in[i];
+    }
+    Q.chunks_a = ceil_div(Q.h_in, kWgCols);
     Q.units_a = ceil_div(Q.chunks_a, walk);
     Q.unit0 = units;
     Q.drop_bits = bits[i];
     Q.drop_pitch = h_in[i] / 8;
-    units += Q.units_a + ceil_div(ceil_div(h_out[i], kWgCols), walk);
+    units += Q.units_a + ceil_div(ceil_div(Q.h_out, kWgCols), walk);
   }
   wa.pitch = L.pitch;
   wa.r = r;

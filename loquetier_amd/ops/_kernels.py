@@ -466,13 +466,16 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                        part_scale: Optional[torch.Tensor] = None,
                        dropout: Optional[DropoutSpec] = None,
                        adapter_rank: Optional[torch.Tensor] = None,
-                       workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
+                       workspace: Optional[Workspace] = None, packed_ranks: bool = False,
+                       is_row_major: bool = False) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
-    forward's stream with seg_p per partition; x is the tensor before dropout."""
+    forward's stream with seg_p per partition; x is the tensor before dropout.
+    is_row_major: weights and gradients in the reference's other layout, A [h_in, r], B [r, h_out]."""
     smlm_lora_backward_multi([dx], [da_ptrs], [db_ptrs], [dy], [x], None if v is None else [v], [a_ptrs],
                              [b_ptrs], plan, rank, part_scale=part_scale, dropout=dropout,
-                             adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks)
+                             adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks,
+                             is_row_major=is_row_major)
 
 
 _BWD_MULTI_SIZES: Dict[Tuple, int] = {}
@@ -497,14 +500,16 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
                              dropout: Optional[DropoutSpec] = None,
                              adapter_rank: Optional[torch.Tensor] = None,
                              workspace: Optional[Workspace] = None, packed_ranks: bool = False,
-                             stages: int = 0) -> None:
+                             stages: int = 0, is_row_major: bool = False) -> None:
     """The backward of several projections of one batch (q/k/v/o, gate/up/down) in one set of
     launches; lists of equal length, one entry per projection, each what smlm_lora_backward
     takes.  vs: None, or the saved intermediate of every projection.  The results equal
     per-projection calls bit for bit.  dropout: projection i uses the stream offset + i and
     the keep bits of the projections lie end to end (as smlm_lora_forward_multi leaves them).
     stages: 0 = everything; else SMLM_BWD_* bits (1 products v / dV, 2 dX, 4 weight gradients): the stages
-    may be issued as separate calls with the same arguments, workspace and stream, in that order."""
+    may be issued as separate calls with the same arguments, workspace and stream, in that order.
+    is_row_major: the weights and their gradients are A [h_in, r], B [r, h_out] (the layout the reference's
+    backward lines are written for, kernel_utils.py:139-145) instead of PEFT's A [r, h_in], B [h_out, r]."""
     n = len(dxs)
     lists = (da_ptrs, db_ptrs, dys, xs, a_ptrs, b_ptrs) + (() if vs is None else (vs,))
     if not (1 <= n <= 8) or any(len(l) != n for l in lists):
@@ -550,6 +555,9 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
         if stages:
             opts = opts or _lib.LoraOpts()
             opts.bwd_stages = int(stages)
+        if is_row_major:
+            opts = opts or _lib.LoraOpts()
+            opts.w_row_major = 1
         arr = lambda ts: VP(*[t.data_ptr() for t in ts])
         rc = _lib.load().smlm_lora_bwd_multi_ex(
             n, arr(dxs), arr(da_ptrs), arr(db_ptrs), arr(dys), arr(xs), None if vs is None else arr(vs),
