@@ -489,15 +489,29 @@ def reference_surface_bench(args, torch, K):
         K.smlm_forward_cutlass(st["v"], st["x"], st["wa_ptr"], seg_t, tmp_t, False)
         K.smlm_forward_cutlass(st["y"], st["v"], st["wb_ptr"], seg_t, tmp_t, False)
     t_two_k = per_call_us(two_call_kernels)
+    # the mirror's operator alone (one plan grouped by the (A, B) address pairs, built inside the shrink launch)
+    t_mirror_k = per_call_us(lambda st: add_lora.apply((T, ho), st["x"], st["wa_ptr"], st["wb_ptr"], seg_t, r, 0, []))
+    # the fused call when it has to build its plan itself, as every call of the reference surface must
+    bufs = [torch.empty(K.SegmentPlan.nbytes(T, S), dtype=torch.uint8, device=dev) for _ in sets]
+
+    def fused_own_plan(st):
+        K.smlm_lora_forward(st["base"], st["x"], st["a_tab"], st["b_tab"],
+                            K.SegmentPlan(seg_t, ids_t, T, buf=bufs[sets.index(st)], defer=True), r,
+                            seg_scale=scale_seg, beta=1.0)
+    t_fused_own = per_call_us(fused_own_plan)
     nbytes = algorithmic_bytes(w, hi, ho)
     return dict(workload=w["name"] + ", one layer call",
                 fused_call_us=round(t_fused, 2),
                 reference_lines_two_calls_us=round(t_two, 2),
                 reference_lines_two_calls_kernels_only_us=round(t_two_k, 2),
                 add_lora_mirror_us=round(t_mirror, 2),
+                add_lora_mirror_kernels_only_us=round(t_mirror_k, 2),
+                fused_call_building_its_plan_us=round(t_fused_own, 2),
                 ratio_two_calls_vs_fused=round(t_two / t_fused, 2),
                 ratio_kernels_only_vs_fused=round(t_two_k / t_fused, 2),
                 ratio_mirror_vs_fused=round(t_mirror / t_fused, 2),
+                ratio_mirror_kernels_only_vs_fused=round(t_mirror_k / t_fused, 2),
+                ratio_mirror_kernels_only_vs_fused_building_its_plan=round(t_mirror_k / t_fused_own, 2),
                 fused_call_hbm_gbps=round(nbytes / (t_fused * 1e-6) / 1e9, 1),
                 note="GPU time per layer call, graph replay over 16 rotating buffer sets; the reference-surface "
                      "legs include the caller's scale multiply and residual add (two more passes over y) unless "

@@ -45,6 +45,7 @@ extern "C" {
 #define SMLM_KEY_NONE 0 /* every segment is its own group                    */
 #define SMLM_KEY_I32 1  /* int32 adapter id per segment                      */
 #define SMLM_KEY_PTR 2  /* 64-bit weight address per segment                 */
+#define SMLM_KEY_PTR2 3 /* a pair of 64-bit weight addresses per segment (smlm_plan_build2) */
 
 /* stages of the fused forward (smlm_lora_fwd_multi) */
 #define SMLM_STAGE_SHRINK 1 /* v = x A^T, left in the workspace                */
@@ -101,6 +102,16 @@ SMLM_API int smlm_tmp_size(int num_problems, size_t* bytes);
 SMLM_API int smlm_plan_size(int T, int S, size_t* bytes);
 SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_indptr,
                              const void* seg_key, int key_kind, int T, int S, void* stream);
+/*
+ * The plan of a batch whose segments name their weights by a PAIR of addresses (device arrays
+ * of S addresses each), as the reference's add_lora.forward is handed them: wa_ptr[i] and
+ * wb_ptr[i] per problem (src/loquetier_src/kernel_utils.py:115-119).  Segments are grouped
+ * where BOTH addresses agree, so segments may share A and differ in B; one such plan serves
+ * the shrink and the expand of the fused forward, whose tables then have one entry per segment.
+ */
+SMLM_API int smlm_plan_build2(void* plan, size_t plan_bytes, const int32_t* seg_indptr,
+                              const void* const* seg_key_a, const void* const* seg_key_b, int T, int S,
+                              void* stream);
 
 /*
  * Grouped GEMM  Y_i = beta*Y_i + scale_i * X_i W_i  over the segments.
@@ -293,6 +304,11 @@ typedef struct smlm_dropout {
  *                  smlm_lora_bwd_ex takes the pair (part_indptr, part_adapter) the same way and
  *                  builds its plan inside the dV launch when r <= 64, P <= 512,
  *                  n_rows / 16 + P < 1024, v is given and there is no dropout.
+ *   build_seg_key_a, build_seg_key_b (both or neither, with build_seg_indptr, instead of
+ *                  build_seg_adapter; smlm_lora_fwd_multi_ex only):
+ *                  the plan to build is the one smlm_plan_build2 builds from these two arrays of S
+ *                  addresses; with S <= 1024 (and the other limits above) inside the shrink launch.
+ *                  The weight tables of the call have one entry per segment (n_weights = S).
  *   bwd_stages   : (backward entry points) 0 = the whole backward; else a set of SMLM_BWD_* bits: the
  *                  stages of one backward may be issued as separate calls with the same arguments,
  *                  workspace and stream, in the order PRODUCTS, DX, WGRAD (each reads what the stage
@@ -314,6 +330,8 @@ typedef struct smlm_lora_opts {
   const int32_t* build_seg_adapter;
   int bwd_stages;
   int w_row_major;
+  const void* const* build_seg_key_a;
+  const void* const* build_seg_key_b;
 } smlm_lora_opts;
 
 /* smlm_lora_fwd_multi with options. */

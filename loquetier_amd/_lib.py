@@ -12,7 +12,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "lib", "libsmlm_hip.so")
 
 SMLM_DTYPE_F16, SMLM_DTYPE_BF16 = 0, 1
-SMLM_KEY_NONE, SMLM_KEY_I32, SMLM_KEY_PTR = 0, 1, 2
+SMLM_KEY_NONE, SMLM_KEY_I32, SMLM_KEY_PTR, SMLM_KEY_PTR2 = 0, 1, 2, 3
 SMLM_ERR_DTYPE = -2
 SMLM_ERR_SCRATCH = -7
 SMLM_STATIC_SCRATCH_BYTES = 8 << 20
@@ -34,7 +34,7 @@ class LoraOpts(C.Structure):
     """struct smlm_lora_opts of include/smlm.h."""
     _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p), ("packed_ranks", C.c_int),
                 ("build_seg_indptr", C.c_void_p), ("build_seg_adapter", C.c_void_p), ("bwd_stages", C.c_int),
-                ("w_row_major", C.c_int)]
+                ("w_row_major", C.c_int), ("build_seg_key_a", C.c_void_p), ("build_seg_key_b", C.c_void_p)]
 
 
 _popts = C.POINTER(LoraOpts)
@@ -46,6 +46,7 @@ SIGNATURES = {
     "smlm_tmp_size": (_i, [_i, _psz]),
     "smlm_plan_size": (_i, [_i, _i, _psz]),
     "smlm_plan_build": (_i, [_vp, _sz, _vp, _vp, _i, _i, _i, _vp]),
+    "smlm_plan_build2": (_i, [_vp, _sz, _vp, _vp, _vp, _i, _i, _vp]),
     "smlm_gemm_workspace_size": (_i, [_i, _i, _i, _i, _psz]),
     "smlm_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "smlm_gemm_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),

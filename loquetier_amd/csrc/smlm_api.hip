@@ -280,7 +280,12 @@ int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups,
   sp.sh = a;
   sp.plan = build;
   sp.n_weights = groups;
+  // rows of workgroups: one per unit the batch can have, but no more than its rows in whole units plus 32
+  // part-filled ones -- units beyond that (more than 32 adapters in use) are taken by the same workgroups
+  // in a second round
   sp.units = tile_units_max(a.T, S, groups, c.MT);
+  const int usual = a.T / (kTileRows * c.MT) + 1 + 32;
+  if (sp.units > usual) sp.units = usual;
   int rows = 1;
   for (int i = 0; i < a.items.nproj; ++i)
     if (a.items.row_start[i + 1] - a.items.row_start[i] > rows) rows = a.items.row_start[i + 1] - a.items.row_start[i];
@@ -423,9 +428,9 @@ int check_common(int T, int S, int dtype) {
 }
 
 int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* seg_key,
-                    int key_kind, int S, hipStream_t st) {
+                    int key_kind, int S, hipStream_t st, const void* seg_key2 = nullptr) {
   const int N = next_pow2(S);
-  const PlanSortArgs sa{pv, seg_indptr, seg_key, key_kind, S, N};
+  const PlanSortArgs sa{pv, seg_indptr, seg_key, key_kind, S, N, seg_key2};
   if (S <= kPlanSmallSegs && pv.nt_max <= kPlanSmallTiles)
     return launch(plan_small_kernel, dim3(1), dim3(kPlanThreads), st, sa);
   int rc = (N <= kPlanLdsKeys)
@@ -630,6 +635,19 @@ SMLM_API int smlm_plan_build(void* plan, size_t plan_bytes, const int32_t* seg_i
   return plan_build_impl(pv, seg_indptr, seg_key, key_kind, S, (hipStream_t)stream);
 }
 
+SMLM_API int smlm_plan_build2(void* plan, size_t plan_bytes, const int32_t* seg_indptr,
+                              const void* const* seg_key_a, const void* const* seg_key_b, int T, int S,
+                              void* stream) {
+  if (T < 0 || S < 0) return SMLM_ERR_ARG;
+  if (S >= kMaxSegments || T > (1 << 30)) return SMLM_ERR_LIMIT;
+  if (S == 0) return SMLM_OK;
+  if (!plan || !seg_indptr || !seg_key_a || !seg_key_b) return SMLM_ERR_ARG;
+  if (!aligned16(plan)) return SMLM_ERR_ALIGN;
+  PlanView pv;
+  if (plan_carve(plan, T, S, &pv) > plan_bytes) return SMLM_ERR_WORKSPACE;
+  return plan_build_impl(pv, seg_indptr, seg_key_a, SMLM_KEY_PTR2, S, (hipStream_t)stream, seg_key_b);
+}
+
 SMLM_API int smlm_gemm_planned_workspace_size(int T, int d_in, int d_out, size_t* bytes) {
   if (T < 0 || d_in <= 0 || d_out <= 0 || !bytes) return SMLM_ERR_ARG;
   if (T > (1 << 30)) return SMLM_ERR_LIMIT;
@@ -723,6 +741,23 @@ SMLM_API int smlm_gemm(void* y, const void* x, const void* const* w_ptrs, const 
   hipStream_t st = (hipStream_t)stream;
   PlanView pv;
   const size_t plan_bytes = plan_carve(workspace, T, S, &pv);
+  // The plan groups the segments by their weight address.  A product that runs on the shrink kernels
+  // (d_in >= d_out, weights [n][k]) over few enough segments builds it inside its own launch: every
+  // workgroup numbers the addresses by their first occurrence and finds its tile itself, a few more
+  // write the plan for the fold launch behind it (as the fused forward does with adapter ids).
+  const int mt = tiles_per_wave(T, d_out);
+  const int nw = shrink_waves(mt, 1, &d_in, d_out);
+  const int ks = shrink_cfg(T, d_in, d_out, nw, false, mt).ksplit;
+  const bool in_launch = d_in >= d_out && !w_row_major && self_planned_ok(T, S, S, pv.nt_max, mt) &&
+                         (mt > 1 ? (S <= kFwdThreads || ks % 2 == 0)
+                                 : (nw == kDecodeWaves && (S <= kSelfPlanThreads || ks % 2 == 0)));
+  if (in_launch) {
+    if (!aligned16(y) || !aligned16(x)) return SMLM_ERR_ALIGN;
+    const PlanSortArgs build{pv, seg_indptr, w_ptrs, SMLM_KEY_PTR2, S, next_pow2(S), w_ptrs};
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan_bytes);
+    return run_shrink(dtype, false, pv, T, S, S, 1, &x, &w_ptrs, &partial, &y, &d_in, d_out, &w_ld, beta,
+                      seg_scale, mt, st, true, false, nullptr, nullptr, 0, &build);
+  }
   rc = plan_build_impl(pv, seg_indptr, w_ptrs, SMLM_KEY_PTR, S, st);
   if (rc) return rc;
   return smlm_gemm_planned(y, x, w_ptrs, S, workspace, reinterpret_cast<char*>(workspace) + plan_bytes,
@@ -798,7 +833,15 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   const int32_t* w_rank = opts ? opts->adapter_rank : nullptr;
   const int packed = (opts && opts->adapter_rank) ? opts->packed_ranks : 0;
   const int32_t* build_s = opts ? opts->build_seg_indptr : nullptr;
-  const int32_t* build_k = opts ? opts->build_seg_adapter : nullptr;
+  const void* build_k = opts ? opts->build_seg_adapter : nullptr;
+  const void* build_k2 = nullptr;
+  int build_kind = SMLM_KEY_I32;
+  if (opts && (opts->build_seg_key_a || opts->build_seg_key_b)) {  // grouped by pairs of addresses instead of ids
+    if (build_k || !opts->build_seg_key_a || !opts->build_seg_key_b) return SMLM_ERR_ARG;
+    build_k = opts->build_seg_key_a;
+    build_k2 = opts->build_seg_key_b;
+    build_kind = SMLM_KEY_PTR2;
+  }
   if ((build_s != nullptr) != (build_k != nullptr)) return SMLM_ERR_ARG;
   if (build_s && !(stages & SMLM_STAGE_SHRINK)) return SMLM_ERR_ARG;  // the plan is built with the shrink
   if (n_proj < 1 || n_proj > kMaxProj || r <= 0 || !y || !x || !a_ptrs || !b_ptrs || !h_in || !h_out)
@@ -854,14 +897,14 @@ SMLM_API int smlm_lora_fwd_multi_ex(int n_proj, void* const* y, const void* cons
   }
   // A plan still to be built (opts->build_*): decode batches build it inside the shrink launch,
   // every other batch with the plan launch first.
-  PlanSortArgs build{pv, build_s, build_k, SMLM_KEY_I32, S, next_pow2(S)};
+  PlanSortArgs build{pv, build_s, build_k, build_kind, S, next_pow2(S), build_k2};
   bool even_splits = true;  // (the decode route pairs k slices up beyond 512 segments)
   for (int i = 0; i < n_proj; ++i) even_splits = even_splits && (vsplit[i] % 2 == 0);
   // (both routes pair k slices up in one workgroup beyond 512 / 256 segments)
   const bool self_planned = build_s && !drop.seg_p && self_planned_ok(T, S, n_weights, pv.nt_max, mt) &&
                             (mt > 1 ? (S <= kFwdThreads || even_splits)
                                                    : (expand_folds && (S <= kSelfPlanThreads || even_splits)));
-  if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, SMLM_KEY_I32, S, st))) return rc;
+  if (build_s && !self_planned && (rc = plan_build_impl(pv, build_s, build_k, build_kind, S, st, build_k2))) return rc;
   if (stages & SMLM_STAGE_SHRINK) {
     rc = run_shrink(dtype, false, pv, T, S, n_weights, n_proj, x, a_ptrs, partial, v16, h_in, r, h_in,
                     0.0f, nullptr, mt, st, !expand_folds, false, &drop, w_rank, packed,

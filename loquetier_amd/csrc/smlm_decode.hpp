@@ -50,9 +50,12 @@ struct FindLds {
   int32_t hist[kSelfPlanWeights];   // rows per adapter
   uint64_t wtab[kSelfPlanWeights];  // this projection's weight table
   int32_t rtab[kSelfPlanWeights];   // true ranks, when given
+  uint64_t ka[kSelfPlanWeights], kb[kSelfPlanWeights];  // SMLM_KEY_PTR2: the segments' pairs of addresses
+  int32_t first[kSelfPlanWeights];  //   and the first segment with the same pair: the segment's id
+  int32_t slot[2][kSelfPlanWeights];  //   (scratch of first_equal_pair)
   uint32_t tot_a[THREADS / kWaveSize], tot_b[THREADS / kWaveSize];  // wave totals of the two scans
   int32_t rows[kBlkTiles * kTileRows], rseg[kBlkTiles * kTileRows];
-  int32_t sel[2];                   // adapter of the unit (-1: no such unit), unit's index within the adapter
+  int32_t sel[3];                   // adapter of the unit (-1: no such unit), unit's index within the adapter, units in all
 };
 struct FindSeg {  // the segment a thread holds
   int key, s0, len;
@@ -62,6 +65,7 @@ struct FoundUnit {
   int wid;        // adapter (table index), -1: the unit lies past the last one
   int sub;        // index of the unit among the adapter's units
   int tiles;      // tiles of the unit (1 .. UT)
+  int total;      // units of the whole batch
 };
 
 // Exclusive prefix of v over the workgroup with ONE barrier: every wave leaves its total,
@@ -89,8 +93,15 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
   constexpr int kEnt = kSelfPlanWeights / THREADS;  // table entries a thread holds: kEnt * tid ...
   const int tid = threadIdx.x, lane = tid & 63;
   int key = -1, s0 = 0, len = 0;
+  const bool pairs = pa.key_kind == SMLM_KEY_PTR2;  // uniform over the launch
+  uint64_t pair_a = 0, pair_b = 0;
   if (tid < pa.S) {
-    key = ((const SMLM_GLOBAL int32_t*)pa.key)[tid];
+    if (pairs) {
+      pair_a = ((const SMLM_GLOBAL uint64_t*)pa.key)[tid];
+      pair_b = ((const SMLM_GLOBAL uint64_t*)pa.key2)[tid];
+    } else {
+      key = ((const SMLM_GLOBAL int32_t*)pa.key)[tid];
+    }
     s0 = ((const SMLM_GLOBAL int32_t*)pa.s)[tid];
     const int s1 = ((const SMLM_GLOBAL int32_t*)pa.s)[tid + 1];
     len = s1 > s0 ? s1 - s0 : 0;
@@ -109,7 +120,15 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
   for (int e = 0; e < kEnt; ++e) F.hist[kEnt * tid + e] = 0;
   if (tid < UT * kTileRows) F.rows[tid] = -1, F.rseg[tid] = -1;
   if (tid == 0) F.sel[0] = -1;
-  __syncthreads();
+  if (pairs) {
+    // groups by pairs of addresses: the id of a segment is the first segment with its pair, as the plan
+    // builders number them (first_equal_pair; its barriers also cover the clearing above)
+    if (tid < pa.S) F.ka[tid] = pair_a, F.kb[tid] = pair_b;
+    first_equal_pair<kSelfPlanWeights>(F.ka, F.kb, F.first, F.slot[0], F.slot[1], pa.S);
+    if (tid < pa.S) key = F.first[tid];
+  } else {
+    __syncthreads();
+  }
   const bool counted = len > 0 && key >= 0 && key < NA;  // ids outside the table own no unit here
   if (counted) atomicAdd(&F.hist[key], len);              // integer adds: the total does not depend on their order
 #pragma unroll
@@ -120,7 +139,7 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
   auto units_of = [&](int a) -> uint32_t {
     return a < NA ? (uint32_t)((F.hist[a] + UT * kTileRows - 1) / (UT * kTileRows)) : 0u;
   };
-  FoundUnit u{-1, 0, 0};
+  FoundUnit u{-1, 0, 0, 0};
   if (NA <= kSelfPlanWaveScan) {
     // few adapters: every wave walks the table by itself, 64 adapters a step, and needs no barrier
     uint32_t carry = 0;
@@ -132,10 +151,10 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
         const int l = __builtin_ctzll(hit);
         u.wid = a0 + l;
         u.sub = unit - (int)__builtin_amdgcn_readlane((int)first, l);
-        break;
       }
       carry = (uint32_t)__builtin_amdgcn_readlane((int)last, kWaveSize - 1);
     }
+    u.total = (int)carry;
   } else {
     // many adapters: one scan over the workgroup, a thread holding kEnt neighbouring adapters
     uint32_t n[kEnt], sum = 0;
@@ -143,6 +162,7 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
     for (int e = 0; e < kEnt; ++e) n[e] = units_of(kEnt * tid + e), sum += n[e];
     uint32_t last;
     uint32_t first = block_scan_excl_1<THREADS>(sum, F.tot_a, &last);
+    if (tid == THREADS - 1) F.sel[2] = (int)last;
     if ((uint32_t)unit >= first && (uint32_t)unit < last) {
 #pragma unroll
       for (int e = 0; e < kEnt; ++e) {
@@ -156,6 +176,7 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
     __syncthreads();
     u.wid = F.sel[0];
     u.sub = F.sel[1];
+    u.total = F.sel[2];
   }
   if (u.wid >= 0) {
     const int tiles_a = (F.hist[u.wid] + kTileRows - 1) / kTileRows;
@@ -229,7 +250,7 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
   }
   // grid x: (k slice, 64-column block) of the projection, k slices fastest -- in pairs when a
   // workgroup takes two (the host launches that kind only when every k split is even)
-  const int pj = blockIdx.z, tile = blockIdx.y;
+  const int pj = blockIdx.z;
   if ((int)blockIdx.x * HALVES >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
   const ShrinkProj P = a.sh.p[pj];
   FindLds<THREADS>& F = sm.work.find;
@@ -243,6 +264,10 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
   const int kend = min(kbeg + P.k_per_wave, P.d_in);
   const uint16_t* zeros = reinterpret_cast<const uint16_t*>(self_plan_zeros);
 
+  // The launch has a row of workgroups for every tile the batch usually has (its rows in whole tiles plus a
+  // few dozen part-filled ones: a tile per adapter in use), not for every tile it could have (one more per
+  // table entry): a batch with more tiles than rows of workgroups sends them round again.
+  for (int tile = blockIdx.y;; tile += a.units) {
   FindSeg seg;
   const FoundUnit un =
       find_adapter<THREADS, 1>(F, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tile, &seg);
@@ -319,6 +344,9 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
         store4<DT>(P.out + (long)row * P.d_out + n, sum, scale, a.sh.beta);
     }
   }
+  if (tile + a.units >= un.total) return;  // uniform over the workgroup: no tile is left for it
+  __syncthreads();                         // the sums are read: the finder takes its LDS back
+  }
 }
 
 // ---- larger batches: the tile-block shrink_block_kernel ------------------------
@@ -358,7 +386,7 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
   }
   // grid x: (k slice, 64-column block) of the projection, k slices fastest -- in pairs when a
   // workgroup takes two (the host launches that kind only when every k split is even)
-  const int pj = blockIdx.z, tb = blockIdx.y;
+  const int pj = blockIdx.z;
   if ((int)blockIdx.x * GROUPS >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
   const ShrinkProj P = a.sh.p[pj];
   const int grp = threadIdx.x / kFwdThreads, tl = threadIdx.x % kFwdThreads;  // group of four waves, thread in it
@@ -372,6 +400,9 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
   const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
   const int kstop = GROUPS > 1 ? kbeg + kFwdWaves * P.k_per_wave : kend;  // the same number of batches for both groups
 
+  // (a row of workgroups for every tile block the batch usually has; the others go round again, as in
+  // shrink_self_planned_kernel)
+  for (int tb = blockIdx.y;; tb += a.units) {
   FindSeg seg;
   const FoundUnit un =
       find_adapter<THREADS, kBlkTiles>(sm.find, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tb, &seg);
@@ -474,6 +505,9 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
       else
         store4<DT>(P.out + (long)row * P.d_out + n, acc[nb], scale, a.sh.beta);
     }
+  }
+  if (tb + a.units >= un.total) return;  // uniform over the workgroup: no tile block is left for it
+  __syncthreads();                       // the staged weights are read: the finder takes its LDS back
   }
 }
 

@@ -26,7 +26,66 @@ struct PlanSortArgs {
   const int32_t* s;  // [S+1] segment boundaries
   const void* key;   // per-segment keys, see SMLM_KEY_*
   int key_kind, S, N;  // N = power of two >= S
+  const void* key2;  // SMLM_KEY_PTR2: the second address of every segment (the first is in `key`)
 };
+
+// SMLM_KEY_PTR2 in the one-workgroup routes: segments are grouped by a PAIR of addresses.  The pair of
+// segment i is replaced by the index of the first segment that has the same pair -- a small integer that
+// then serves as an adapter id (it indexes the caller's per-segment tables at an entry that holds this
+// group's weights), so everything built for SMLM_KEY_I32 plans applies.  ka / kb: the pairs by segment
+// (LDS), first[i] receives the index; t1, t2: scratch of M int32 each (M a power of two); S <= blockDim.x.
+// Two rounds of "smallest index per hash slot" (integer minima: the order of the atomics does not matter):
+// a segment whose slot's winner holds its pair has found its first occurrence -- every segment with that
+// pair hashes to the same slot -- and the few that lose their slot to another pair try a second hash among
+// themselves; what is still open after that (two collisions in a row) is searched for directly.  Comparing
+// every pair with every other instead costs S x S LDS reads and took longer than the shrink it serves.
+// Contains barriers; leaves the result visible to every thread.
+template <int M, typename A64, typename A32, typename T32>
+__device__ __forceinline__ void first_equal_pair(A64& ka, A64& kb, A32& first, T32& t1, T32& t2, int S) {
+  const int tid = threadIdx.x;
+  for (int m = tid; m < M; m += blockDim.x) t1[m] = 0x7fffffff, t2[m] = 0x7fffffff;
+  uint64_t a = 0, b = 0;
+  uint32_t h1 = 0, h2 = 0;
+  if (tid < S) {
+    a = ka[tid], b = kb[tid];
+    const uint64_t h = (a >> 4) * 0x9E3779B97F4A7C15ull ^ (b >> 4) * 0xC2B2AE3D27D4EB4Full;
+    h1 = (uint32_t)(h >> 40) & (M - 1);
+    h2 = (uint32_t)(h >> 24) & (M - 1);
+  }
+  __syncthreads();
+  if (tid < S) atomicMin(&t1[h1], tid);
+  __syncthreads();
+  int found = -1;
+  if (tid < S) {
+    const int c = t1[h1];
+    if (ka[c] == a && kb[c] == b) found = c;
+    else atomicMin(&t2[h2], tid);
+  }
+  __syncthreads();
+  bool open = false;
+  if (tid < S && found < 0) {
+    const int c = t2[h2];
+    if (ka[c] == a && kb[c] == b) found = c;
+    else open = true;
+  }
+  if (__ballot(open)) {  // uniform over the wave: a plain search for the lanes still open
+    int best = tid;
+    for (int j = 0; j < S; j += 8) {
+      uint64_t ca[8], cb[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int je = j + e < S ? j + e : S - 1;
+        ca[e] = ka[je], cb[e] = kb[je];
+      }
+#pragma unroll
+      for (int e = 7; e >= 0; --e)
+        if (j + e < best && ca[e] == a && cb[e] == b) best = j + e;
+    }
+    if (open) found = best;
+  }
+  if (tid < S) first[tid] = found;
+  __syncthreads();
+}
 
 // Inclusive scan of a 32-bit value over the wave with DPP adds: four shifts
 // inside each row of 16 lanes (a lane whose source falls outside its row adds
@@ -183,27 +242,37 @@ __device__ __forceinline__ void plan_small_body(const PlanSortArgs& args, PlanSm
   const PlanView pv = args.pv;
   const int S = args.S, tid = threadIdx.x;  // blockDim.x >= S
 
-  uint64_t raw = 0;
+  uint64_t raw = 0, raw2 = 0;
   int s0 = 0, s1 = 0;
   if (tid < S) {
     if (args.key_kind == SMLM_KEY_I32) raw = (uint32_t) reinterpret_cast<const int32_t*>(args.key)[tid];
-    if (args.key_kind == SMLM_KEY_PTR) raw = reinterpret_cast<const uint64_t*>(args.key)[tid];
+    if (args.key_kind == SMLM_KEY_PTR || args.key_kind == SMLM_KEY_PTR2) raw = reinterpret_cast<const uint64_t*>(args.key)[tid];
+    if (args.key_kind == SMLM_KEY_PTR2) raw2 = reinterpret_cast<const uint64_t*>(args.key2)[tid];
     s0 = args.s[tid];
     s1 = args.s[tid + 1];
+  }
+  int key_kind = args.key_kind;
+  if (key_kind == SMLM_KEY_PTR2) {  // pairs of addresses -> the first segment with the same pair, an id from here on
+    if (tid < S) K0[tid] = raw, K[tid] = raw2;
+    // (scratch: two of the group tables, CAP + 1 entries each, not in use yet)
+    first_equal_pair<CAP>(K0, K, sseg, grow, gtile, S);
+    if (tid < S) raw = (uint32_t)sseg[tid];
+    key_kind = SMLM_KEY_I32;
+    __syncthreads();  // K0, K, sseg are free again
   }
   if (tid == 0) bad_key = 0, wide_key = 0;
   __syncthreads();
   // A 16-byte aligned address below 2^48 packs into 44 bits; anything else
   // cannot be a sort key, so such a batch is planned segment by segment.
-  if (args.key_kind == SMLM_KEY_PTR && tid < S && ((raw >> 48) != 0 || (raw & 15) != 0)) bad_key = 1;
+  if (key_kind == SMLM_KEY_PTR && tid < S && ((raw >> 48) != 0 || (raw & 15) != 0)) bad_key = 1;
   // adapter ids below 2^21 sort as 32-bit keys (id, segment), half the LDS traffic and compares
-  if (tid < S && (args.key_kind != SMLM_KEY_I32 || raw >= (1u << kNarrowIdBits))) wide_key = 1;
+  if (tid < S && (key_kind != SMLM_KEY_I32 || raw >= (1u << kNarrowIdBits))) wide_key = 1;
   if (tid < S) {
     start0[tid] = s0;
     len0[tid] = s1 > s0 ? s1 - s0 : 0;
   }
   __syncthreads();
-  const int kind = bad_key ? SMLM_KEY_NONE : args.key_kind;
+  const int kind = bad_key ? SMLM_KEY_NONE : key_kind;
   uint64_t mine = ~0ull;
   if (tid < S) {
     const uint64_t gkey = kind == SMLM_KEY_I32 ? raw : (kind == SMLM_KEY_PTR ? raw >> 4 : (uint64_t)tid);
@@ -366,7 +435,11 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
   const PlanView pv = args.pv;
   const int32_t* __restrict__ s = args.s;
   const int S = args.S, N = args.N, tid = threadIdx.x;
-  const int kind = usable_kind(args.key, args.key_kind, S, &bad_key);
+  // pairs of addresses: sorted by the first address; a group also ends where the second changes (segments that
+  // share the first address and differ in the second may then fall into more groups than they need, never fewer)
+  const int kind = usable_kind(args.key, args.key_kind == SMLM_KEY_PTR2 ? SMLM_KEY_PTR : args.key_kind, S, &bad_key);
+  const uint64_t* key2 = (args.key_kind == SMLM_KEY_PTR2 && kind == SMLM_KEY_PTR)
+                             ? reinterpret_cast<const uint64_t*>(args.key2) : nullptr;
 
   if (USE_LDS) {
     for (int i = tid; i < N; i += kPlanThreads) lds_keys[i] = i < S ? make_key(args.key, kind, i) : ~0ull;
@@ -398,7 +471,10 @@ __global__ __launch_bounds__(kPlanThreads) void plan_sort_kernel(PlanSortArgs ar
       len = s[seg + 1] - s[seg];
       if (len < 0) len = 0;
       head = true;
-      if (p > 0) head = (K[p - 1] >> kSegBits) != gk;
+      if (p > 0) {
+        head = (K[p - 1] >> kSegBits) != gk;
+        if (!head && key2) head = key2[(int)(K[p - 1] & (kMaxSegments - 1))] != key2[seg];
+      }
     }
     const uint64_t v = (uint64_t)len | ((uint64_t)(head ? 1 : 0) << 32);
     const uint64_t incl = block_scan_incl(v, wave_tot) + carry;

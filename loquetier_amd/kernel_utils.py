@@ -198,14 +198,10 @@ class add_lora(Function):
         need_v = len(args) > 0 and train_len > 0
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
         # The reference looks up wa_ptr[i] and wb_ptr[i] per problem, so two segments may share A and
-        # differ in B.  A plan groups segments by ONE key and reads the weights of a group's first
-        # segment: the shrink stage runs over a plan keyed by the A addresses, the expand stage over
-        # one keyed by the B addresses (v lies between them by row, whatever the grouping).
-        plan_a = kernel.SegmentPlan(s, wa_ptr, x.size(0))
-        plan_b = kernel.SegmentPlan(s, wb_ptr, x.size(0))
-        v_arg = None if v is None else [v]  # both stages: where the shrink leaves v is where the expand finds it
-        kernel.smlm_lora_forward_multi([y], [x], [wa_ptr], [wb_ptr], plan_a, lora_rank, stages=1, v_out=v_arg)
-        kernel.smlm_lora_forward_multi([y], [x], [wa_ptr], [wb_ptr], plan_b, lora_rank, stages=2, v_out=v_arg)
+        # differ in B: the plan groups the segments where BOTH addresses agree, and is built by the
+        # fused call itself (for batches of few segments inside its shrink launch).
+        plan = kernel.SegmentPlan(s, (wa_ptr, wb_ptr), x.size(0), defer=True)
+        kernel.smlm_lora_forward(y, x, wa_ptr, wb_ptr, plan, lora_rank, v_out=v)
         # what the reference's setup_context keeps (kernel_utils.py:122-126), plus v
         ctx.tp = train_partition
         ctx.rank = lora_rank

@@ -194,10 +194,15 @@ class SegmentPlan:
     per-problem table inside every kernel call,
     smlm_forward_cutlass.cuh:76-79).
 
-    defer=True (plans keyed by int32 adapter ids): nothing is launched here; the first
-    smlm_lora_forward(_multi) or smlm_lora_backward call that gets the plan builds it --
-    for batches of few enough segments inside its first launch, at no launch of its own --
-    and every other user builds it with the plan launch first (ensure_built)."""
+    seg_key: None (every segment its own group), int32 adapter ids, int64 weight addresses, or a
+    PAIR of int64 address tensors (wa_ptr, wb_ptr) as the reference's add_lora.forward is handed
+    them (kernel_utils.py:115-119): segments are then grouped where both addresses agree, and one
+    plan serves both GEMMs of the fused forward (per-segment tables).
+
+    defer=True (plans keyed by int32 adapter ids or by a pair of address tensors): nothing is
+    launched here; the first smlm_lora_forward(_multi) or smlm_lora_backward call that gets the
+    plan builds it -- for batches of few enough segments inside its first launch, at no launch of
+    its own -- and every other user builds it with the plan launch first (ensure_built)."""
 
     def __init__(self, segment: torch.Tensor, seg_key: Optional[torch.Tensor], T: int,
                  buf: Optional[torch.Tensor] = None, defer: bool = False):
@@ -207,19 +212,27 @@ class SegmentPlan:
         self.segment = segment
         self.S = segment.size(0) - 1
         self.T = int(T)
+        self.seg_key2 = None
+        if isinstance(seg_key, (tuple, list)):
+            if len(seg_key) != 2 or any(k.dtype != torch.int64 for k in seg_key):
+                raise RuntimeError("a pair key is two int64 tensors of weight addresses")
+            seg_key, self.seg_key2 = seg_key
         self.seg_key = seg_key
         if seg_key is None:
             kind = _lib.SMLM_KEY_NONE
+        elif self.seg_key2 is not None:
+            kind = _lib.SMLM_KEY_PTR2
         elif seg_key.dtype == torch.int32:
             kind = _lib.SMLM_KEY_I32
         elif seg_key.dtype == torch.int64:
             kind = _lib.SMLM_KEY_PTR
         else:
             raise RuntimeError("seg_key must be int32 adapter ids or int64 addresses")
-        if seg_key is not None:
-            _check_input(seg_key, "seg_key")
-            if seg_key.dim() != 1 or seg_key.size(0) != self.S:
-                raise RuntimeError("seg_key must have one entry per segment")
+        for key in (seg_key, self.seg_key2):
+            if key is not None:
+                _check_input(key, "seg_key")
+                if key.dim() != 1 or key.size(0) != self.S:
+                    raise RuntimeError("seg_key must have one entry per segment")
         self.kind = kind
         dev = segment.device
         nbytes = _lib.size_query("smlm_plan_size", self.T, self.S)
@@ -229,7 +242,7 @@ class SegmentPlan:
             raise RuntimeError(f"plan buffer must be a uint8 tensor of >= {nbytes} bytes on {dev}")
         self.buf = buf
         self.built = False
-        if not (defer and kind == _lib.SMLM_KEY_I32):
+        if not (defer and kind in (_lib.SMLM_KEY_I32, _lib.SMLM_KEY_PTR2)):
             self.ensure_built()
 
     def ensure_built(self) -> None:
@@ -237,8 +250,13 @@ class SegmentPlan:
             return
         dev = self.segment.device
         with _on(dev):
-            rc = _lib.load().smlm_plan_build(self.buf.data_ptr(), self.buf.numel(), self.segment.data_ptr(),
-                                             _ptr(self.seg_key), self.kind, self.T, self.S, _stream(dev))
+            if self.kind == _lib.SMLM_KEY_PTR2:
+                rc = _lib.load().smlm_plan_build2(self.buf.data_ptr(), self.buf.numel(), self.segment.data_ptr(),
+                                                  self.seg_key.data_ptr(), self.seg_key2.data_ptr(), self.T,
+                                                  self.S, _stream(dev))
+            else:
+                rc = _lib.load().smlm_plan_build(self.buf.data_ptr(), self.buf.numel(), self.segment.data_ptr(),
+                                                 _ptr(self.seg_key), self.kind, self.T, self.S, _stream(dev))
         _lib.check(rc, "smlm_plan_build")
         self.built = True
 
@@ -447,7 +465,11 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
             if stages & _lib.SMLM_STAGE_SHRINK:  # a deferred plan: this call builds it
                 opts = opts or _lib.LoraOpts()
                 opts.build_seg_indptr = plan.segment.data_ptr()
-                opts.build_seg_adapter = plan.seg_key.data_ptr()
+                if plan.kind == _lib.SMLM_KEY_PTR2:
+                    opts.build_seg_key_a = plan.seg_key.data_ptr()
+                    opts.build_seg_key_b = plan.seg_key2.data_ptr()
+                else:
+                    opts.build_seg_adapter = plan.seg_key.data_ptr()
             else:
                 plan.ensure_built()
         rc = _lib.load().smlm_lora_fwd_multi_ex(

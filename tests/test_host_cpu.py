@@ -110,7 +110,7 @@ def test_plan_on_first_use_argument_validation(lib):
     o.build_seg_adapter = p
     assert call(o, stages=2) == -1        # the plan is built with the shrink
     assert call(o, T=0) == 0              # empty batch: nothing to build, nothing launched
-    assert ctypes.sizeof(lib.LoraOpts) == 48  # (two ints after the five pointers-and-ints: still 48)
+    assert ctypes.sizeof(lib.LoraOpts) == 64  # as the C struct: four pointers, three ints (one padded), two pointers
     # stage-by-stage calls: only a call that runs one stage may leave out the other stage's tensors
     full = lambda y, x, stages: L.smlm_lora_fwd_multi(1, VP(y), VP(x), None, VP(p), VP(p), 2, CI(64), CI(64), p, p,
                                                        1 << 30, 16, 2, 16, 0, 0.0, None, stages, None)
