@@ -492,11 +492,12 @@ def reference_surface_bench(args, torch, K):
     # the mirror's operator alone (one plan grouped by the (A, B) address pairs, built inside the shrink launch)
     t_mirror_k = per_call_us(lambda st: add_lora.apply((T, ho), st["x"], st["wa_ptr"], st["wb_ptr"], seg_t, r, 0, []))
     # the fused call when it has to build its plan itself, as every call of the reference surface must
-    bufs = [torch.empty(K.SegmentPlan.nbytes(T, S), dtype=torch.uint8, device=dev) for _ in sets]
+    for st in sets:
+        st["plan_buf"] = torch.empty(K.SegmentPlan.nbytes(T, S), dtype=torch.uint8, device=dev)
 
     def fused_own_plan(st):
         K.smlm_lora_forward(st["base"], st["x"], st["a_tab"], st["b_tab"],
-                            K.SegmentPlan(seg_t, ids_t, T, buf=bufs[sets.index(st)], defer=True), r,
+                            K.SegmentPlan(seg_t, ids_t, T, buf=st["plan_buf"], defer=True), r,
                             seg_scale=scale_seg, beta=1.0)
     t_fused_own = per_call_us(fused_own_plan)
     nbytes = algorithmic_bytes(w, hi, ho)
