@@ -374,7 +374,7 @@ def model_step_bench(args, torch, K, finetune=True):
 
     params = [p for layer, _ in layers for p in layer.parameters() if p.requires_grad]
 
-    def train_step():
+    def train_step(one_engine_run=False):
         for p in params:  # what optimizer.zero_grad() does by default: the backward then hands its buffers over
             p.grad = None
         update(w, ctx, [0, 1, 2, 3])
@@ -382,28 +382,44 @@ def model_step_bench(args, torch, K, finetune=True):
         for layer, x in layers:
             outs.append(layer(x))  # dX is computed and handed to autograd, which has no use for it here
         t_f = time.perf_counter()
-        for o in reversed(outs):
-            o.backward(grads[o.size(1)])
+        if one_engine_run:  # as loss.backward() of a model does: autograd's engine starts once for all the layers
+            torch.autograd.backward(outs[::-1], [grads[o.size(1)] for o in outs[::-1]])
+        else:               # the engine is started (and its device thread woken) once per layer
+            for o in reversed(outs):
+                o.backward(grads[o.size(1)])
         return t_f
+
+    def timed(one_engine_run, n=7):
+        rows = []
+        for _ in range(n):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            t_f = train_step(one_engine_run)
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            rows.append(((t_f - t0) * 1e6 / len(layers), (t1 - t_f) * 1e6 / len(layers), (t2 - t0) * 1e6 / len(layers)))
+        return rows
+    med = lambda rows, i: round(float(np.median([r[i] for r in rows])), 2)
     with torch.cuda.stream(cap):
         for _ in range(2 + max(0, min(args.steps, 50) - 5) // 4):  # (more steps on request: copy-trace runs)
             train_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        t_f = train_step()
-        t1 = time.perf_counter()
-        torch.cuda.synchronize()
-        t2 = time.perf_counter()
+            train_step(True)
+        per_layer, one_run = timed(False), timed(True)
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
         a.record(cap)
-        train_step()
+        train_step(True)
         b.record(cap)
         torch.cuda.synchronize()
     out["finetune_forward_backward"] = dict(
         workload=w["name"], calls_per_step=len(layers), training_rows=n_train,
-        host_us_per_call_forward=round((t_f - t0) * 1e6 / len(layers), 2),
-        host_us_per_call_backward=round((t1 - t_f) * 1e6 / len(layers), 2),
-        eager_us_per_call_incl_gpu=round((t2 - t0) * 1e6 / len(layers), 2),
+        timing="median of 7 steps, each started on an idle GPU",
+        host_us_per_call_forward=med(per_layer + one_run, 0),
+        host_us_per_call_backward=med(one_run, 1),
+        host_us_per_call_backward_one_backward_call_per_layer=med(per_layer, 1),
+        eager_us_per_call_incl_gpu=med(one_run, 2),
+        eager_us_per_call_incl_gpu_one_backward_call_per_layer=med(per_layer, 2),
         event_us_per_call=round(a.elapsed_time(b) * 1e3 / len(layers), 2))
     return out
 

@@ -125,31 +125,44 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
         grad_x[tl:].zero_()
     if tp[0] > 0:
         grad_x[: tp[0]].zero_()
-    prepared = step is not None and step.bwd_plan is not None and step.grad_offsets is not None
+    prepared = step is not None and step.bwd_plan is not None and step.grad_layout is not None
     if prepared:
         part_adapter = step.part_adapter
-        shapes, numel = step.grad_shapes
-        buf = torch.empty(numel, dtype=dt, device=dev)          # all dA, then all dB, in one allocation
-        mats = [buf[o: o + shape[0] * shape[1]].view(shape) for o, shape in shapes]
-        NA = len(mats) // 2
-        da, db = mats[:NA], mats[NA:]
+        lay = step.grad_layout
+        uniform, known = lay["grad_uniform"], lay["grad_tabs"]
         # addresses of the gradients: device arithmetic, no copy from the host; torch's allocator hands the
-        # same block out step after step, so the table of an address is kept
-        tabs = None if step.grad_tabs is None else step.grad_tabs.get(buf.data_ptr())
-        if tabs is None:
-            tabs = step.grad_offsets + buf.data_ptr()
-            if step.grad_tabs is not None:
-                if len(step.grad_tabs) >= 64:
-                    step.grad_tabs.clear()
-                step.grad_tabs[buf.data_ptr()] = tabs
+        # same blocks out step after step, so the tables of an address are kept
+        if uniform is not None:   # matrices of one shape: one tensor for the dA, one for the dB
+            NA, sa, sb = uniform
+            ga, gb = torch.empty((NA,) + sa, dtype=dt, device=dev), torch.empty((NA,) + sb, dtype=dt, device=dev)
+            da, db = ga.unbind(0), gb.unbind(0)
+            bufs, where = (ga, gb), (ga.data_ptr(), gb.data_ptr())
+            tabs = known.get(where)
+            if tabs is None:
+                tabs = (lay["grad_offsets_a"] + where[0], lay["grad_offsets_b"] + where[1])
+        else:                     # all dA, then all dB, in one allocation
+            buf = torch.empty(lay["grad_numel"], dtype=dt, device=dev)
+            mats = [buf[o: o + shape[0] * shape[1]].view(shape) for o, shape in lay["grad_shapes"]]
+            NA = len(mats) // 2
+            da, db = mats[:NA], mats[NA:]
+            bufs, where = (buf,), buf.data_ptr()
+            tabs = known.get(where)
+            if tabs is None:
+                both = lay["grad_offsets"] + where
+                tabs = (both[:NA], both[NA:])
+        if where not in known:
+            if len(known) >= 64:
+                known.clear()
+            known[where] = tabs
         if tl > 0:
             g = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
-            kernel.smlm_lora_backward(grad_x, tabs[:NA], tabs[NA:], g, x_train, v_train, step.a_tab, step.b_tab,
+            kernel.smlm_lora_backward(grad_x, tabs[0], tabs[1], g, x_train, v_train, step.a_tab, step.b_tab,
                                       step.bwd_plan, lora_rank, part_scale, dropout=dropout,
                                       adapter_rank=adapter_rank, workspace=step.workspace,
-                                      packed_ranks=step.packed)
+                                      packed_ranks=step.packed, cache=step.cache)
         else:
-            buf.zero_()
+            for b in bufs:
+                b.zero_()
     else:
         pairs, part_adapter = _unique_adapters(weight_list[: 2 * n_parts])
         da = [torch.empty_like(wa) for wa, _ in pairs]

@@ -273,7 +273,8 @@ class fused_add_lora(Function):
         kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
                                  beta=1.0, v_out=v, dropout=dropout, adapter_rank=adapter_rank,
                                  workspace=None if step is None else step.workspace,
-                                 packed_ranks=step is not None and step.packed)
+                                 packed_ranks=step is not None and step.packed,
+                                 cache=None if step is None else step.cache)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
@@ -300,7 +301,7 @@ class fused_add_lora(Function):
                 ctx.part_drop = kernel.DropoutSpec(gather(dropout.seg_p), train_len,
                                                    dropout.seed, dropout.offset, dropout.mask_bits)
         if need_v:
-            ctx.save_for_backward(x[:train_len, ...], v[:train_len, ...], *weights)
+            ctx.save_for_backward(x, v, *weights)  # (whole: the backward reads the plan's rows of them)
         return result
 
     @staticmethod
@@ -325,11 +326,14 @@ class LayerStep:
     part_adapter: Optional[List[int]] = None       # training-adapter index of every partition
     a_tab: Optional[torch.Tensor] = None           # addresses of the training adapters' A / B, in order
     b_tab: Optional[torch.Tensor] = None
-    grad_offsets: Optional[torch.Tensor] = None    # byte offsets of dA_0.., dB_0.. inside one gradient buffer
-    grad_shapes: Optional[list] = None             # [(offset in elements, shape)] in the same order
-    grad_tabs: Optional[dict] = None               # gradient buffer address -> device table of the gradients' addresses
+    # where the gradients go (MixedLoraLinear._train_tables): byte offsets of dA_0.., dB_0.. inside one buffer
+    # (grad_offsets) or inside one buffer for the dA and one for the dB (grad_offsets_a / _b, when the matrices
+    # have one shape: grad_uniform), [(offset in elements, shape)] in the same order (grad_shapes, grad_numel),
+    # and the device tables of the gradients' addresses by buffer address (grad_tabs)
+    grad_layout: Optional[dict] = None
     memo: Any = None                               # the context's per-step memo (MixedLoraContext.memo)
     packed: bool = False                           # the adapters are stored at their true ranks
+    cache: Optional[dict] = None                   # the layer's checked operator calls (kernel.smlm_lora_forward_multi)
 
     def gather(self, table: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
         """table[index], computed once per step for a given pair of tensors."""
@@ -374,6 +378,7 @@ class ProjectionGroup:
             if (ra is None) != (rb is None) or (ra is not None and not torch.equal(ra, rb)):
                 raise ValueError("the layers of a group must hold adapters of the same true ranks")
         self.suspended = False  # set while the members' adapter sets disagree (one of them was changed alone)
+        self._call_cache: dict = {}  # argument blocks of the group's operator calls that have been checked once
         for i, l in enumerate(self.layers):
             l._group = (self, i)
 
@@ -386,7 +391,7 @@ class ProjectionGroup:
                                        [l.wb_ptrs for l in self.layers], plan, first.rank, seg_scale=seg_scale,
                                        beta=1.0, stages=2, adapter_rank=first.adapter_rank,
                                        workspace=first.root_context.group_workspace(first.device),
-                                       packed_ranks=first.packed, dims=self.dims())
+                                       packed_ranks=first.packed, dims=self.dims(), cache=self._call_cache)
 
     def flush(self, state) -> None:
         """The expands a deferred pass still owes: one launch per distinct scale tensor (normally one)."""
@@ -433,7 +438,8 @@ class ProjectionGroup:
                                            [l.wb_ptrs for l in self.layers], plan, first.rank, stages=1,
                                            adapter_rank=first.adapter_rank,
                                            workspace=ctx.group_workspace(first.device),
-                                           packed_ranks=first.packed, dims=self.dims())
+                                           packed_ranks=first.packed, dims=self.dims(),
+                                           cache=self._call_cache)
             # (the tensors are kept so that their addresses cannot be handed to others while the pass is open)
             state = ctx._step["open_group"] = {"group": self, "key": key, "pending": set(range(n)), "x": x,
                                                "src": src, "plan": plan, "waiting": []}
@@ -516,6 +522,8 @@ class MixedLoraLinear(nn.Module):
         self._scaling_key = None if self.is_scaled else tuple(float(a.scaling) for a in adapters)
         self._train_tabs: dict = {}   # training-adapter order -> pointer tables and gradient layout
         self._drop_probs: dict = {}   # adapter dropout probabilities -> device tensor
+        self._train_weights: dict = {}  # training adapters of a step -> their parameters, A and B in turn
+        self._call_cache: dict = {}   # argument blocks of operator calls that have been checked once
 
     def _train_tables(self, order):
         """Pointer tables of the training adapters' weights and the layout of one buffer holding all
@@ -532,22 +540,49 @@ class MixedLoraLinear(nn.Module):
                     shapes.append((off, tuple(w.shape)))
                     offsets.append(off * w.element_size())
                     off += (w.numel() + 7) // 8 * 8   # every matrix 16-byte aligned
+            was = [tuple(self.adapters[i].wa.shape) for i in order]
+            wbs = [tuple(self.adapters[i].wb.shape) for i in order]
+            # matrices of one shape lie evenly spaced: the gradients are then views taken in one go
+            uniform = ((len(order), was[0], wbs[0]) if order and len(set(was)) == 1 and len(set(wbs)) == 1
+                       and (was[0][0] * was[0][1]) % 8 == 0 and (wbs[0][0] * wbs[0][1]) % 8 == 0 else None)
+            grad_offsets = torch.tensor(offsets, dtype=torch.int64, device=self.device)
+            n_ad = len(key)
             tabs = dict(a_tab=self.wa_ptrs[idx].contiguous(), b_tab=self.wb_ptrs[idx].contiguous(),
-                        grad_offsets=torch.tensor(offsets, dtype=torch.int64, device=self.device),
-                        grad_shapes=shapes, grad_numel=off, grad_tabs={})
+                        grad_offsets=grad_offsets, grad_shapes=shapes, grad_numel=off, grad_uniform=uniform,
+                        # (offsets of the dA inside a buffer of their own, and of the dB likewise)
+                        grad_offsets_a=grad_offsets[:n_ad].contiguous(),
+                        grad_offsets_b=(grad_offsets[n_ad:] - grad_offsets[n_ad:n_ad + 1]).contiguous(),
+                        grad_tabs={})
             self._train_tabs[key] = tabs
         return tabs
 
     def _seg_dropout(self, ctx, train_idx):
         """Dropout probability of every segment (device float32) or None when no training adapter drops."""
+        for idx in train_idx:
+            d = self.adapters[idx].dropout
+            if isinstance(d, nn.Dropout) and d.training and d.p > 0.0:
+                break
+        else:
+            return None
         probs = tuple(float(a.dropout.p) if isinstance(a.dropout, nn.Dropout) and a.dropout.training else 0.0
                       for a in self.adapters)
-        if not any(probs[idx] > 0.0 for idx in train_idx):
-            return None
         table = self._drop_probs.get(probs)
         if table is None:
             table = self._drop_probs[probs] = torch.tensor(probs, dtype=torch.float32, device=self.device)
         return ctx.memo(("seg_p", probs, self.device), lambda: table[ctx.seg_adapter_long(self.device)])
+
+    def _weights_of(self, train_idx):
+        """The parameters of the step's training adapters, A and B in turn (looked up once per set: the
+        parameters are registered by set_trainable and stay the same objects)."""
+        key = tuple(train_idx)
+        weights = self._train_weights.get(key)
+        if weights is None:
+            weights = [w for idx in key for w in (self.get_parameter(f"lora-{idx}-A"),
+                                                  self.get_parameter(f"lora-{idx}-B"))]
+            if len(self._train_weights) >= 64:
+                self._train_weights.clear()
+            self._train_weights[key] = weights
+        return weights
 
     def _rank_args(self, train_idx):
         """(ranks of all adapters, ranks of the training adapters in order of first appearance),
@@ -579,6 +614,7 @@ class MixedLoraLinear(nn.Module):
         for idx in train_idx:
             self.register_parameter(f"lora-{idx}-A", nn.Parameter(self.adapters[idx].wa))
             self.register_parameter(f"lora-{idx}-B", nn.Parameter(self.adapters[idx].wb))
+        self._train_weights = {}
 
     def forward(self, x: torch.Tensor, *args: Any, **kwargs: Any) -> torch.Tensor:
         result = self.base_layer(x, *args, **kwargs)
@@ -605,8 +641,7 @@ class MixedLoraLinear(nn.Module):
                 start, end = blen.train_partition[pi], blen.train_partition[pi + 1]
                 dropped_x.append(self.adapters[idx].dropout(x[start:end, :]))
             x = torch.cat(dropped_x + [x[blen.tlen:, :]])
-        weights = [w for idx in train_idx for w in (self.get_parameter(f"lora-{idx}-A"),
-                                                    self.get_parameter(f"lora-{idx}-B"))]
+        weights = self._weights_of(train_idx)
         if self.fused:
             # per-step tables come from the context (built once for all layers), per-layer ones from
             # the layer (built once per adapter set): nothing is copied from the host in here
@@ -631,16 +666,17 @@ class MixedLoraLinear(nn.Module):
                 # nothing to differentiate: the operator is called directly, without autograd's bookkeeping
                 kernel.smlm_lora_forward(result, x, self.wa_ptrs, self.wb_ptrs, plan, self.rank,
                                          seg_scale=seg_scale, beta=1.0, adapter_rank=self.adapter_rank,
-                                         workspace=ctx.workspace(self.device), packed_ranks=self.packed)
+                                         workspace=ctx.workspace(self.device), packed_ranks=self.packed,
+                                         cache=self._call_cache)
                 return result.to(torch_result_dtype)
-            step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed)
+            step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed,
+                             cache=self._call_cache)
             if weights and blen.tlen > 0:
                 step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
                 step.part_segments = ctx.part_segments(self.device, plan)
                 tabs = self._train_tables(ctx.train_order())
                 step.a_tab, step.b_tab = tabs["a_tab"], tabs["b_tab"]
-                step.grad_offsets, step.grad_shapes = tabs["grad_offsets"], (tabs["grad_shapes"], tabs["grad_numel"])
-                step.grad_tabs = tabs["grad_tabs"]
+                step.grad_layout = tabs
             result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale, plan, self.rank,
                                           blen.tlen, blen.train_partition, drop_spec,
                                           self._rank_args(train_idx), step, *weights)

@@ -52,7 +52,8 @@ _WORKSPACES: Dict[Tuple[int, int], Workspace] = {}
 
 
 def _stream(dev: torch.device) -> int:
-    return torch.cuda.current_stream(dev).cuda_stream
+    # (the handle itself: building a torch.cuda.Stream object around it costs microseconds per call)
+    return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch.cuda.current_device())
 
 
 class _NoSwitch:
@@ -355,14 +356,14 @@ class DropoutSpec:
 
 
 def _opts(plan: SegmentPlan, dropout: Optional["DropoutSpec"], widths, adapter_rank: Optional[torch.Tensor],
-          n_weights: int, packed_ranks: bool = False):
+          n_weights: int, packed_ranks: bool = False, checked: bool = False):
     """struct smlm_lora_opts for a call (None when there is nothing to say).  The returned
-    object keeps the dropout struct alive."""
+    object keeps the dropout struct alive.  checked: the arguments were looked at by an earlier call."""
     if packed_ranks and adapter_rank is None:
         raise RuntimeError("packed_ranks needs adapter_rank: the kernels must know each adapter's stored rank")
     if dropout is None and adapter_rank is None:
         return None
-    if adapter_rank is not None:
+    if adapter_rank is not None and not checked:
         _check_input(adapter_rank, "adapter_rank")
         if adapter_rank.dtype != torch.int32 or adapter_rank.dim() != 1 or adapter_rank.size(0) < n_weights:
             raise RuntimeError("adapter_rank must be a 1D int32 tensor with one entry per weight table entry")
@@ -380,16 +381,68 @@ def smlm_lora_forward(y: torch.Tensor, x: torch.Tensor, a_ptrs: torch.Tensor, b_
                       beta: float = 0.0, v_out: Optional[torch.Tensor] = None,
                       dropout: Optional[DropoutSpec] = None,
                       adapter_rank: Optional[torch.Tensor] = None,
-                      workspace: Optional[Workspace] = None, packed_ranks: bool = False) -> None:
+                      workspace: Optional[Workspace] = None, packed_ranks: bool = False,
+                      cache: Optional[dict] = None) -> None:
     """y = beta*y + seg_scale * round(x A^T) B^T in one stream-ordered call (two launches).
     a_ptrs / b_ptrs are indexed by adapter id when the plan was built from int32
-    adapter ids, by segment otherwise."""
+    adapter ids, by segment otherwise.  cache: see smlm_lora_forward_multi."""
     smlm_lora_forward_multi([y], [x], [a_ptrs], [b_ptrs], plan, rank, seg_scale=seg_scale, beta=beta,
                             v_out=None if v_out is None else [v_out], dropout=dropout,
-                            adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks)
+                            adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks,
+                            cache=cache)
 
 
 _FWD_MULTI_SIZES: Dict[Tuple, int] = {}
+
+
+class _Checked:
+    """What a checked call leaves behind for the next call from the same place: what its tensors looked
+    like (a later call is compared with that, cheaply) and the argument blocks that do not change."""
+    __slots__ = ("descs", "same", "code", "dev", "arrs", "h_in", "h_out", "a_arr", "b_arr", "n_weights", "need",
+                 "opts")
+
+    def matches(self, tensor_lists, objects) -> bool:
+        """tensor_lists: the call's data tensors, list by list; objects: the tables and other tensors that are
+        expected to be the very objects of the checked call."""
+        for o, mine in zip(objects, self.same):
+            if o is not mine:
+                return False
+        k = 0
+        descs = self.descs
+        for ts in tensor_lists:
+            for t in ts:
+                d = descs[k]
+                k += 1
+                if t is None:
+                    if d is not None:
+                        return False
+                elif d is None or t.shape != d[0] or t.dtype != d[1] or t.device != d[2] or not t.is_contiguous():
+                    return False
+        return k == len(descs)
+
+
+def _descs(tensor_lists):
+    return [None if t is None else (t.shape, t.dtype, t.device) for ts in tensor_lists for t in ts]
+
+
+def _mask(ts) -> int:
+    m = 0
+    for i, t in enumerate(ts):
+        if t is not None:
+            m |= 1 << i
+    return m
+
+
+def _fill(arr, ts):
+    for i, t in enumerate(ts):
+        arr[i] = None if t is None else t.data_ptr()
+    return arr
+
+
+def _remember(cache: dict, key, hit: "_Checked") -> None:
+    if len(cache) >= 32:
+        cache.clear()
+    cache[key] = hit
 
 
 def _fwd_multi_workspace_size(T: int, widths_in: Tuple[int, ...], rank: int) -> int:
@@ -409,7 +462,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
                             v_out=None, stages: int = 3, dropout: Optional[DropoutSpec] = None,
                             adapter_rank: Optional[torch.Tensor] = None,
                             workspace: Optional[Workspace] = None, packed_ranks: bool = False,
-                            dims=None) -> None:
+                            dims=None, cache: Optional[dict] = None) -> None:
     """The fused forward for several projections of one batch (q/k/v/o, gate/up/down)
     in two launches.  Lists of equal length; entries of xs may be the same tensor.
     stages: 1 = shrink only, 2 = expand only (after a shrink call with the same
@@ -420,8 +473,43 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
     dropped inside the shrink kernel; projection i uses the stream offset + i.
     adapter_rank (int32, indexed like the tables): true ranks of adapters stored
     zero-padded to `rank`; the padding is then not read.  packed_ranks: the adapters are stored
-    AT their true rank rounded up to 8 (A_a [r_a, h_in], B_a [h_out, r_a]) instead of padded."""
+    AT their true rank rounded up to 8 (A_a [r_a, h_in], B_a [h_out, r_a]) instead of padded.
+    cache: a dict the caller keeps (one per layer): after a call has been checked, later calls with
+    tensors of the same shapes, dtype, device and contiguity and the same tables skip the checks and
+    reuse the argument blocks that do not change."""
     n = len(ys)
+    key = None
+    if cache is not None and dropout is None and len(xs) == n:  # (a dropout descriptor is checked call by call)
+        scale_list = () if seg_scale is None else (seg_scale,)
+        key = ("fwd", n, stages, plan.T, plan.S, plan.kind, rank, bool(packed_ranks), _mask(xs), _mask(ys),
+               None if v_out is None else _mask(v_out), len(scale_list),
+               dims if dims is None or isinstance(dims, tuple) else tuple(tuple(d_) for d_ in dims))
+        hit = cache.get(key)
+        if hit is not None and hit.matches((xs, ys, v_out or (), scale_list), (*a_ptrs, *b_ptrs, adapter_rank)):
+            dev = hit.dev
+            with _on(dev):
+                ws = _workspace(dev, hit.need, workspace)
+                opts = hit.opts
+                if not plan.built and not (stages & _lib.SMLM_STAGE_SHRINK):
+                    plan.ensure_built()
+                if not plan.built:  # a deferred plan: this call builds it
+                    opts = _opts(plan, None, None, adapter_rank, hit.n_weights, packed_ranks, checked=True) \
+                        or _lib.LoraOpts()
+                    opts.build_seg_indptr = plan.segment.data_ptr()
+                    if plan.kind == _lib.SMLM_KEY_PTR2:
+                        opts.build_seg_key_a = plan.seg_key.data_ptr()
+                        opts.build_seg_key_b = plan.seg_key2.data_ptr()
+                    else:
+                        opts.build_seg_adapter = plan.seg_key.data_ptr()
+                y_arr, x_arr, v_arr = hit.arrs
+                rc = _lib.load().smlm_lora_fwd_multi_ex(
+                    n, _fill(y_arr, ys), _fill(x_arr, xs), None if v_out is None else _fill(v_arr, v_out),
+                    hit.a_arr, hit.b_arr, hit.n_weights, hit.h_in, hit.h_out, plan.buf.data_ptr(), ws.data_ptr(),
+                    ws.numel(), plan.T, plan.S, rank, hit.code, float(beta), _ptr(seg_scale), int(stages),
+                    None if opts is None else C.byref(opts), _stream(dev))
+            _lib.check(rc, "smlm_lora_forward")
+            plan.built = True
+            return
     if not (1 <= n <= 8) or len(xs) != n or len(a_ptrs) != n or len(b_ptrs) != n or \
             (v_out is not None and len(v_out) != n):
         raise RuntimeError("between 1 and 8 projections, all lists of one length")
@@ -458,9 +546,19 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
     h_out = CI(*[dims[i][1] if ys[i] is None else ys[i].size(1) for i in range(n)])
     vo_arr = None if v_out is None else VP(*[_ptr(t) for t in v_out])
     with _on(dev):
-        ws = _workspace(dev, _fwd_multi_workspace_size(plan.T, tuple(widths_in), rank), workspace)
+        need = _fwd_multi_workspace_size(plan.T, tuple(widths_in), rank)
+        ws = _workspace(dev, need, workspace)
         n_weights = min(t.size(0) for t in list(a_ptrs) + list(b_ptrs))
         opts = _opts(plan, dropout, widths_in, adapter_rank, n_weights, packed_ranks)
+        a_arr, b_arr = VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs])
+        if key is not None:  # (every check has passed: the next call like this one takes the short way)
+            hit = _Checked()
+            hit.descs = _descs((xs, ys, v_out or (), () if seg_scale is None else (seg_scale,)))
+            hit.same = (*a_ptrs, *b_ptrs, adapter_rank)
+            hit.code, hit.dev, hit.arrs, hit.h_in, hit.h_out = code, dev, (VP(), VP(), VP()), h_in, h_out
+            hit.a_arr, hit.b_arr, hit.n_weights, hit.need = a_arr, b_arr, n_weights, need
+            hit.opts = _opts(plan, None, None, adapter_rank, n_weights, packed_ranks, checked=True)
+            _remember(cache, key, hit)
         if not plan.built:
             if stages & _lib.SMLM_STAGE_SHRINK:  # a deferred plan: this call builds it
                 opts = opts or _lib.LoraOpts()
@@ -474,7 +572,7 @@ def smlm_lora_forward_multi(ys, xs, a_ptrs, b_ptrs, plan: SegmentPlan, rank: int
                 plan.ensure_built()
         rc = _lib.load().smlm_lora_fwd_multi_ex(
             n, VP(*[_ptr(t) for t in ys]), VP(*[_ptr(t) for t in xs]), vo_arr,
-            VP(*[t.data_ptr() for t in a_ptrs]), VP(*[t.data_ptr() for t in b_ptrs]),
+            a_arr, b_arr,
             n_weights, h_in, h_out,
             plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, rank, code, float(beta),
             _ptr(seg_scale), int(stages), None if opts is None else C.byref(opts), _stream(dev))
@@ -489,7 +587,7 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                        dropout: Optional[DropoutSpec] = None,
                        adapter_rank: Optional[torch.Tensor] = None,
                        workspace: Optional[Workspace] = None, packed_ranks: bool = False,
-                       is_row_major: bool = False) -> None:
+                       is_row_major: bool = False, cache: Optional[dict] = None) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
     forward's stream with seg_p per partition; x is the tensor before dropout.
@@ -497,10 +595,22 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     smlm_lora_backward_multi([dx], [da_ptrs], [db_ptrs], [dy], [x], None if v is None else [v], [a_ptrs],
                              [b_ptrs], plan, rank, part_scale=part_scale, dropout=dropout,
                              adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks,
-                             is_row_major=is_row_major)
+                             is_row_major=is_row_major, cache=cache)
 
 
 _BWD_MULTI_SIZES: Dict[Tuple, int] = {}
+
+
+def _bwd_opts(plan, adapter_rank, n_weights, packed_ranks, stages, is_row_major, checked, dropout=None, widths=None):
+    """struct smlm_lora_opts of a backward call (None when there is nothing to say)."""
+    opts = _opts(plan, dropout, widths, adapter_rank, n_weights, packed_ranks, checked=checked)
+    if stages:
+        opts = opts or _lib.LoraOpts()
+        opts.bwd_stages = int(stages)
+    if is_row_major:
+        opts = opts or _lib.LoraOpts()
+        opts.w_row_major = 1
+    return opts
 
 
 def _bwd_multi_workspace_size(n_rows: int, P: int, NA: int, widths_in: Tuple[int, ...],
@@ -522,7 +632,8 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
                              dropout: Optional[DropoutSpec] = None,
                              adapter_rank: Optional[torch.Tensor] = None,
                              workspace: Optional[Workspace] = None, packed_ranks: bool = False,
-                             stages: int = 0, is_row_major: bool = False) -> None:
+                             stages: int = 0, is_row_major: bool = False,
+                             cache: Optional[dict] = None) -> None:
     """The backward of several projections of one batch (q/k/v/o, gate/up/down) in one set of
     launches; lists of equal length, one entry per projection, each what smlm_lora_backward
     takes.  vs: None, or the saved intermediate of every projection.  The results equal
@@ -531,8 +642,38 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
     stages: 0 = everything; else SMLM_BWD_* bits (1 products v / dV, 2 dX, 4 weight gradients): the stages
     may be issued as separate calls with the same arguments, workspace and stream, in that order.
     is_row_major: the weights and their gradients are A [h_in, r], B [r, h_out] (the layout the reference's
-    backward lines are written for, kernel_utils.py:139-145) instead of PEFT's A [r, h_in], B [h_out, r]."""
+    backward lines are written for, kernel_utils.py:139-145) instead of PEFT's A [r, h_in], B [h_out, r].
+    cache: as in smlm_lora_forward_multi (the same dict may serve a layer's forward and backward)."""
     n = len(dxs)
+    key = None
+    if cache is not None and dropout is None:  # (a dropout descriptor is checked call by call)
+        scale_list = () if part_scale is None else (part_scale,)
+        key = ("bwd", n, stages, plan.T, plan.S, plan.kind, rank, bool(packed_ranks), bool(is_row_major),
+               vs is None, len(scale_list))
+        hit = cache.get(key)
+        if hit is not None and hit.matches((dxs, dys, xs, vs or (), da_ptrs, db_ptrs, scale_list),
+                                           (*a_ptrs, *b_ptrs, adapter_rank)):
+            dev = hit.dev
+            with _on(dev):
+                ws = _workspace(dev, hit.need, workspace)
+                opts = hit.opts
+                if not plan.built and stages and not (stages & _lib.SMLM_BWD_PRODUCTS):
+                    plan.ensure_built()
+                if not plan.built:  # a deferred plan: this call builds it
+                    opts = _bwd_opts(plan, adapter_rank, hit.n_weights, packed_ranks, stages, is_row_major, True) \
+                        or _lib.LoraOpts()
+                    opts.build_seg_indptr = plan.segment.data_ptr()
+                    opts.build_seg_adapter = plan.seg_key.data_ptr()
+                dx_arr, dy_arr, x_arr, v_arr, da_arr, db_arr = hit.arrs
+                rc = _lib.load().smlm_lora_bwd_multi_ex(
+                    n, _fill(dx_arr, dxs), _fill(da_arr, da_ptrs), _fill(db_arr, db_ptrs), _fill(dy_arr, dys),
+                    _fill(x_arr, xs), None if vs is None else _fill(v_arr, vs), hit.a_arr, hit.b_arr,
+                    plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), plan.T, plan.S, hit.n_weights, hit.h_in,
+                    hit.h_out, rank, hit.code, _ptr(part_scale), None if opts is None else C.byref(opts),
+                    _stream(dev))
+            _lib.check(rc, "smlm_lora_backward")
+            plan.built = True
+            return
     lists = (da_ptrs, db_ptrs, dys, xs, a_ptrs, b_ptrs) + (() if vs is None else (vs,))
     if not (1 <= n <= 8) or any(len(l) != n for l in lists):
         raise RuntimeError("between 1 and 8 projections, all lists of one length")
@@ -563,10 +704,22 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
     dev = dys[0].device
     VP, CI = C.c_void_p * n, C.c_int * n
     with _on(dev):
-        ws = _workspace(dev, _bwd_multi_workspace_size(n_rows, plan.S, NA, widths_in, widths_out, rank), workspace)
+        need = _bwd_multi_workspace_size(n_rows, plan.S, NA, widths_in, widths_out, rank)
+        ws = _workspace(dev, need, workspace)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
-        opts = _opts(plan, dropout, list(widths_in), adapter_rank, NA, packed_ranks)
+        opts = _bwd_opts(plan, adapter_rank, NA, packed_ranks, stages, is_row_major, False, dropout,
+                         list(widths_in))
+        arr = lambda ts: VP(*[t.data_ptr() for t in ts])
+        a_arr, b_arr, h_in, h_out = arr(a_ptrs), arr(b_ptrs), CI(*widths_in), CI(*widths_out)
+        if key is not None:  # (every check has passed: the next call like this one takes the short way)
+            hit = _Checked()
+            hit.descs = _descs((dxs, dys, xs, vs or (), da_ptrs, db_ptrs, () if part_scale is None else (part_scale,)))
+            hit.same = (*a_ptrs, *b_ptrs, adapter_rank)
+            hit.code, hit.dev, hit.arrs, hit.h_in, hit.h_out = code, dev, tuple(VP() for _ in range(6)), h_in, h_out
+            hit.a_arr, hit.b_arr, hit.n_weights, hit.need = a_arr, b_arr, NA, need
+            hit.opts = _bwd_opts(plan, adapter_rank, NA, packed_ranks, stages, is_row_major, True)
+            _remember(cache, key, hit)
         if not plan.built:  # a deferred plan: this call builds it (inside its first launch where it can)
             if stages and not (stages & _lib.SMLM_BWD_PRODUCTS):
                 plan.ensure_built()
@@ -574,17 +727,10 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
                 opts = opts or _lib.LoraOpts()
                 opts.build_seg_indptr = plan.segment.data_ptr()
                 opts.build_seg_adapter = plan.seg_key.data_ptr()
-        if stages:
-            opts = opts or _lib.LoraOpts()
-            opts.bwd_stages = int(stages)
-        if is_row_major:
-            opts = opts or _lib.LoraOpts()
-            opts.w_row_major = 1
-        arr = lambda ts: VP(*[t.data_ptr() for t in ts])
         rc = _lib.load().smlm_lora_bwd_multi_ex(
             n, arr(dxs), arr(da_ptrs), arr(db_ptrs), arr(dys), arr(xs), None if vs is None else arr(vs),
-            arr(a_ptrs), arr(b_ptrs), plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), n_rows, plan.S, NA,
-            CI(*widths_in), CI(*widths_out), rank, code, _ptr(part_scale),
+            a_arr, b_arr, plan.buf.data_ptr(), ws.data_ptr(), ws.numel(), n_rows, plan.S, NA,
+            h_in, h_out, rank, code, _ptr(part_scale),
             None if opts is None else C.byref(opts), _stream(dev))
     _lib.check(rc, "smlm_lora_backward")
     plan.built = True

@@ -163,3 +163,42 @@ def test_multi_argument_errors(K, oracle, gpu_device):
     with pytest.raises(RuntimeError):  # v of some projections only
         v0 = torch.zeros(n_rows, r, dtype=TDT[dt], device=d)
         _multi(K, projs, outs, plan, r, vs=[v0, None, None])
+
+
+def test_checked_call_cache_changes_nothing(K, oracle, gpu_device):
+    """A layer's dict of checked calls: the second call with the same shapes skips the argument checks and
+    reuses the argument blocks; its results equal an uncached call's, other shapes or a tensor the checks
+    refuse never take the short way."""
+    case, dt = CASES[1], "bf16"
+    name, tp, part_ad, NA, dims, r = case
+    d, n_rows = gpu_device, tp[-1]
+    cache = {}
+    projs, pi, pa = _setup(oracle, d, case, dt, dy=False)
+    for shift in (0, 1, 2):   # the first call fills the cache, the later ones use it with other data
+        for p in projs:
+            p["xd"] = p["xd"] + shift
+        plan = K.SegmentPlan(pi, pa, n_rows)
+        ys = [[torch.zeros(n_rows, h_out, dtype=TDT[dt], device=d) for _, h_out in dims] for _ in range(2)]
+        vs = [[torch.zeros(n_rows, r, dtype=TDT[dt], device=d) for _ in dims] for _ in range(2)]
+        for which, c in ((0, cache), (1, None)):
+            K.smlm_lora_forward_multi(ys[which], [p["xd"] for p in projs], [p["a_tab"] for p in projs],
+                                      [p["b_tab"] for p in projs], plan, r, v_out=vs[which], cache=c)
+        for a, b in zip(ys[0] + vs[0], ys[1] + vs[1]):
+            assert torch.equal(a, b)
+        cached, plain = _outputs(projs, d, dt, n_rows), _outputs(projs, d, dt, n_rows)
+        _multi(K, projs, cached, plan, r, vs=vs[0], cache=cache)
+        _multi(K, projs, plain, plan, r, vs=vs[0])
+        for m, s in zip(cached, plain):
+            assert torch.equal(m["dx"], s["dx"])
+            for a in range(NA):
+                assert torch.equal(m["dA"][a], s["dA"][a]) and torch.equal(m["dB"][a], s["dB"][a])
+    assert len(cache) == 2
+    # a strided x of the same shape is still refused
+    wide = torch.zeros(n_rows, 2 * dims[0][0], dtype=TDT[dt], device=d)
+    with pytest.raises(RuntimeError):
+        K.smlm_lora_forward_multi(ys[0], [wide[:, ::2]] + [p["xd"] for p in projs[1:]], [p["a_tab"] for p in projs],
+                                  [p["b_tab"] for p in projs], plan, r, v_out=vs[0], cache=cache)
+    # fewer rows than the plan covers: checked and refused, not cut short
+    with pytest.raises(RuntimeError):
+        K.smlm_lora_forward_multi([y[:-16] for y in ys[0]], [p["xd"] for p in projs], [p["a_tab"] for p in projs],
+                                  [p["b_tab"] for p in projs], plan, r, cache=cache)
