@@ -238,28 +238,28 @@ int launch_shrink(int dtype, bool row_major, const ShrinkCfg& c, int S, int grou
              : launch_shrink_dt<SMLM_DTYPE_BF16, false>(row_major, c.NB, MT, c.NW, grid, st, a);
 }
 
-template <int DT, int THREADS>
+template <int DT, int THREADS, bool PAIRS>
 int launch_self_planned_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
   const dim3 block(THREADS);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_self_planned_kernel<DT, 1, 4, THREADS>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_self_planned_kernel<DT, 2, 4, THREADS>, grid, block, st, a);
-  return launch(shrink_self_planned_kernel<DT, 4, 2, THREADS>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_self_planned_kernel<DT, 1, 4, THREADS, PAIRS>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_self_planned_kernel<DT, 2, 4, THREADS, PAIRS>, grid, block, st, a);
+  return launch(shrink_self_planned_kernel<DT, 4, 2, THREADS, PAIRS>, grid, block, st, a);
 }
 
-template <int DT, bool WKN, int THREADS>
+template <int DT, bool WKN, int THREADS, bool PAIRS>
 int launch_self_planned_block_nb(int NB, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
   const dim3 block(THREADS);  // U must match shrink_cfg
-  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4, WKN, THREADS>, grid, block, st, a);
-  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4, WKN, THREADS>, grid, block, st, a);
-  return launch(shrink_block_self_planned_kernel<DT, 4, 4, WKN, THREADS>, grid, block, st, a);
+  if (NB == 1) return launch(shrink_block_self_planned_kernel<DT, 1, 4, WKN, THREADS, PAIRS>, grid, block, st, a);
+  if (NB == 2) return launch(shrink_block_self_planned_kernel<DT, 2, 4, WKN, THREADS, PAIRS>, grid, block, st, a);
+  return launch(shrink_block_self_planned_kernel<DT, 4, 4, WKN, THREADS, PAIRS>, grid, block, st, a);
 }
-template <int DT, bool WKN>
+template <int DT, bool WKN, bool PAIRS>
 int launch_self_planned_block(int NB, int S, dim3 grid, hipStream_t st, const SelfPlanArgs& a) {
-  if (S <= kFwdThreads) return launch_self_planned_block_nb<DT, WKN, kFwdThreads>(NB, grid, st, a);
+  if (S <= kFwdThreads) return launch_self_planned_block_nb<DT, WKN, kFwdThreads, PAIRS>(NB, grid, st, a);
   // more segments than the four-wave workgroup has threads: two such groups a workgroup, each
   // taking one of two neighbouring k slices (the caller has checked that the splits are even)
   grid.x = (grid.x + 1) / 2;
-  return launch_self_planned_block_nb<DT, WKN, 2 * kFwdThreads>(NB, grid, st, a);
+  return launch_self_planned_block_nb<DT, WKN, 2 * kFwdThreads, PAIRS>(NB, grid, st, a);
 }
 
 // batches this route takes: few enough segments for the plan-building workgroups of the launch
@@ -272,6 +272,23 @@ bool self_planned_ok(int T, int S, int n_weights, int nt_max, int mt) {
          tile_units_max(T, S, n_weights, mt) < kMaxGridY;
 }
 
+template <int DT>
+int launch_self_planned_dt(bool pairs, const ShrinkCfg& c, int S, dim3 grid, hipStream_t st, const SelfPlanArgs& sp) {
+  if (c.MT == 1 && S > kSelfPlanThreads) {
+    // more segments than the eight-wave workgroup has threads: workgroups of two such groups of
+    // waves, each taking two neighbouring k slices (the caller has checked that the splits are even)
+    grid.x = (grid.x + 1) / 2;
+    return pairs ? launch_self_planned_nb<DT, 2 * kSelfPlanThreads, true>(c.NB, grid, st, sp)
+                 : launch_self_planned_nb<DT, 2 * kSelfPlanThreads, false>(c.NB, grid, st, sp);
+  }
+  if (c.MT > 1 && sp.sh.w_kn) return launch_self_planned_block<DT, true, false>(c.NB, S, grid, st, sp);
+  if (c.MT > 1)
+    return pairs ? launch_self_planned_block<DT, false, true>(c.NB, S, grid, st, sp)
+                 : launch_self_planned_block<DT, false, false>(c.NB, S, grid, st, sp);
+  return pairs ? launch_self_planned_nb<DT, kSelfPlanThreads, true>(c.NB, grid, st, sp)
+               : launch_self_planned_nb<DT, kSelfPlanThreads, false>(c.NB, grid, st, sp);
+}
+
 int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups, const PlanSortArgs& build,
                                hipStream_t st, const ShrinkArgs& a) {
   if (c.MT == 1 && c.NW * kWaveSize != kSelfPlanThreads) return SMLM_ERR_ARG;
@@ -280,35 +297,32 @@ int launch_shrink_self_planned(int dtype, const ShrinkCfg& c, int S, int groups,
   sp.sh = a;
   sp.plan = build;
   sp.n_weights = groups;
-  // rows of workgroups: one per unit the batch can have, but no more than its rows in whole units plus 32
-  // part-filled ones -- units beyond that (more than 32 adapters in use) are taken by the same workgroups
-  // in a second round
+  // rows of workgroups: one per unit the batch can have.  Plans keyed by pairs of addresses (a table entry per
+  // segment, so nearly all of those rows would find no unit) get no more than the batch's rows in whole units
+  // plus 32 part-filled ones; their kernels take the units beyond that in further rounds.
+  const bool pairs = build.key_kind == SMLM_KEY_PTR2;
   sp.units = tile_units_max(a.T, S, groups, c.MT);
   const int usual = a.T / (kTileRows * c.MT) + 1 + 32;
-  if (sp.units > usual) sp.units = usual;
+  if (pairs && sp.units > usual) sp.units = usual;
+  if (pairs && a.w_kn) return SMLM_ERR_ARG;  // (no caller: the row-major products build their plan with a launch)
   int rows = 1;
   for (int i = 0; i < a.items.nproj; ++i)
     if (a.items.row_start[i + 1] - a.items.row_start[i] > rows) rows = a.items.row_start[i + 1] - a.items.row_start[i];
   dim3 grid((unsigned)rows, (unsigned)sp.units + 1u, (unsigned)a.items.nproj);
-  if (c.MT == 1 && S > kSelfPlanThreads) {
-    // more segments than the eight-wave workgroup has threads: workgroups of two such groups of
-    // waves, each taking two neighbouring k slices (the caller has checked that the splits are even)
-    grid.x = (unsigned)ceil_div(rows, 2);
-    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_nb<SMLM_DTYPE_F16, 2 * kSelfPlanThreads>(c.NB, grid, st, sp)
-                                   : launch_self_planned_nb<SMLM_DTYPE_BF16, 2 * kSelfPlanThreads>(c.NB, grid, st, sp);
-  }
-  if (c.MT > 1 && a.w_kn)
-    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block<SMLM_DTYPE_F16, true>(c.NB, S, grid, st, sp)
-                                   : launch_self_planned_block<SMLM_DTYPE_BF16, true>(c.NB, S, grid, st, sp);
-  if (c.MT > 1)
-    return dtype == SMLM_DTYPE_F16 ? launch_self_planned_block<SMLM_DTYPE_F16, false>(c.NB, S, grid, st, sp)
-                                   : launch_self_planned_block<SMLM_DTYPE_BF16, false>(c.NB, S, grid, st, sp);
-  if (dtype == SMLM_DTYPE_F16) return launch_self_planned_nb<SMLM_DTYPE_F16, kSelfPlanThreads>(c.NB, grid, st, sp);
-  return launch_self_planned_nb<SMLM_DTYPE_BF16, kSelfPlanThreads>(c.NB, grid, st, sp);
+  return dtype == SMLM_DTYPE_F16 ? launch_self_planned_dt<SMLM_DTYPE_F16>(pairs, c, S, grid, st, sp)
+                                 : launch_self_planned_dt<SMLM_DTYPE_BF16>(pairs, c, S, grid, st, sp);
 }
 
-int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a) {
+int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a, bool side = false) {
   const int row_tiles = ceil_div(a.T, kTileRows);
+  if (side) {  // by tile slot: the by-products are stored in slot order
+    const int units = tile_units_max(a.T, S, groups, 1);
+    const long items = (long)units * a.nproj;
+    a.units_max = items <= kDirectItems ? units : 0;
+    const dim3 grid = a.units_max ? dim3((unsigned)items) : work_grid(items);
+    if (dtype == SMLM_DTYPE_F16) return launch(reduce_kernel<SMLM_DTYPE_F16, true>, grid, dim3(256), st, a);
+    return launch(reduce_kernel<SMLM_DTYPE_BF16, true>, grid, dim3(256), st, a);
+  }
   if (!a.seg_scale && row_tiles <= kMaxGridY * 64) {  // no scale to look up: fold row by row
     const dim3 grid((unsigned)row_tiles, (unsigned)a.nproj);
     if (dtype == SMLM_DTYPE_F16) return launch(reduce_rows_kernel<SMLM_DTYPE_F16>, grid, dim3(256), st, a);
@@ -446,13 +460,24 @@ int plan_build_impl(const PlanView& pv, const int32_t* seg_indptr, const void* s
 // out[i] = beta*out[i] + scale * x[i] W_i^T in 16 bits, via k-split fp32 partial
 // sums folded by a second launch when the split is wider than one workgroup
 // (fold = false leaves every projection's fp32 partials, one or more, for the consumer to fold)
+// by-products a fold may leave behind (ReduceProj::pt_a ...)
+struct SideOut {
+  uint16_t* pt_a[kMaxProj];
+  uint16_t* pt_b[kMaxProj];
+  const uint16_t* v2[kMaxProj];
+  const float* scale;
+  long pitch;
+};
+
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
                const void* const* x, const void* const* const* w_ptrs, float* const* partial,
                void* const* out, const int* d_in, int d_out, const int* ldw, float beta,
                const float* seg_scale, int mt, hipStream_t st, bool fold = true, bool w_kn = false,
                const DropArgs* drop = nullptr, const int32_t* w_rank = nullptr, int packed = 0,
-               const PlanSortArgs* build = nullptr, bool solo = false) {
+               const PlanSortArgs* build = nullptr, bool solo = false, const SideOut* side = nullptr,
+               bool* side_done = nullptr) {
   if (drop && drop->seg_p && (row_major || w_kn)) return SMLM_ERR_ARG;
+  if (side_done) *side_done = false;
   ShrinkArgs a{};
   if (drop) a.drop = *drop;
   a.w_kn = w_kn ? 1 : 0;
@@ -465,7 +490,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   a.items.nproj = nproj;
   a.items.row_start[0] = 0;
   ReduceArgs ra{};
-  bool need_reduce = false;
+  bool need_reduce = false, all_reduce = true;
   ShrinkCfg c0{};
   size_t bits_off = 0;
   const int nw = row_major ? kFwdWaves : shrink_waves(mt, nproj, d_in, d_out);
@@ -491,8 +516,10 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
     int rows = c.ksplit * c.zblocks;
     if (nproj == 1 && !build && rows > 1 && (rows & 1)) rows += 1;
     a.items.row_start[i + 1] = a.items.row_start[i] + rows;
-    ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit};
+    ra.p[i] = ReduceProj{partial[i], P.out, c.ksplit, side ? side->pt_a[i] : nullptr, side ? side->pt_b[i] : nullptr,
+                         side ? side->v2[i] : nullptr};
     need_reduce = need_reduce || c.ksplit > 1;
+    all_reduce = all_reduce && c.ksplit > 1;
   }
   // Folding the k-split partials inside the shrink launch (last-arriving workgroup, ticket
   // counters) was measured and dropped: the device-scope release/acquire it needs writes back
@@ -507,7 +534,14 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   ra.seg_scale = seg_scale;
   ra.beta = beta;
   ra.T = T; ra.d_out = d_out; ra.nproj = nproj;
-  return launch_reduce(dtype, S, groups, st, ra);
+  // the by-products go with the fold when every projection is folded (else they are left to the caller)
+  const bool with_side = side && all_reduce;
+  if (with_side) {
+    ra.side_scale = side->scale;
+    ra.side_pitch = side->pitch;
+  }
+  if (side_done) *side_done = with_side;
+  return launch_reduce(dtype, S, groups, st, ra, with_side);
 }
 
 template <int DT>
@@ -990,6 +1024,15 @@ SMLM_API int smlm_lora_bwd_ex(void* dx, void* const* da_ptrs, void* const* db_pt
                                 opts, stream);
 }
 
+// every projection's dV product is folded from k-split partials: the fold then writes what the weight gradients read
+static bool bwd_all_folded(int n_proj, int n_rows, const int* h_out, int r) {
+  const int mt = bwd_tiles_per_wave(n_rows, r);
+  const int nw = shrink_waves(mt, n_proj, h_out, r);
+  for (int i = 0; i < n_proj; ++i)
+    if (shrink_cfg(n_rows, h_out[i], r, nw, true, mt).ksplit <= 1) return false;
+  return true;
+}
+
 SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* const* da_ptrs,
                                     void* const* const* db_ptrs, const void* const* dy,
                                     const void* const* x, const void* const* v,
@@ -1124,10 +1167,28 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     btp[i] = in_place ? b_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].bt_ptrs);
     b_ld[i] = (in_place && !rm) ? r : h_out[i];  // B [h_out, r] read as [k][n]; B [r, h_out] and the copies as [n][k]
   }
+  // The weight gradients read s*dV and s*v by tile slot, transposed.  The fold of dV leaves them behind when there is
+  // one for every projection (cheaper there than among dX's stores: cfg4-like batch dV 12.5 -> 13.5, dX 10.8 -> 8.2 us;
+  // ragged 32-row partitions over six projections dV 84 -> 91, dX 90 -> 74 us); else dX's launch writes them.
+  // (With them out of dX's launch, dX and the weight gradients need nothing of each other.  Issuing the weight
+  // gradients on a second stream, forked after the fold and joined at the end, was measured under graph replay and
+  // dropped: the two launches did not overlap to any gain and the fork and join cost 6 us.)
+  SideOut side{};
+  for (int i = 0; i < n_proj; ++i) {
+    side.pt_a[i] = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_a);
+    side.pt_b[i] = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_b);
+    side.v2[i] = reinterpret_cast<const uint16_t*>(vv[i]);
+  }
+  side.scale = part_scale;
+  side.pitch = L.pitch;
+  // (a function of the shapes and the option: the same in every call of a staged backward)
+  const bool side_in_fold = bwd_all_folded(n_proj, n_rows, h_out, r);
+  bool side_done = false;
   if (products && (rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, dy, btp, partial, dv16, h_out, r, b_ld,
                                    0.0f, nullptr, mt, st, true, in_place && !rm, nullptr, w_rank, in_place ? packed : 0,
-                                   self_planned ? &build : nullptr, true)))
+                                   self_planned ? &build : nullptr, true, side_in_fold ? &side : nullptr, &side_done)))
     return rc;  // (B in place is read at its stored rank; the transposed copies keep the full-rank strides)
+  if (products && side_done != side_in_fold) return SMLM_ERR_ARG;  // (cannot happen: both follow shrink_cfg)
 
   // 4. dX = s dV A, and the slot-ordered transposed s*dV, s*v for step 5
   ExpandArgs ea{};
@@ -1143,9 +1204,9 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
     E.v = reinterpret_cast<const uint16_t*>(dv16[i]);
     E.w_ptrs = in_place ? a_ptrs[i] : reinterpret_cast<const void* const*>(ws + L.p[i].at_ptrs);
     E.d_in = r; E.d_out = h_in[i]; E.ldw = (in_place && !rm) ? h_in[i] : r;  // A [r, h_in] as [k][n]; A [h_in, r] as [n][k]
-    E.pt_a = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_a);
-    E.pt_b = reinterpret_cast<uint16_t*>(ws + L.p[i].pt_b);
-    E.v2 = reinterpret_cast<const uint16_t*>(vv[i]);
+    E.pt_a = side_in_fold ? nullptr : side.pt_a[i];
+    E.pt_b = side_in_fold ? nullptr : side.pt_b[i];
+    E.v2 = side.v2[i];
     E.drop_bits = bits[i];
     E.drop_pitch = h_in[i] / 8;
     if (h_in[i] > widest) widest = h_in[i];

@@ -45,14 +45,24 @@ struct SelfPlanArgs {
 __device__ __attribute__((aligned(16))) uint32_t self_plan_zeros[4];
 
 // ---- finding a unit of work (UT tiles of one adapter) without a plan ------------------------
-template <int THREADS>
+// PAIRS: the kernels built for plans keyed by pairs of addresses (SMLM_KEY_PTR2).  They are kernels of their
+// own because what they add costs the others dearly: the arrays below triple the finder's LDS, and their
+// workgroups may take several units in turn (see shrink_self_planned_kernel), a loop around the whole body
+// that takes the tile-block kernel from 68 to 128 registers a lane.
+template <int N>
+struct FindPairs {
+  uint64_t ka[N], kb[N];  // the segments' pairs of addresses
+  int32_t first[N];       // the first segment with the same pair: the segment's id
+  int32_t slot[2][N];     // (scratch of first_equal_pair)
+};
+template <>
+struct FindPairs<0> {};
+template <int THREADS, bool PAIRS>
 struct FindLds {
   int32_t hist[kSelfPlanWeights];   // rows per adapter
   uint64_t wtab[kSelfPlanWeights];  // this projection's weight table
   int32_t rtab[kSelfPlanWeights];   // true ranks, when given
-  uint64_t ka[kSelfPlanWeights], kb[kSelfPlanWeights];  // SMLM_KEY_PTR2: the segments' pairs of addresses
-  int32_t first[kSelfPlanWeights];  //   and the first segment with the same pair: the segment's id
-  int32_t slot[2][kSelfPlanWeights];  //   (scratch of first_equal_pair)
+  FindPairs<PAIRS ? kSelfPlanWeights : 0> pr;
   uint32_t tot_a[THREADS / kWaveSize], tot_b[THREADS / kWaveSize];  // wave totals of the two scans
   int32_t rows[kBlkTiles * kTileRows], rseg[kBlkTiles * kTileRows];
   int32_t sel[3];                   // adapter of the unit (-1: no such unit), unit's index within the adapter, units in all
@@ -86,17 +96,16 @@ __device__ __forceinline__ uint32_t block_scan_excl_1(uint32_t v, uint32_t* tot,
 // Which adapter owns unit `unit` (a unit = UT consecutive tiles of one adapter; adapters in
 // ascending order, as the plan's groups are).  Everything global is requested at once; the
 // first barrier (LDS cleared) passes while those loads are on their way.  THREADS >= S.
-template <int THREADS, int UT>
-__device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const PlanSortArgs& pa,
+template <int THREADS, int UT, bool PAIRS>
+__device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS, PAIRS>& F, const PlanSortArgs& pa,
                                                   const void* const* w_ptrs, const int32_t* w_rank, int NA,
                                                   int unit, FindSeg* seg) {
   constexpr int kEnt = kSelfPlanWeights / THREADS;  // table entries a thread holds: kEnt * tid ...
   const int tid = threadIdx.x, lane = tid & 63;
   int key = -1, s0 = 0, len = 0;
-  const bool pairs = pa.key_kind == SMLM_KEY_PTR2;  // uniform over the launch
   uint64_t pair_a = 0, pair_b = 0;
   if (tid < pa.S) {
-    if (pairs) {
+    if constexpr (PAIRS) {
       pair_a = ((const SMLM_GLOBAL uint64_t*)pa.key)[tid];
       pair_b = ((const SMLM_GLOBAL uint64_t*)pa.key2)[tid];
     } else {
@@ -120,12 +129,12 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
   for (int e = 0; e < kEnt; ++e) F.hist[kEnt * tid + e] = 0;
   if (tid < UT * kTileRows) F.rows[tid] = -1, F.rseg[tid] = -1;
   if (tid == 0) F.sel[0] = -1;
-  if (pairs) {
+  if constexpr (PAIRS) {
     // groups by pairs of addresses: the id of a segment is the first segment with its pair, as the plan
     // builders number them (first_equal_pair; its barriers also cover the clearing above)
-    if (tid < pa.S) F.ka[tid] = pair_a, F.kb[tid] = pair_b;
-    first_equal_pair<kSelfPlanWeights>(F.ka, F.kb, F.first, F.slot[0], F.slot[1], pa.S);
-    if (tid < pa.S) key = F.first[tid];
+    if (tid < pa.S) F.pr.ka[tid] = pair_a, F.pr.kb[tid] = pair_b;
+    first_equal_pair<kSelfPlanWeights>(F.pr.ka, F.pr.kb, F.pr.first, F.pr.slot[0], F.pr.slot[1], pa.S);
+    if (tid < pa.S) key = F.pr.first[tid];
   } else {
     __syncthreads();
   }
@@ -187,8 +196,8 @@ __device__ __forceinline__ FoundUnit find_adapter(FindLds<THREADS>& F, const Pla
 
 // The rows of the unit, into F.rows / F.rseg (slot 16 w + c = row c of the unit's tile w; -1 =
 // empty): the adapter's rows in segment order, of which the unit holds 16 UT sub ... + 16 UT - 1.
-template <int THREADS, int UT>
-__device__ __forceinline__ void find_rows(FindLds<THREADS>& F, const FindSeg& seg, const FoundUnit& u) {
+template <int THREADS, int UT, bool PAIRS>
+__device__ __forceinline__ void find_rows(FindLds<THREADS, PAIRS>& F, const FindSeg& seg, const FoundUnit& u) {
   const int q_lo = u.sub * UT * kTileRows;
   const uint32_t mine = (seg.counted && seg.key == u.wid) ? (uint32_t)seg.len : 0u;
   uint32_t hi_u;
@@ -220,28 +229,28 @@ __device__ __forceinline__ void find_rows(FindLds<THREADS>& F, const FindSeg& se
 // each for itself -- the same sums as two workgroups of the 512-thread kind.
 // The sums' staging area lies behind the finder's LDS where both fit under the plan builders'
 // and over it otherwise.
-template <int NB, int THREADS>
+template <int NB, int THREADS, bool PAIRS>
 struct SelfPlanWork {
   static constexpr int kWaves = THREADS / kWaveSize;
-  static constexpr bool kOverlay = sizeof(FindLds<THREADS>) + sizeof(f32x4) * kWaves * NB * kWaveSize >
+  static constexpr bool kOverlay = sizeof(FindLds<THREADS, PAIRS>) + sizeof(f32x4) * kWaves * NB * kWaveSize >
                                    sizeof(PlanSmallLdsT<THREADS>);
-  FindLds<THREADS> find;
+  FindLds<THREADS, PAIRS> find;
   f32x4 red[kOverlay ? 1 : kWaves][NB][kWaveSize];
 };
-template <int NB, int THREADS>
+template <int NB, int THREADS, bool PAIRS>
 union SelfPlanLds {
   PlanSmallLdsT<THREADS> plan;                      // the plan-building workgroups
-  SelfPlanWork<NB, THREADS> work;                   // the others: finding their tile, then the cross-wave sums
+  SelfPlanWork<NB, THREADS, PAIRS> work;            // the others: finding their tile, then the cross-wave sums
   f32x4 red[THREADS / kWaveSize][NB][kWaveSize];    // ... which reuse the finder's memory when the two do not fit side by side
 };
 
-template <int DT, int NB, int U, int THREADS>
+template <int DT, int NB, int U, int THREADS, bool PAIRS = false>
 __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanArgs a) {
   static_assert(THREADS == kSelfPlanThreads || THREADS == 2 * kSelfPlanThreads, "one or two groups of eight waves");
-  __shared__ SelfPlanLds<NB, THREADS> sm;
+  __shared__ SelfPlanLds<NB, THREADS, PAIRS> sm;
   constexpr int NW = kSelfPlanThreads / kWaveSize;  // waves that sum one k slice
   constexpr int HALVES = THREADS / kSelfPlanThreads;
-  constexpr bool kOverlay = SelfPlanWork<NB, THREADS>::kOverlay;
+  constexpr bool kOverlay = SelfPlanWork<NB, THREADS, PAIRS>::kOverlay;
   const int tid = threadIdx.x;
   if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
     const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
@@ -253,7 +262,7 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
   const int pj = blockIdx.z;
   if ((int)blockIdx.x * HALVES >= a.sh.items.row_start[pj + 1] - a.sh.items.row_start[pj]) return;
   const ShrinkProj P = a.sh.p[pj];
-  FindLds<THREADS>& F = sm.work.find;
+  FindLds<THREADS, PAIRS>& F = sm.work.find;
   const int wave_all = tid >> 6, lane = tid & 63;
   const int wave = wave_all % NW;           // wave within its group of eight
   const int yy = (int)blockIdx.x * HALVES + wave_all / NW;
@@ -264,13 +273,14 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
   const int kend = min(kbeg + P.k_per_wave, P.d_in);
   const uint16_t* zeros = reinterpret_cast<const uint16_t*>(self_plan_zeros);
 
-  // The launch has a row of workgroups for every tile the batch usually has (its rows in whole tiles plus a
-  // few dozen part-filled ones: a tile per adapter in use), not for every tile it could have (one more per
-  // table entry): a batch with more tiles than rows of workgroups sends them round again.
+  // PAIRS: the table has an entry per segment, and a row of workgroups for every tile the batch could have
+  // (one more per table entry) would be mostly idle ones.  The launch has a row for every tile such a batch
+  // usually has -- its rows in whole tiles plus a few dozen part-filled ones -- and a batch with more tiles
+  // sends its workgroups round again.  The other kind has a row per possible tile and takes one turn.
   for (int tile = blockIdx.y;; tile += a.units) {
   FindSeg seg;
   const FoundUnit un =
-      find_adapter<THREADS, 1>(F, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tile, &seg);
+      find_adapter<THREADS, 1, PAIRS>(F, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tile, &seg);
   const int wid = un.wid;
   if (wid < 0) return;  // past the last tile; uniform over the workgroup
   const uint16_t* W = reinterpret_cast<const uint16_t*>(F.wtab[wid]);
@@ -294,7 +304,7 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
   u32x4 wf[NB][U];
   load_w(kbeg, wf);
 
-  find_rows<THREADS, 1>(F, seg, un);
+  find_rows<THREADS, 1, PAIRS>(F, seg, un);
   const int row = F.rows[c], rseg = F.rseg[c];
   if (kOverlay) __syncthreads();  // every wave holds its tile: the finder's LDS turns into the sum's staging area
 
@@ -344,7 +354,7 @@ __global__ __launch_bounds__(THREADS) void shrink_self_planned_kernel(SelfPlanAr
         store4<DT>(P.out + (long)row * P.d_out + n, sum, scale, a.sh.beta);
     }
   }
-  if (tile + a.units >= un.total) return;  // uniform over the workgroup: no tile is left for it
+  if (!PAIRS || tile + a.units >= un.total) return;  // uniform over the workgroup: no tile is left for it
   __syncthreads();                         // the sums are read: the finder takes its LDS back
   }
 }
@@ -362,14 +372,14 @@ struct SelfPlanBlockStage {
   static constexpr int kPitch = WKN ? 16 * NB + 8 : 32 * U + 8;
   uint16_t wlds[GROUPS][2][(WKN ? 32 * U : 16 * NB) * kPitch];
 };
-template <int NB, int U, bool WKN, int THREADS>
+template <int NB, int U, bool WKN, int THREADS, bool PAIRS>
 union SelfPlanBlockLds {
   PlanSmallLdsT<THREADS> plan;                                  // the plan-building workgroups
-  FindLds<THREADS> find;                                        // the others: first while they find their tile block ...
+  FindLds<THREADS, PAIRS> find;                                 // the others: first while they find their tile block ...
   SelfPlanBlockStage<NB, U, WKN, THREADS / kFwdThreads> stage;  // ... then the staged weight batches
 };
 
-template <int DT, int NB, int U, bool WKN, int THREADS>
+template <int DT, int NB, int U, bool WKN, int THREADS, bool PAIRS = false>
 __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(SelfPlanArgs a) {
   static_assert(THREADS == kFwdThreads || THREADS == 2 * kFwdThreads, "one or two groups of four waves");
   constexpr int GROUPS = THREADS / kFwdThreads;
@@ -378,7 +388,7 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
   constexpr int kPitch = SelfPlanBlockStage<NB, U, WKN, GROUPS>::kPitch;
   constexpr int kPieces = kRowsW * (KB / 8); // 16-byte pieces of one staged batch
   constexpr int kPer = (kPieces + kFwdThreads - 1) / kFwdThreads;
-  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U, WKN, THREADS> sm;
+  __shared__ __attribute__((aligned(16))) SelfPlanBlockLds<NB, U, WKN, THREADS, PAIRS> sm;
   if ((int)blockIdx.y == a.units) {  // the extra row of the grid: up to kSelfPlanBuilders workgroups build the plan
     const int part = (int)(blockIdx.z * gridDim.x + blockIdx.x), all = (int)(gridDim.x * gridDim.z);
     if (part < kSelfPlanBuilders) plan_small_body(a.plan, sm.plan, part, all < kSelfPlanBuilders ? all : kSelfPlanBuilders);
@@ -400,12 +410,12 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
   const int kend = min(kbeg + kFwdWaves * P.k_per_wave, P.d_in);
   const int kstop = GROUPS > 1 ? kbeg + kFwdWaves * P.k_per_wave : kend;  // the same number of batches for both groups
 
-  // (a row of workgroups for every tile block the batch usually has; the others go round again, as in
+  // (PAIRS: a row of workgroups for every tile block the batch usually has; the others go round again, as in
   // shrink_self_planned_kernel)
   for (int tb = blockIdx.y;; tb += a.units) {
   FindSeg seg;
   const FoundUnit un =
-      find_adapter<THREADS, kBlkTiles>(sm.find, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tb, &seg);
+      find_adapter<THREADS, kBlkTiles, PAIRS>(sm.find, a.plan, P.w_ptrs, a.sh.plan.w_rank, a.n_weights, tb, &seg);
   if (un.wid < 0) return;  // past the last tile block; uniform over the workgroup
   const uint16_t* W = reinterpret_cast<const uint16_t*>(sm.find.wtab[un.wid]);
   int nlim = P.d_out;  // weight rows at or past it are zero padding
@@ -450,7 +460,7 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
   u32x4 wst[kPer];
   load_w(kbeg, wst);
 
-  find_rows<THREADS, kBlkTiles>(sm.find, seg, un);
+  find_rows<THREADS, kBlkTiles, PAIRS>(sm.find, seg, un);
   const bool active = wave < un.tiles;
   const int row = active ? sm.find.rows[wave * kTileRows + c] : -1;
   const int rseg = active ? sm.find.rseg[wave * kTileRows + c] : -1;
@@ -506,7 +516,7 @@ __global__ __launch_bounds__(THREADS) void shrink_block_self_planned_kernel(Self
         store4<DT>(P.out + (long)row * P.d_out + n, acc[nb], scale, a.sh.beta);
     }
   }
-  if (tb + a.units >= un.total) return;  // uniform over the workgroup: no tile block is left for it
+  if (!PAIRS || tb + a.units >= un.total) return;  // uniform over the workgroup: no tile block is left for it
   __syncthreads();                       // the staged weights are read: the finder takes its LDS back
   }
 }

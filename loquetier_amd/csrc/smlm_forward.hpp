@@ -467,6 +467,11 @@ struct ReduceProj {
   const float* partial;  // [ksplit, T, d_out]
   uint16_t* out;         // [T, d_out]
   int ksplit;            // 1: nothing to fold for this projection
+  // SIDE folds (the backward's dV): side_scale * out by tile slot, transposed ([d_out][side_pitch]), and the
+  // same treatment of v2 (a second [T, d_out] matrix) -- what the weight-gradient kernel reads
+  uint16_t* pt_a;
+  uint16_t* pt_b;
+  const uint16_t* v2;
 };
 
 struct ReduceArgs {
@@ -476,12 +481,16 @@ struct ReduceArgs {
   float beta;
   int T, d_out, nproj;
   int units_max;  // > 0: direct mode, one (projection, tile) per workgroup over this tile bound
+  const float* side_scale;  // SIDE folds: per segment, or null for 1
+  long side_pitch;          // SIDE folds: slots per row of pt_a / pt_b
 };
 
 // Folds the k-split partial sums of a shrink launch, in split order, into the
 // 16-bit result (the reference's "v in the I/O dtype"): work item -> (projection,
 // tile), 16 threads per row.
-template <int DT>
+// SIDE: the fold of the backward's dV, which also leaves the by-products of write_side (further down)
+// behind -- the rounded sums and v2, scaled, by tile slot and transposed; slots without a row get zeros.
+template <int DT, bool SIDE = false>
 __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
   const int units = tile_units<1>(a.plan, a.units_max);
   const int c = threadIdx.x >> 4, q = threadIdx.x & 15;
@@ -491,9 +500,10 @@ __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
     const ReduceProj P = a.p[pj];
     if (P.ksplit <= 1) continue;
     if (!wid_ok(a.plan, uload(a.plan.tile_wid, tile))) continue;  // past the last tile (direct mode), or no such adapter
-    const int row = a.plan.tile_row[tile * kTileRows + c];
-    if (row < 0) continue;
-    const float scale = a.seg_scale ? a.seg_scale[a.plan.tile_rseg[tile * kTileRows + c]] : 1.0f;
+    const int slot = tile * kTileRows + c;
+    const int row = a.plan.tile_row[slot];
+    if (!SIDE && row < 0) continue;
+    const float scale = (a.seg_scale && row >= 0) ? a.seg_scale[a.plan.tile_rseg[slot]] : 1.0f;
     const float* zf = reinterpret_cast<const float*>(a.plan.hdr + kHdrZeros);
     for (int n = 4 * q; n < a.d_out; n += 64) {
       // all partials are requested before the first add waits for one; past ksplit the loads
@@ -501,11 +511,27 @@ __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
       f32x4 part[kMaxKsplit];
 #pragma unroll
       for (int z = 0; z < kMaxKsplit; ++z)
-        part[z] = ldg_f4(z < P.ksplit ? P.partial + ((long)z * a.T + row) * a.d_out + n : zf);
+        part[z] = ldg_f4((z < P.ksplit && row >= 0) ? P.partial + ((long)z * a.T + row) * a.d_out + n : zf);
+      u32x2 second = {0u, 0u};
+      if (SIDE && P.pt_b && row >= 0) second = *reinterpret_cast<const u32x2*>(P.v2 + (long)row * a.d_out + n);
       f32x4 sum = part[0];
 #pragma unroll
       for (int z = 1; z < kMaxKsplit; ++z) sum += part[z];
-      store4<DT>(P.out + (long)row * a.d_out + n, sum, scale, a.beta);
+      if (row >= 0) store4<DT>(P.out + (long)row * a.d_out + n, sum, scale, a.beta);
+      if (SIDE) {
+        const float ss = (a.side_scale && row >= 0) ? a.side_scale[a.plan.tile_rseg[slot]] : 1.0f;
+        // (from the rounded value, as a reader of `out` would scale it)
+        const u32x2 first = {pack2<DT>(scale * sum[0], scale * sum[1]), pack2<DT>(scale * sum[2], scale * sum[3])};
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          P.pt_a[(n + 2 * e) * a.side_pitch + slot] = (uint16_t)Num<DT>::bits(ss * Num<DT>::lo(first[e]));
+          P.pt_a[(n + 2 * e + 1) * a.side_pitch + slot] = (uint16_t)Num<DT>::bits(ss * Num<DT>::hi(first[e]));
+          if (P.pt_b) {
+            P.pt_b[(n + 2 * e) * a.side_pitch + slot] = (uint16_t)Num<DT>::bits(ss * Num<DT>::lo(second[e]));
+            P.pt_b[(n + 2 * e + 1) * a.side_pitch + slot] = (uint16_t)Num<DT>::bits(ss * Num<DT>::hi(second[e]));
+          }
+        }
+      }
     }
   }
 }

@@ -202,3 +202,67 @@ def test_checked_call_cache_changes_nothing(K, oracle, gpu_device):
     with pytest.raises(RuntimeError):
         K.smlm_lora_forward_multi([y[:-16] for y in ys[0]], [p["xd"] for p in projs], [p["a_tab"] for p in projs],
                                   [p["b_tab"] for p in projs], plan, r, cache=cache)
+
+
+SIDE_CASES = [
+    ("q-o-wide", [0, 600, 1100], [1, 0], 2, [(512, 2048), (2048, 2048)], 16),
+    ("mlp-rank64", [0, 300, 700, 1300], [1, 0, 2], 3, [(512, 2816), (512, 2816), (2816, 512)], 64),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+@pytest.mark.parametrize("case", SIDE_CASES, ids=[c[0] for c in SIDE_CASES])
+def test_fold_writes_what_the_weight_gradients_read(K, oracle, gpu_device, case, dt):
+    """Wide outputs: the dV product of every projection is folded from k-split partials and the fold leaves the
+    scaled, transposed dV and v behind for the weight-gradient launch (narrow outputs leave that to dX's
+    launch: the cases further up).  Values against the oracle, staged calls and a captured call replayed with
+    new inputs against the call in one piece, bit for bit."""
+    name, tp, part_ad, NA, dims, r = case
+    d, n_rows = gpu_device, tp[-1]
+    projs, pi, pa = _setup(oracle, d, case, dt, dy=False)
+    scales = [0.5, 2.0, 1.0][: len(part_ad)]   # (powers of two: scaled values are the unscaled ones' exact multiples)
+    scale = torch.tensor(scales, device=d)
+    vs = []
+    for p in projs:
+        _, vo = oracle.add_lora_forward(p["x"], [p["A"][a] for a in part_ad], [p["B"][a] for a in part_ad],
+                                        tp, p["g"].shape[1], dt)
+        vs.append(dev_t(vo, dt, d))
+    plan = K.SegmentPlan(pi, pa, n_rows)
+    whole, staged = _outputs(projs, d, dt, n_rows), _outputs(projs, d, dt, n_rows)
+    _multi(K, projs, whole, plan, r, vs=vs, scale=scale)
+    for st in (1, 2, 4):   # SMLM_BWD_PRODUCTS, _DX, _WGRAD
+        _multi(K, projs, staged, plan, r, vs=vs, scale=scale, stages=st)
+
+    def same(got, want, what):
+        for i, (m, s) in enumerate(zip(got, want)):
+            assert torch.equal(m["dx"], s["dx"]), (what, i)
+            for a in range(NA):
+                assert torch.equal(m["dA"][a], s["dA"][a]) and torch.equal(m["dB"][a], s["dB"][a]), (what, i, a)
+    same(staged, whole, "staged")
+    for i, (p, m) in enumerate(zip(projs, whole)):
+        gx, ga, gb = oracle.add_lora_backward(p["g"], p["x"], p["A"], p["B"], tp, part_ad, dt)
+        for q, a in enumerate(part_ad):   # (every adapter trains one partition here)
+            close(to_np(m["dA"][a]), scales[q] * ga[a], atol=ATOL * max(1.0, float(np.abs(scales[q] * ga[a]).max())))
+            close(to_np(m["dB"][a]), scales[q] * gb[a], atol=ATOL * max(1.0, float(np.abs(scales[q] * gb[a]).max())))
+
+    cap = torch.cuda.Stream()
+    static = _outputs(projs, d, dt, n_rows)
+    with torch.cuda.stream(cap):
+        _multi(K, projs, static, plan, r, vs=vs, scale=scale)   # (sizes the workspace of this stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=cap):
+        _multi(K, projs, static, plan, r, vs=vs, scale=scale)
+    for k in range(3):
+        for p in projs:
+            p["gd"].copy_(p["gd"] * 0.5 + k)
+        for o in static:
+            o["dx"].fill_(7.0)
+            for t in o["dA"] + o["dB"]:
+                t.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        eager = _outputs(projs, d, dt, n_rows)
+        _multi(K, projs, eager, plan, r, vs=vs, scale=scale)
+        torch.cuda.synchronize()
+        same(static, eager, f"replay {k}")
