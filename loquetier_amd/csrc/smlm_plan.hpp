@@ -162,7 +162,8 @@ __device__ __forceinline__ int usable_kind(const void* key, int key_kind, int S,
 // IN_LDS: the keys lie in LDS.  A stage of stride <= 64 then keeps every wave inside the 128 keys it already
 // owns (pair i of a wave's 64 pairs lies in keys [128 w, 128 w + 128), in every pass of the loop over i), and
 // a wave's LDS accesses complete in order: between two such stages the waves need not meet, which takes the
-// barriers of 56 of the 66 stages of a 2048-key sort away (1075 segments: 27 -> see the plan launch's time).
+// barriers of 56 of the 66 stages of a 2048-key sort away (1075 segments: the launch 27.1 -> 25.6 us; placing every
+// key by counting the keys below it instead, all lanes reading one LDS address at a time: 38.5 us).
 template <bool IN_LDS = false, typename KeyArray>
 __device__ __forceinline__ void bitonic_sort(KeyArray K, int N) {
   bool own = false;  // the stage before this one was one of those
