@@ -324,16 +324,20 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
           qf[ks][nb] = u32x4{q0[0], q0[1], q1[0], q1[1]};
         }
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+      for (int jb = 0; jb < NBJ; ++jb) {
+        // rank blocks past the adapter's own rank would multiply the zeros their operand was given: their sums
+        // stay the zeros they start as (uniform over the workgroup)
+        if (NBJ > 1 && j0 + 16 * jb >= rlim) continue;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
+        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-          for (int jb = 0; jb < NBJ; ++jb) {
+          for (int nb = 0; nb < 4; ++nb) {
             // dA: rows = columns of x, cols = rank -> lane holds 4 consecutive x columns of rank c
             // dB: rows = rank, cols = columns of dY -> lane holds 4 consecutive ranks of column c
             acc[jb][nb] = is_a ? Num<DT>::mfma(qf[ks][nb], pf[jb][ks], acc[jb][nb])
                                : Num<DT>::mfma(pf[jb][ks], qf[ks][nb], acc[jb][nb]);
           }
+      }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       // the token-side operand of the next step, into the registers the multiplies above are done with (it
@@ -377,6 +381,7 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
       // columns 16nb + 4g .. +3
 #pragma unroll
       for (int jb = 0; jb < NBJ; ++jb) {
+        if (NBJ > 1 && a.packed && j0 + 16 * jb >= rlim) continue;  // rows the packed gradient does not have
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) *reinterpret_cast<f32x4*>(&sto[c * kSPitch + 16 * nb + 4 * g]) = acc[jb][nb];
         wave_sync();
