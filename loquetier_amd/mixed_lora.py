@@ -244,26 +244,26 @@ def prepare_weight(weight: torch.Tensor, rank: int, dtype: torch.dtype, device, 
 class fused_add_lora(Function):
     """result <- result + scale_seg * (x A_seg^T) B_seg^T, in place, one call.
 
-    Arguments: (result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-    train_len, train_partition, dropout, adapter_rank, step, *weights); the tables
-    hold one address per adapter and the plan is keyed by adapter id.  `adapter_rank`
-    (None, or a pair of int32 device tensors: the true rank of every adapter, and
-    of the training adapters in order of first appearance among the partitions)
-    tells the kernels which adapters are stored zero-padded.  `dropout` (a
-    kernel.DropoutSpec or None) drops the training rows of x inside the kernels,
-    in place of the reference's nn.Dropout calls and torch.cat before the op
-    (src/loquetier_src/models/mixed_lora.py:185-192); x is the tensor before
-    dropout.  `step` (None, or a LayerStep) carries what the step's context and the
-    layer have prepared once: scratch memory, the backward's plan and pointer tables.
-    Returns `result`.
+    Arguments: (result, x, call, *weights).  `call` (a LayerStep) names everything that is not
+    differentiated, so that autograd has three arguments to look at besides the weights: the tables
+    (one address per adapter; the plan is keyed by adapter id), the per-segment scale, the plan, the
+    rank, the training rows and partitions, `adapter_rank` (None, or a pair of int32 device tensors:
+    the true rank of every adapter, and of the training adapters in order of first appearance among
+    the partitions; tells the kernels which adapters are stored zero-padded), `dropout` (a
+    kernel.DropoutSpec or None: drops the training rows of x inside the kernels, in place of the
+    reference's nn.Dropout calls and torch.cat before the op,
+    src/loquetier_src/models/mixed_lora.py:185-192; x is the tensor before dropout), and what the
+    step's context and the layer have prepared once: scratch memory, the backward's plan and pointer
+    tables.  Returns `result`.
     Gradients: result -> passed through, x -> dX on train rows (zero elsewhere),
     each trainable weight -> its summed gradient (None when not training)."""
 
     @staticmethod
-    def forward(ctx: FunctionCtx, result, x, wa_table, wb_table, seg_scale, plan, lora_rank,
-                train_len, train_partition, dropout, adapter_rank, step, *weights):
+    def forward(ctx: FunctionCtx, result, x, step, *weights):
+        wa_table, wb_table, seg_scale, plan, lora_rank = step.wa_table, step.wb_table, step.seg_scale, step.plan, step.rank
+        train_len, train_partition, dropout = step.train_len, step.train_partition, step.dropout
         need_v = len(weights) > 0 and train_len > 0
-        adapter_rank, train_rank = adapter_rank if adapter_rank is not None else (None, None)
+        adapter_rank, train_rank = step.adapter_rank if step.adapter_rank is not None else (None, None)
         v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device) if need_v else None
         if dropout is not None and need_v and dropout.mask_bits is None:
             # the backward reads the forward's keep bits (1/16 of x's bytes) instead of making them again
@@ -272,9 +272,7 @@ class fused_add_lora(Function):
             dropout = kernel.DropoutSpec(dropout.seg_p, dropout.rows, dropout.seed, dropout.offset, bits)
         kernel.smlm_lora_forward(result, x, wa_table, wb_table, plan, lora_rank, seg_scale=seg_scale,
                                  beta=1.0, v_out=v, dropout=dropout, adapter_rank=adapter_rank,
-                                 workspace=None if step is None else step.workspace,
-                                 packed_ranks=step is not None and step.packed,
-                                 cache=None if step is None else step.cache)
+                                 workspace=step.workspace, packed_ranks=step.packed, cache=step.cache)
         ctx.mark_dirty(result)
         ctx.tp = train_partition
         ctx.rank = lora_rank
@@ -287,14 +285,14 @@ class fused_add_lora(Function):
         ctx.part_drop = None
         ctx.train_rank = train_rank if need_v else None
         if need_v and (seg_scale is not None or dropout is not None):
-            if step is not None:
-                seg_of = step.part_segments
-            else:
+            seg_of = step.part_segments
+            if seg_of is None:
                 starts = torch.tensor([int(t) for t in train_partition][: ctx.n_parts],
                                       dtype=torch.int32, device=x.device)
                 seg_of = (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, plan.S - 1)
-            # (gathers of one step's tensors are shared by the layers that use the same tensors)
-            gather = (lambda t: step.gather(t, seg_of)) if step is not None else (lambda t: t[seg_of].contiguous())
+                gather = lambda t: t[seg_of].contiguous()
+            else:  # (gathers of one step's tensors are shared by the layers that use the same tensors)
+                gather = lambda t: step.gather(t, seg_of)
             if seg_scale is not None:
                 ctx.part_scale = gather(seg_scale)
             if dropout is not None:  # the same stream, probabilities by train partition
@@ -306,7 +304,7 @@ class fused_add_lora(Function):
 
     @staticmethod
     def backward(ctx: FunctionCtx, grad_output: torch.Tensor):
-        n_fixed = 12
+        n_fixed = 3
         if not ctx.has_v:
             return (grad_output, None) + (None,) * (n_fixed - 2) + (None,) * (2 * ctx.n_parts)
         x, v, *weight_list = ctx.saved_tensors
@@ -316,24 +314,33 @@ class fused_add_lora(Function):
         return (grad_output, grad_x) + (None,) * (n_fixed - 2) + tuple(grads)
 
 
-@dataclass
 class LayerStep:
-    """What one layer call hands to the operator besides tensors: prepared once per step by the
-    context (shared by all layers) or once per adapter set by the layer, never inside the call."""
-    workspace: Any                      # kernel.Workspace owned by the context
-    part_segments: Optional[torch.Tensor] = None   # segment that starts every train partition
-    bwd_plan: Optional[Any] = None      # kernel.SegmentPlan over the train partitions
-    part_adapter: Optional[List[int]] = None       # training-adapter index of every partition
-    a_tab: Optional[torch.Tensor] = None           # addresses of the training adapters' A / B, in order
-    b_tab: Optional[torch.Tensor] = None
-    # where the gradients go (MixedLoraLinear._train_tables): byte offsets of dA_0.., dB_0.. inside one buffer
-    # (grad_offsets) or inside one buffer for the dA and one for the dB (grad_offsets_a / _b, when the matrices
-    # have one shape: grad_uniform), [(offset in elements, shape)] in the same order (grad_shapes, grad_numel),
-    # and the device tables of the gradients' addresses by buffer address (grad_tabs)
-    grad_layout: Optional[dict] = None
-    memo: Any = None                               # the context's per-step memo (MixedLoraContext.memo)
-    packed: bool = False                           # the adapters are stored at their true ranks
-    cache: Optional[dict] = None                   # the layer's checked operator calls (kernel.smlm_lora_forward_multi)
+    """What one layer call hands to the operator besides the tensors it differentiates: the call's own
+    arguments, and what was prepared once per step by the context (shared by all layers) or once per
+    adapter set by the layer, never inside the call."""
+    __slots__ = ("workspace", "memo", "packed", "cache", "wa_table", "wb_table", "seg_scale", "plan", "rank",
+                 "train_len", "train_partition", "dropout", "adapter_rank", "part_segments", "bwd_plan",
+                 "part_adapter", "a_tab", "b_tab", "grad_layout")
+
+    def __init__(self, workspace, memo=None, packed=False, cache=None):
+        self.workspace = workspace      # kernel.Workspace owned by the context
+        self.memo = memo                # the context's per-step memo (MixedLoraContext.memo)
+        self.packed = packed            # the adapters are stored at their true ranks
+        self.cache = cache              # the layer's checked operator calls (kernel.smlm_lora_forward_multi)
+        # the call: pointer tables by adapter, per-segment scale, plan, rank, training rows and partitions,
+        # dropout descriptor, (ranks of all adapters, ranks of the training adapters) or None
+        self.wa_table = self.wb_table = self.seg_scale = self.plan = self.dropout = self.adapter_rank = None
+        self.rank = self.train_len = 0
+        self.train_partition = ()
+        self.part_segments = None       # segment that starts every train partition
+        self.bwd_plan = None            # kernel.SegmentPlan over the train partitions
+        self.part_adapter = None        # training-adapter index of every partition
+        self.a_tab = self.b_tab = None  # addresses of the training adapters' A / B, in order
+        # where the gradients go (MixedLoraLinear._train_tables): byte offsets of dA_0.., dB_0.. inside one buffer
+        # (grad_offsets) or inside one buffer for the dA and one for the dB (grad_offsets_a / _b, when the matrices
+        # have one shape: grad_uniform), [(offset in elements, shape)] in the same order (grad_shapes, grad_numel),
+        # and the device tables of the gradients' addresses by buffer address (grad_tabs)
+        self.grad_layout = None
 
     def gather(self, table: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
         """table[index], computed once per step for a given pair of tensors."""
@@ -625,7 +632,8 @@ class MixedLoraLinear(nn.Module):
         train_idx = ctx.train_idx
 
         x_arg = x  # the tensor the caller handed over (a projection group recognises its input by it)
-        x = x.to(self.dtype)
+        if x.dtype != self.dtype:
+            x = x.to(self.dtype)
         drop_spec = None
         if blen.tlen > 0 and self.fused:
             # the kernels drop the training rows themselves: no dropped copy, no torch.cat
@@ -650,17 +658,21 @@ class MixedLoraLinear(nn.Module):
                 # (layers whose adapters have the same scales share one gather per step)
                 seg_scale = ctx.memo(("seg_scale", self._scaling_key, self.device),
                                      lambda: self._scaling_f32[ctx.seg_adapter_long(self.device)])
-            result = result.to(self.dtype).contiguous()
+            if result.dtype != self.dtype:
+                result = result.to(self.dtype)
+            if not result.is_contiguous():
+                result = result.contiguous()
             if not x.is_contiguous():
                 x = x.contiguous()
+            same_dtype = result.dtype == torch_result_dtype
             ctx.check_adapter_ids(len(self.adapters))
             plan = ctx.plan(self.device, x.size(0))
             if self._group is not None and not self._group[0].suspended and blen.tlen == 0 and not weights and not (
                     torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):
                 # a serving step: the group's members share one shrink launch
                 self._group[0].expand_member(self._group[1], result, x, seg_scale, plan,
-                                             may_defer=result.dtype == torch_result_dtype, src=x_arg)
-                return result.to(torch_result_dtype)
+                                             may_defer=same_dtype, src=x_arg)
+                return result if same_dtype else result.to(torch_result_dtype)
             if not weights and drop_spec is None and not (
                     torch.is_grad_enabled() and (x.requires_grad or result.requires_grad)):
                 # nothing to differentiate: the operator is called directly, without autograd's bookkeeping
@@ -668,19 +680,20 @@ class MixedLoraLinear(nn.Module):
                                          seg_scale=seg_scale, beta=1.0, adapter_rank=self.adapter_rank,
                                          workspace=ctx.workspace(self.device), packed_ranks=self.packed,
                                          cache=self._call_cache)
-                return result.to(torch_result_dtype)
-            step = LayerStep(workspace=ctx.workspace(self.device), memo=ctx.memo, packed=self.packed,
-                             cache=self._call_cache)
+                return result if same_dtype else result.to(torch_result_dtype)
+            step = LayerStep(ctx.workspace(self.device), ctx.memo, self.packed, self._call_cache)
+            step.wa_table, step.wb_table, step.seg_scale, step.plan, step.rank = \
+                self.wa_ptrs, self.wb_ptrs, seg_scale, plan, self.rank
+            step.train_len, step.train_partition, step.dropout = blen.tlen, blen.train_partition, drop_spec
+            step.adapter_rank = self._rank_args(train_idx)
             if weights and blen.tlen > 0:
                 step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
                 step.part_segments = ctx.part_segments(self.device, plan)
                 tabs = self._train_tables(ctx.train_order())
                 step.a_tab, step.b_tab = tabs["a_tab"], tabs["b_tab"]
                 step.grad_layout = tabs
-            result = fused_add_lora.apply(result, x, self.wa_ptrs, self.wb_ptrs, seg_scale, plan, self.rank,
-                                          blen.tlen, blen.train_partition, drop_spec,
-                                          self._rank_args(train_idx), step, *weights)
-            return result.to(torch_result_dtype)
+            result = fused_add_lora.apply(result, x, step, *weights)
+            return result if same_dtype else result.to(torch_result_dtype)
 
         segment = ctx.segment.to(self.device)
         wa_ptr, wb_ptr = self.wa_ptrs[lora_ids], self.wb_ptrs[lora_ids]
