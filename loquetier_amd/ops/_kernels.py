@@ -51,9 +51,15 @@ class Workspace:
 _WORKSPACES: Dict[Tuple[int, int], Workspace] = {}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(dev: torch.device) -> int:
-    # (the handle itself: building a torch.cuda.Stream object around it costs microseconds per call)
-    return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch.cuda.current_device())
+    # (the handle itself where torch hands it out: building a torch.cuda.Stream object around it costs
+    # microseconds per call)
+    if _raw_stream is None:
+        return torch.cuda.current_stream(dev).cuda_stream
+    return _raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
 
 
 class _NoSwitch:
