@@ -1274,8 +1274,10 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   wa.packed = packed;
   wa.drop = drop;  // dA against the dropped x
   // ranks above 64 are covered 64 at a time along the grid's z axis
-  dim3 grid(units, NA, ceil_div(r, 64));
   const int nbj = r > 64 ? 4 : ceil_div(r, 16);
+  // (along z: 64 ranks a workgroup, or what a dA workgroup of the launched kernel takes when that is less)
+  const int z_per_64 = nbj / wgrad_nbj_a(nbj, split ? 4 : 1, drop.seg_p != nullptr);
+  dim3 grid(units, NA, ceil_div(r, 64) * z_per_64);
   return dtype == SMLM_DTYPE_F16 ? launch_wgrad<SMLM_DTYPE_F16>(nbj, split, grid, st, wa)
                                  : launch_wgrad<SMLM_DTYPE_BF16>(nbj, split, grid, st, wa);
 }

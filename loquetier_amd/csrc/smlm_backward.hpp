@@ -124,7 +124,8 @@ __device__ __forceinline__ int wg_lds_row(int s) {
   return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1);
 }
 
-// grid: (sum over the projections of their dA and dB units, NA, ceil(r/64)), block 64*NW; a unit is
+// grid: (sum over the projections of their dA and dB units, NA, ceil(r/64) -- twice that for the kernel named at
+// wgrad_nbj_a), block 64*NW; a unit is
 // `walk` neighbouring 64-column chunks of one projection's dA or dB.  A workgroup owns the unit's columns (and
 // up to 64 ranks) of one adapter's gradient and walks all of that adapter's tiles once per chunk, 64
 // gathered rows (four tiles, two MFMA k steps) per wave and loop step.  With
@@ -146,13 +147,13 @@ __device__ __forceinline__ int wg_lds_row(int s) {
 // once from the group's first segment.
 template <int DT, int NBJ, int NW, bool IS_A, bool DROP = false>
 __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& P, int chunk_first, int n_chunks,
-                                           char* smem) {
+                                           int j0, char* smem) {
   constexpr int kWgWaves = NW;
   constexpr int kStageElems = kWgSlots * kWgPitch;
   constexpr int kRedBytes = NW > 1 ? NW * 4 * kWaveSize * 16 : 0;
 
   const int ad = blockIdx.y;
-  const int j0 = 64 * blockIdx.z;  // first rank of this workgroup (ranks above 64: 64 per z)
+  // j0: first rank of this workgroup (16 * NBJ ranks per workgroup along the grid's z axis)
   constexpr bool is_a = IS_A;
   const int h = is_a ? P.h_in : P.h_out;
   const uint16_t* Q = is_a ? P.q_a : P.q_b;
@@ -418,6 +419,9 @@ __device__ __forceinline__ void wgrad_body(const WgradArgs& a, const WgradProj& 
   }
 }
 
+// rank blocks of 16 a dA workgroup takes (a dB workgroup: NBJ)
+constexpr int wgrad_nbj_a(int nbj, int nw, bool drop) { return (drop && nw == 1 && nbj == 4) ? 2 : nbj; }
+
 template <int DT, int NBJ, int NW, bool DROP = false>
 // (two waves a SIMD at every rank: the one-wave kernels hide their latencies through occupancy)
 __global__ __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(2))) void wgrad_kernel(WgradArgs a) {
@@ -430,13 +434,18 @@ __global__ __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(
   const WgradProj& P = a.p[pj];
   const int unit = (int)blockIdx.x - P.unit0;
   const int walk = NW > 1 ? 1 : a.walk;
+  // The one-wave kernel that applies dropout to 64 ranks at a time does not fit the registers of a lane
+  // (200 bytes of spills, and twice the time of the kernel without dropout): its dA workgroups take 32 ranks
+  // each, two along z where the others have one; dB, which no dropout touches, keeps 64.
+  constexpr int NBJ_A = wgrad_nbj_a(NBJ, NW, DROP), ZA = NBJ / NBJ_A;
   if (unit < P.units_a) {  // uniform over the workgroup
     const int first = unit * walk, left = P.chunks_a - first;
-    wgrad_body<DT, NBJ, NW, true, DROP>(a, P, first, left < walk ? left : walk, smem);
+    wgrad_body<DT, NBJ_A, NW, true, DROP>(a, P, first, left < walk ? left : walk, 16 * NBJ_A * (int)blockIdx.z, smem);
   } else {
+    if (blockIdx.z % ZA) return;
     const int chunks_b = (P.h_out + kWgCols - 1) / kWgCols;
     const int first = (unit - P.units_a) * walk, left = chunks_b - first;
-    wgrad_body<DT, NBJ, NW, false>(a, P, first, left < walk ? left : walk, smem);
+    wgrad_body<DT, NBJ, NW, false>(a, P, first, left < walk ? left : walk, 16 * NBJ * (int)(blockIdx.z / ZA), smem);
   }
 }
 
