@@ -20,6 +20,12 @@ CASES = [
     ("tile-blocks", [0, 700, 1100, 1101, 1500, 2300], [0, 1, 0, 1, 0], [2, 1, 2, 0, 2], 512, 320, 64),
     ("600-segments", list(range(0, 1200, 2)) + [1200], [(i * 7) % 11 for i in range(600)], [(i * 3) % 4 for i in range(600)],
      2048, 128, 16),
+    # more tiles (tile blocks) than the launch has rows of workgroups -- a table entry per segment, so the launch
+    # is sized for the usual batch (rows / 16 + 33 tiles): its workgroups go round again
+    ("100-distinct-pairs-three-rounds", list(range(101)), [i % 10 for i in range(100)], [(i // 10) % 10 for i in range(100)],
+     2048, 128, 16),
+    ("80-distinct-pairs-tile-blocks-two-rounds", list(range(0, 644, 4)), [i % 10 for i in range(160)],
+     [(i // 10) % 8 for i in range(160)], 2048, 192, 64),
     ("1500-segments-two-launch-plan", list(range(1501)), [(i * 7) % 9 for i in range(1500)],
      [(i * 5) % 6 for i in range(1500)], 256, 128, 8),
 ]
