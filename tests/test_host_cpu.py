@@ -376,3 +376,22 @@ def test_refused_adapter_set_leaves_the_layer_unchanged():
     assert len(fused.adapters) == 2 and fused.wa_ptrs.numel() == 2 and not fused.packed
     fused.add_adapter(bad)  # stored at its own rank beside padded ones: served (packed_ranks)
     assert len(fused.adapters) == 3 and fused.packed and fused.adapter_rank.tolist() == [16, 16, 8]
+
+
+def test_checked_call_signature_compares_what_the_checks_look_at():
+    """The record a checked operator call leaves behind (ops/_kernels._Checked): a later call takes the short way
+    only with tensors of the same shapes, dtypes, devices and contiguity and the very same table objects."""
+    from loquetier_amd.ops import _kernels as K
+    x, y, tab_a, tab_b = torch.zeros(8, 16), torch.zeros(8, 32), torch.zeros(4, dtype=torch.int64), torch.zeros(4, dtype=torch.int64)
+    hit = K._Checked()
+    hit.descs = K._descs(([x], [y], ()))
+    hit.same = (tab_a, tab_b, None)
+    assert hit.matches(([torch.ones(8, 16)], [torch.ones(8, 32)], ()), (tab_a, tab_b, None))
+    assert not hit.matches(([torch.ones(8, 16)], [torch.ones(8, 32)], ()), (tab_a.clone(), tab_b, None))   # another table
+    assert not hit.matches(([torch.ones(9, 16)], [torch.ones(8, 32)], ()), (tab_a, tab_b, None))           # other rows
+    assert not hit.matches(([torch.ones(8, 16).half()], [torch.ones(8, 32)], ()), (tab_a, tab_b, None))    # other dtype
+    assert not hit.matches(([torch.ones(8, 32)[:, ::2]], [torch.ones(8, 32)], ()), (tab_a, tab_b, None))   # strided
+    assert not hit.matches(([None], [torch.ones(8, 32)], ()), (tab_a, tab_b, None))                        # left out
+    assert not hit.matches(([torch.ones(8, 16)], [torch.ones(8, 32)], [torch.ones(8, 4)]), (tab_a, tab_b, None))  # one more
+    assert not hit.matches(([torch.ones(8, 16)], [torch.ones(8, 32)], ()), (tab_a, tab_b, tab_a))          # a rank table now
+    assert K._mask([x, None, y]) == 0b101
