@@ -417,6 +417,8 @@ class _Checked:
         descs = self.descs
         for ts in tensor_lists:
             for t in ts:
+                if k == len(descs):
+                    return False
                 d = descs[k]
                 k += 1
                 if t is None:
