@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SMLM_ABI_VERSION 4
+#define SMLM_ABI_VERSION 5
 
 #if defined(__GNUC__)
 #define SMLM_API __attribute__((visibility("default")))
@@ -321,11 +321,17 @@ typedef struct smlm_dropout {
  *                  with dA_a [h_in, r] and dB_a [r, h_out] in the weights' own shapes.  Same kernels, no
  *                  copies; not together with dropout or packed_ranks.  (The forward in this layout is
  *                  smlm_gemm / smlm_gemm_planned with w_row_major = 1.)
+ *   dx_rows      : (backward entry points) 0, or the number of rows every dx buffer has, >= n_rows: the call
+ *                  then also sets rows [n_rows, dx_rows) of every dx to zero -- the rows of the batch that are
+ *                  not trained, when dx is the gradient of the whole batch's x as autograd wants it -- at no
+ *                  launch of its own where the dV product is folded (the fold's launch has the workgroups), by
+ *                  one small launch otherwise.  With bwd_stages the SMLM_BWD_PRODUCTS stage does it.
  */
 typedef struct smlm_lora_opts {
   const smlm_dropout* dropout;
   const int32_t* adapter_rank;
   int packed_ranks;
+  int dx_rows;
   const int32_t* build_seg_indptr;
   const int32_t* build_seg_adapter;
   int bwd_stages;

@@ -33,7 +33,7 @@ class Dropout(C.Structure):
 class LoraOpts(C.Structure):
     """struct smlm_lora_opts of include/smlm.h."""
     _fields_ = [("dropout", C.POINTER(Dropout)), ("adapter_rank", C.c_void_p), ("packed_ranks", C.c_int),
-                ("build_seg_indptr", C.c_void_p), ("build_seg_adapter", C.c_void_p), ("bwd_stages", C.c_int),
+                ("dx_rows", C.c_int), ("build_seg_indptr", C.c_void_p), ("build_seg_adapter", C.c_void_p), ("bwd_stages", C.c_int),
                 ("w_row_major", C.c_int), ("build_seg_key_a", C.c_void_p), ("build_seg_key_b", C.c_void_p)]
 
 

@@ -319,7 +319,12 @@ int launch_reduce(int dtype, int S, int groups, hipStream_t st, ReduceArgs& a, b
     const int units = tile_units_max(a.T, S, groups, 1);
     const long items = (long)units * a.nproj;
     a.units_max = items <= kDirectItems ? units : 0;
-    const dim3 grid = a.units_max ? dim3((unsigned)items) : work_grid(items);
+    const int zero_blocks = a.zero.n ? a.zero.first[a.zero.n] : 0;
+    if (zero_blocks && !a.units_max) {  // (a launch that walks its items has no workgroups to spare)
+      const int rc = launch(zero_spans_kernel, dim3((unsigned)zero_blocks), dim3(256), st, a.zero);
+      if (rc) return rc;
+    }
+    const dim3 grid = a.units_max ? dim3((unsigned)(items + zero_blocks)) : work_grid(items);
     if (dtype == SMLM_DTYPE_F16) return launch(reduce_kernel<SMLM_DTYPE_F16, true>, grid, dim3(256), st, a);
     return launch(reduce_kernel<SMLM_DTYPE_BF16, true>, grid, dim3(256), st, a);
   }
@@ -467,6 +472,7 @@ struct SideOut {
   const uint16_t* v2[kMaxProj];
   const float* scale;
   long pitch;
+  ZeroSpans zero;  // memory the fold's launch is to clear as well (n = 0: none)
 };
 
 int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int groups, int nproj,
@@ -539,6 +545,7 @@ int run_shrink(int dtype, bool row_major, const PlanView& pv, int T, int S, int 
   if (with_side) {
     ra.side_scale = side->scale;
     ra.side_pitch = side->pitch;
+    ra.zero = side->zero;
   }
   if (side_done) *side_done = with_side;
   return launch_reduce(dtype, S, groups, st, ra, with_side);
@@ -1050,6 +1057,8 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   const int stages = (opts && opts->bwd_stages) ? opts->bwd_stages : (SMLM_BWD_PRODUCTS | SMLM_BWD_DX | SMLM_BWD_WGRAD);
   // the other weight layout (the reference's is_row_major = True): A_a [h_in, r], B_a [r, h_out], and so are dA_a, dB_a
   const bool rm = opts && opts->w_row_major;
+  const int dx_rows = opts ? opts->dx_rows : 0;
+  if (dx_rows != 0 && dx_rows < n_rows) return SMLM_ERR_ARG;
   if (rm && (drop.seg_p || packed)) return SMLM_ERR_ARG;
   if (stages < 0 || stages > (SMLM_BWD_PRODUCTS | SMLM_BWD_DX | SMLM_BWD_WGRAD)) return SMLM_ERR_ARG;
   if (n_proj < 1 || n_proj > kMaxProj || NA < 0 || r <= 0 || !h_in || !h_out) return SMLM_ERR_ARG;
@@ -1181,8 +1190,23 @@ SMLM_API int smlm_lora_bwd_multi_ex(int n_proj, void* const* dx, void* const* co
   }
   side.scale = part_scale;
   side.pitch = L.pitch;
+  // rows of dX past the backward's own (opts->dx_rows): cleared by the fold's launch when it runs in direct mode,
+  // else by a launch of their own
+  ZeroSpans tail{};
+  if (dx_rows > n_rows) {
+    for (int i = 0; i < n_proj; ++i) {
+      tail.ptr[i] = reinterpret_cast<char*>(dx[i]) + (size_t)n_rows * h_in[i] * 2;
+      tail.bytes[i] = (long)(dx_rows - n_rows) * h_in[i] * 2;  // (h_in is a multiple of 8: whole 16-byte pieces)
+      tail.first[i + 1] = tail.first[i] + (int)((tail.bytes[i] + kZeroBlockBytes - 1) / kZeroBlockBytes);
+    }
+    tail.n = n_proj;
+  }
   // (a function of the shapes and the option: the same in every call of a staged backward)
   const bool side_in_fold = bwd_all_folded(n_proj, n_rows, h_out, r);
+  if (side_in_fold) side.zero = tail;
+  else if (tail.n && products &&
+           (rc = launch(zero_spans_kernel, dim3((unsigned)tail.first[tail.n]), dim3(256), st, tail)))
+    return rc;
   bool side_done = false;
   if (products && (rc = run_shrink(dtype, false, pv, n_rows, P, NA, n_proj, dy, btp, partial, dv16, h_out, r, b_ld,
                                    0.0f, nullptr, mt, st, true, in_place && !rm, nullptr, w_rank, in_place ? packed : 0,

@@ -463,6 +463,29 @@ __global__ __launch_bounds__(kFwdThreads) void shrink_block_kernel(ShrinkArgs a)
 
 constexpr int kMaxKsplit = 16;  // upper bound of the k split over workgroups
 
+// Spans of memory to be cleared by workgroups of 256 threads, kZeroBlockBytes each: span i takes blocks
+// [first[i], first[i + 1]).
+constexpr int kZeroBlockBytes = 32768;
+struct ZeroSpans {
+  char* ptr[kMaxProj];
+  long bytes[kMaxProj];     // multiples of 16
+  int first[kMaxProj + 1];
+  int n;
+};
+__device__ __forceinline__ void zero_span_block(const ZeroSpans& z, int block) {
+  int i = 0;
+#pragma unroll
+  for (int j = 1; j < kMaxProj; ++j) i += (j < z.n && block >= z.first[j]) ? 1 : 0;
+  const long off0 = (long)(block - z.first[i]) * kZeroBlockBytes;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < kZeroBlockBytes / (256 * 16); ++e) {
+    const long off = off0 + ((long)e * 256 + threadIdx.x) * 16;
+    if (off < z.bytes[i]) stg16(reinterpret_cast<uint16_t*>(z.ptr[i] + off), zero);
+  }
+}
+__global__ __launch_bounds__(256) void zero_spans_kernel(ZeroSpans z) { zero_span_block(z, (int)blockIdx.x); }
+
 struct ReduceProj {
   const float* partial;  // [ksplit, T, d_out]
   uint16_t* out;         // [T, d_out]
@@ -483,6 +506,8 @@ struct ReduceArgs {
   int units_max;  // > 0: direct mode, one (projection, tile) per workgroup over this tile bound
   const float* side_scale;  // SIDE folds: per segment, or null for 1
   long side_pitch;          // SIDE folds: slots per row of pt_a / pt_b
+  ZeroSpans zero;           // SIDE folds, direct mode: memory the launch's last workgroups clear (the rows of dX
+                            //   past the backward's own)
 };
 
 // Folds the k-split partial sums of a shrink launch, in split order, into the
@@ -493,6 +518,10 @@ struct ReduceArgs {
 template <int DT, bool SIDE = false>
 __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs a) {
   const int units = tile_units<1>(a.plan, a.units_max);
+  if (SIDE && a.units_max > 0 && (int)blockIdx.x >= units * a.nproj) {  // (uniform over the workgroup)
+    zero_span_block(a.zero, (int)blockIdx.x - units * a.nproj);
+    return;
+  }
   const int c = threadIdx.x >> 4, q = threadIdx.x & 15;
   const int last = a.units_max > 0 ? (int)blockIdx.x + 1 : units * a.nproj;
   for (int V = blockIdx.x; V < last; V += gridDim.x) {

@@ -121,8 +121,10 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
     tp = [int(t) for t in tp][: n_parts + 1]
     tl = tp[-1]
     grad_x = torch.empty((T, h_in), dtype=dt, device=dev)
-    if tl < T:
-        grad_x[tl:].zero_()
+    # rows past the training rows: cleared by the backward call itself (inside one of its launches) when one follows
+    tail_in_call = 0 < tl < T
+    if tl == 0:
+        grad_x.zero_()
     if tp[0] > 0:
         grad_x[: tp[0]].zero_()
     prepared = step is not None and step.bwd_plan is not None and step.grad_layout is not None
@@ -159,7 +161,7 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
             kernel.smlm_lora_backward(grad_x, tabs[0], tabs[1], g, x_train, v_train, step.a_tab, step.b_tab,
                                       step.bwd_plan, lora_rank, part_scale, dropout=dropout,
                                       adapter_rank=adapter_rank, workspace=step.workspace,
-                                      packed_ranks=step.packed, cache=step.cache)
+                                      packed_ranks=step.packed, cache=step.cache, zero_dx_tail=tail_in_call)
         else:
             for b in bufs:
                 b.zero_()
@@ -177,7 +179,7 @@ def lora_backward(grad_output: torch.Tensor, x_train: torch.Tensor, v_train: Opt
                 _ptr_table([p[0] for p in pairs], dev), _ptr_table([p[1] for p in pairs], dev),
                 plan, lora_rank, part_scale, dropout=dropout, adapter_rank=adapter_rank,
                 workspace=None if step is None else step.workspace,
-                packed_ranks=step is not None and step.packed)
+                packed_ranks=step is not None and step.packed, zero_dx_tail=tail_in_call)
         else:
             for t in da + db:
                 t.zero_()

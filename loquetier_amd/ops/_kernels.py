@@ -595,7 +595,8 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
                        dropout: Optional[DropoutSpec] = None,
                        adapter_rank: Optional[torch.Tensor] = None,
                        workspace: Optional[Workspace] = None, packed_ranks: bool = False,
-                       is_row_major: bool = False, cache: Optional[dict] = None) -> None:
+                       is_row_major: bool = False, cache: Optional[dict] = None,
+                       zero_dx_tail: bool = False) -> None:
     """dX rows of the train partitions and per-adapter dA / dB (see include/smlm.h).
     `plan` = SegmentPlan(part_indptr, part_adapter int32, n_rows).  dropout: the
     forward's stream with seg_p per partition; x is the tensor before dropout.
@@ -603,15 +604,19 @@ def smlm_lora_backward(dx: torch.Tensor, da_ptrs: torch.Tensor, db_ptrs: torch.T
     smlm_lora_backward_multi([dx], [da_ptrs], [db_ptrs], [dy], [x], None if v is None else [v], [a_ptrs],
                              [b_ptrs], plan, rank, part_scale=part_scale, dropout=dropout,
                              adapter_rank=adapter_rank, workspace=workspace, packed_ranks=packed_ranks,
-                             is_row_major=is_row_major, cache=cache)
+                             is_row_major=is_row_major, cache=cache, zero_dx_tail=zero_dx_tail)
 
 
 _BWD_MULTI_SIZES: Dict[Tuple, int] = {}
 
 
-def _bwd_opts(plan, adapter_rank, n_weights, packed_ranks, stages, is_row_major, checked, dropout=None, widths=None):
+def _bwd_opts(plan, adapter_rank, n_weights, packed_ranks, stages, is_row_major, checked, dropout=None, widths=None,
+              dx_rows=0):
     """struct smlm_lora_opts of a backward call (None when there is nothing to say)."""
     opts = _opts(plan, dropout, widths, adapter_rank, n_weights, packed_ranks, checked=checked)
+    if dx_rows:
+        opts = opts or _lib.LoraOpts()
+        opts.dx_rows = int(dx_rows)
     if stages:
         opts = opts or _lib.LoraOpts()
         opts.bwd_stages = int(stages)
@@ -641,7 +646,7 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
                              adapter_rank: Optional[torch.Tensor] = None,
                              workspace: Optional[Workspace] = None, packed_ranks: bool = False,
                              stages: int = 0, is_row_major: bool = False,
-                             cache: Optional[dict] = None) -> None:
+                             cache: Optional[dict] = None, zero_dx_tail: bool = False) -> None:
     """The backward of several projections of one batch (q/k/v/o, gate/up/down) in one set of
     launches; lists of equal length, one entry per projection, each what smlm_lora_backward
     takes.  vs: None, or the saved intermediate of every projection.  The results equal
@@ -651,13 +656,15 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
     may be issued as separate calls with the same arguments, workspace and stream, in that order.
     is_row_major: the weights and their gradients are A [h_in, r], B [r, h_out] (the layout the reference's
     backward lines are written for, kernel_utils.py:139-145) instead of PEFT's A [r, h_in], B [h_out, r].
-    cache: as in smlm_lora_forward_multi (the same dict may serve a layer's forward and backward)."""
+    cache: as in smlm_lora_forward_multi (the same dict may serve a layer's forward and backward).
+    zero_dx_tail: the dx tensors cover more rows than the plan (the whole batch): the call also sets their rows from
+    plan.T on to zero, inside one of its launches where it can (all dx must then have the same number of rows)."""
     n = len(dxs)
     key = None
     if cache is not None and dropout is None:  # (a dropout descriptor is checked call by call)
         scale_list = () if part_scale is None else (part_scale,)
         key = ("bwd", n, stages, plan.T, plan.S, plan.kind, rank, bool(packed_ranks), bool(is_row_major),
-               vs is None, len(scale_list))
+               vs is None, len(scale_list), bool(zero_dx_tail))
         hit = cache.get(key)
         if hit is not None and hit.matches((dxs, dys, xs, vs or (), da_ptrs, db_ptrs, scale_list),
                                            (*a_ptrs, *b_ptrs, adapter_rank)):
@@ -668,8 +675,8 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
                 if not plan.built and stages and not (stages & _lib.SMLM_BWD_PRODUCTS):
                     plan.ensure_built()
                 if not plan.built:  # a deferred plan: this call builds it
-                    opts = _bwd_opts(plan, adapter_rank, hit.n_weights, packed_ranks, stages, is_row_major, True) \
-                        or _lib.LoraOpts()
+                    opts = _bwd_opts(plan, adapter_rank, hit.n_weights, packed_ranks, stages, is_row_major, True,
+                                     dx_rows=dxs[0].size(0) if zero_dx_tail else 0) or _lib.LoraOpts()
                     opts.build_seg_indptr = plan.segment.data_ptr()
                     opts.build_seg_adapter = plan.seg_key.data_ptr()
                 dx_arr, dy_arr, x_arr, v_arr, da_arr, db_arr = hit.arrs
@@ -716,8 +723,13 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
         ws = _workspace(dev, need, workspace)
         if dropout is not None and dropout.rows < n_rows:
             raise RuntimeError("the dropout descriptor must cover the backward's rows")
+        dx_rows = 0
+        if zero_dx_tail:
+            dx_rows = dxs[0].size(0)
+            if any(t.size(0) != dx_rows for t in dxs):
+                raise RuntimeError("zero_dx_tail: every dx must have the same number of rows")
         opts = _bwd_opts(plan, adapter_rank, NA, packed_ranks, stages, is_row_major, False, dropout,
-                         list(widths_in))
+                         list(widths_in), dx_rows)
         arr = lambda ts: VP(*[t.data_ptr() for t in ts])
         a_arr, b_arr, h_in, h_out = arr(a_ptrs), arr(b_ptrs), CI(*widths_in), CI(*widths_out)
         if key is not None:  # (every check has passed: the next call like this one takes the short way)
@@ -726,7 +738,7 @@ def smlm_lora_backward_multi(dxs, da_ptrs, db_ptrs, dys, xs, vs, a_ptrs, b_ptrs,
             hit.same = (*a_ptrs, *b_ptrs, adapter_rank)
             hit.code, hit.dev, hit.arrs, hit.h_in, hit.h_out = code, dev, tuple(VP() for _ in range(6)), h_in, h_out
             hit.a_arr, hit.b_arr, hit.n_weights, hit.need = a_arr, b_arr, NA, need
-            hit.opts = _bwd_opts(plan, adapter_rank, NA, packed_ranks, stages, is_row_major, True)
+            hit.opts = _bwd_opts(plan, adapter_rank, NA, packed_ranks, stages, is_row_major, True, dx_rows=dx_rows)
             _remember(cache, key, hit)
         if not plan.built:  # a deferred plan: this call builds it (inside its first launch where it can)
             if stages and not (stages & _lib.SMLM_BWD_PRODUCTS):

@@ -266,3 +266,29 @@ def test_fold_writes_what_the_weight_gradients_read(K, oracle, gpu_device, case,
         _multi(K, projs, eager, plan, r, vs=vs, scale=scale)
         torch.cuda.synchronize()
         same(static, eager, f"replay {k}")
+
+
+@pytest.mark.parametrize("case", [CASES[0], SIDE_CASES[0]], ids=["dx-launch-writes-the-side-products", "fold-writes-them"])
+def test_rows_of_dx_past_the_training_rows_are_cleared_by_the_call(K, oracle, gpu_device, case):
+    """dx buffers that cover the whole batch (autograd wants the gradient of all of x): zero_dx_tail makes the call
+    clear the rows past the plan's -- inside the fold's launch where there is one for every projection, by a small
+    launch of its own otherwise -- and changes nothing else; staged calls do it in their first stage."""
+    name, tp, part_ad, NA, dims, r = case
+    d, dt, n_rows, extra = gpu_device, "bf16", tp[-1], 37
+    projs, pi, pa = _setup(oracle, d, case, dt, dy=False)
+    plan = K.SegmentPlan(pi, pa, n_rows)
+    plain = _outputs(projs, d, dt, n_rows)
+    _multi(K, projs, plain, plan, r)
+    for stages in ((0,), (1, 2, 4)):
+        wide = _outputs(projs, d, dt, n_rows + extra)
+        for st in stages:
+            _multi(K, projs, wide, plan, r, zero_dx_tail=True, stages=st)
+        for i, (m, s_) in enumerate(zip(wide, plain)):
+            assert torch.equal(m["dx"][:n_rows], s_["dx"]), (stages, i)
+            assert torch.count_nonzero(m["dx"][n_rows:]) == 0, (stages, i)
+            for a in range(NA):
+                assert torch.equal(m["dA"][a], s_["dA"][a]) and torch.equal(m["dB"][a], s_["dB"][a]), (stages, i, a)
+    with pytest.raises(RuntimeError):  # dx tensors of different heights
+        wide = _outputs(projs, d, dt, n_rows + extra)
+        wide[0]["dx"] = wide[0]["dx"][:-1]
+        _multi(K, projs, wide, plan, r, zero_dx_tail=True)

@@ -31,7 +31,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
     for name in declared:
         assert hasattr(handle, name), f"{name} is declared in smlm.h but not exported"
     assert declared == set(lib.SIGNATURES), "ctypes binding and header disagree"
-    assert lib.load().smlm_abi_version() == 4
+    assert lib.load().smlm_abi_version() == 5
 
 
 def test_missing_library_fails_loudly(lib, monkeypatch):
