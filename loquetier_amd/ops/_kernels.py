@@ -123,6 +123,13 @@ def smlm_forward_cutlass_tmp_size(num_problems: int) -> int:
     return _lib.size_query("smlm_tmp_size", int(num_problems))
 
 
+def smlm_forward_cutlass_workspace_size(T: int, num_problems: int, d_in: int, d_out: int) -> int:
+    """Bytes of a `tmp` that smlm_forward_cutlass uses as its ONLY scratch (plan and k-split partial sums of a
+    [T, d_in] x [d_in, d_out] batch of num_problems segments): a caller that passes a tmp of at least this size
+    owns every byte the call touches.  No counterpart in the reference, whose 60 bytes a problem hold all it needs."""
+    return _lib.size_query("smlm_gemm_workspace_size", int(T), int(num_problems), int(d_in), int(d_out))
+
+
 def smlm_forward_cutlass(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, s: torch.Tensor,
                          tmp: torch.Tensor, is_row_major: bool) -> None:
     """Grouped GEMM y[s_i:s_{i+1}] = x[s_i:s_{i+1}] @ W_i, overwriting y.
@@ -131,7 +138,10 @@ def smlm_forward_cutlass(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, 
     (kernel_src/csrc/loquetier_ops.cc:277-319): y [T,d_out], x [T,d_in] fp16 or
     bf16, w_ptr int64 [S] device addresses, s int32 [S+1], tmp uint8 of exactly
     smlm_forward_cutlass_tmp_size(S) bytes.  Unlike the reference it does not
-    block the host.
+    block the host.  The kernels here need more scratch than that tmp holds: with a tmp of the
+    reference's size it comes from a buffer this module keeps per (device, stream); a tmp of
+    smlm_forward_cutlass_workspace_size(T, S, d_in, d_out) bytes or more (16-byte aligned) is
+    used itself, and the call then touches no memory the caller did not hand it.
     """
     for t, n in ((y, "y"), (x, "x"), (w_ptr, "w_ptr"), (s, "s"), (tmp, "tmp")):
         _check_input(t, n)
@@ -143,9 +153,6 @@ def smlm_forward_cutlass(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, 
     num_problems = s.size(0) - 1
     d_in, d_out = x.size(1), y.size(1)
     w_ld = d_out if is_row_major else d_in
-    if tmp.size(0) != smlm_forward_cutlass_tmp_size(num_problems):
-        raise RuntimeError(f"CHECK_EQ(tmp.size(0), smlm_forward_tmp_size(num_problems)) failed: "
-                           f"{tmp.size(0)} vs {smlm_forward_cutlass_tmp_size(num_problems)}")
     if w_ptr.dtype != torch.int64 or s.dtype != torch.int32:
         raise RuntimeError("w_ptr must be int64 and s must be int32")
     if w_ptr.size(0) != num_problems or y.size(0) != x.size(0) or y.dtype != x.dtype:
@@ -155,7 +162,13 @@ def smlm_forward_cutlass(y: torch.Tensor, x: torch.Tensor, w_ptr: torch.Tensor, 
     dev = tmp.device
     with _on(dev):
         need = _lib.size_query("smlm_gemm_workspace_size", T, num_problems, d_in, d_out)
-        ws = _workspace(dev, need)
+        own = tmp.size(0) >= need and tmp.size(0) != smlm_forward_cutlass_tmp_size(num_problems)
+        if not own and tmp.size(0) != smlm_forward_cutlass_tmp_size(num_problems):
+            raise RuntimeError(f"CHECK_EQ(tmp.size(0), smlm_forward_tmp_size(num_problems)) failed: "
+                               f"{tmp.size(0)} vs {smlm_forward_cutlass_tmp_size(num_problems)}")
+        if own and tmp.data_ptr() % 16:
+            raise RuntimeError("a tmp that serves as the workspace must be 16-byte aligned")
+        ws = tmp if own else _workspace(dev, need)
         rc = _lib.load().smlm_gemm(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s.data_ptr(),
                                    ws.data_ptr(), ws.numel(), T, num_problems, d_in, d_out, w_ld,
                                    int(bool(is_row_major)), code, 0.0, None, _stream(dev))

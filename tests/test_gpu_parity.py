@@ -262,6 +262,31 @@ def test_generic_grouped_gemm_shapes_and_layouts(K, oracle, gpu_device, shape, r
     close(to_np(y), yo)
 
 
+def test_reference_call_with_a_tmp_that_holds_all_its_scratch(K, oracle, gpu_device):
+    """A tmp of smlm_forward_cutlass_workspace_size bytes is the call's only scratch (the reference's
+    ownership rule: everything through tmp, kernel_src/csrc/loquetier_ops.cc:304): same results as with the
+    reference-sized tmp, and the bytes of the large tmp are the ones that get written."""
+    name, T, seg, ids, NA, h_in, h_out, r = FWD_CASES[1]
+    dt, d = "fp16", gpu_device
+    x, A, B = make_case(oracle, 100, T, seg, ids, NA, h_in, h_out, r, dt)
+    xd = dev_t(x, dt, d)
+    Ad = [dev_t(a, dt, d) for a in A]
+    s = torch.tensor(seg, dtype=torch.int32, device=d)
+    wa = ptrs([Ad[i] for i in ids], d)
+    small = torch.empty(K.smlm_forward_cutlass_tmp_size(len(ids)), dtype=torch.uint8, device=d)
+    need = K.smlm_forward_cutlass_workspace_size(T, len(ids), h_in, r)
+    assert need > small.numel()
+    large = torch.full((need + 64,), 0xA5, dtype=torch.uint8, device=d)
+    v1 = torch.full((T, r), 3.0, dtype=TDT[dt], device=d)
+    v2 = torch.full((T, r), 3.0, dtype=TDT[dt], device=d)
+    K.smlm_forward_cutlass(v1, xd, wa, s, small, False)
+    K.smlm_forward_cutlass(v2, xd, wa, s, large, False)
+    assert torch.equal(v1, v2)
+    assert bool((large[:need] != 0xA5).any()) and bool((large[need:] == 0xA5).all())
+    with pytest.raises(RuntimeError, match="aligned"):
+        K.smlm_forward_cutlass(v2, xd, wa, s, torch.empty(need + 24, dtype=torch.uint8, device=d)[8:], False)
+
+
 def test_reference_error_behaviour(K, gpu_device):
     d = gpu_device
     x32 = torch.zeros(4, 16, device=d)
