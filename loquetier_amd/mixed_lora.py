@@ -38,6 +38,8 @@ class MixedLoraContext:
         self._lora_len = None
         self._segment = None
         self._train_idx: List[int] = []
+        self._train_key: tuple = ()
+        self._train_order: Optional[List[int]] = None
         self._plan: Optional[kernel.SegmentPlan] = None
         self._seg_adapter: Optional[torch.Tensor] = None
         self._step: dict = {}          # per-step memo, dropped by update()
@@ -56,6 +58,8 @@ class MixedLoraContext:
         if open_group is not None:   # a deferred group whose last member was never called: its adds happen now
             open_group["group"].flush(open_group)
         self._train_idx = list(train_idx)
+        self._train_key = tuple(self._train_idx)   # (what the layers key their per-training-set tables on)
+        self._train_order = None
         self._plan = None
         self._seg_adapter = None
         self._step = {}
@@ -79,6 +83,11 @@ class MixedLoraContext:
     @property
     def train_idx(self) -> List[int]:
         return self._train_idx
+
+    @property
+    def train_key(self) -> tuple:
+        """train_idx as a tuple, made once per update."""
+        return self._train_key
 
     def memo(self, key, build):
         """Value built once per step (per `update`) and shared by every layer that asks for `key`."""
@@ -161,7 +170,9 @@ class MixedLoraContext:
     def train_order(self) -> List[int]:
         """Training adapters in order of first appearance among the train partitions: the backward
         numbers them 0..NA-1 in this order."""
-        return list(dict.fromkeys(int(i) for i in self._train_idx))
+        if self._train_order is None:
+            self._train_order = list(dict.fromkeys(int(i) for i in self._train_idx))
+        return self._train_order
 
     def backward_tables(self, device: torch.device):
         """(partition plan, partition -> training adapter list) of the step's backward: a function
@@ -189,6 +200,14 @@ class MixedLoraContext:
                                   dtype=torch.int32, device=device)
             return (torch.searchsorted(plan.segment, starts, right=True) - 1).clamp_(0, max(plan.S - 1, 0))
         return self.memo(("part_segments", device), build)
+
+    def train_bundle(self, device: torch.device, plan: kernel.SegmentPlan):
+        """(training adapters in order, backward plan, partition -> training adapter, partition -> segment):
+        what a training layer call needs of the step beyond the forward's plan, in one look-up."""
+        def build():
+            bwd_plan, part_adapter = self.backward_tables(device)
+            return self.train_order(), bwd_plan, part_adapter, self.part_segments(device, plan)
+        return self.memo(("train_bundle", device), build)
 
 
 # Adapter whose parameters a state_dict() call saves (reference: CURRENT_TRAINER_LORA_ID and
@@ -581,7 +600,7 @@ class MixedLoraLinear(nn.Module):
     def _weights_of(self, train_idx):
         """The parameters of the step's training adapters, A and B in turn (looked up once per set: the
         parameters are registered by set_trainable and stay the same objects)."""
-        key = tuple(train_idx)
+        key = train_idx if isinstance(train_idx, tuple) else tuple(train_idx)
         weights = self._train_weights.get(key)
         if weights is None:
             weights = [w for idx in key for w in (self.get_parameter(f"lora-{idx}-A"),
@@ -596,7 +615,7 @@ class MixedLoraLinear(nn.Module):
         or None when every adapter has the layer's rank."""
         if self.adapter_rank is None:
             return None
-        order = list(dict.fromkeys(int(i) for i in train_idx))
+        order = list(dict.fromkeys(int(i) for i in train_idx))   # (a no-op on the context's own order)
         key = tuple(order)
         if self._train_rank_key != key:
             self._train_rank_key = key
@@ -649,7 +668,7 @@ class MixedLoraLinear(nn.Module):
                 start, end = blen.train_partition[pi], blen.train_partition[pi + 1]
                 dropped_x.append(self.adapters[idx].dropout(x[start:end, :]))
             x = torch.cat(dropped_x + [x[blen.tlen:, :]])
-        weights = self._weights_of(train_idx)
+        weights = self._weights_of(ctx.train_key)
         if self.fused:
             # per-step tables come from the context (built once for all layers), per-layer ones from
             # the layer (built once per adapter set): nothing is copied from the host in here
@@ -685,11 +704,10 @@ class MixedLoraLinear(nn.Module):
             step.wa_table, step.wb_table, step.seg_scale, step.plan, step.rank = \
                 self.wa_ptrs, self.wb_ptrs, seg_scale, plan, self.rank
             step.train_len, step.train_partition, step.dropout = blen.tlen, blen.train_partition, drop_spec
-            step.adapter_rank = self._rank_args(train_idx)
+            step.adapter_rank = None if self.adapter_rank is None else self._rank_args(ctx.train_order())
             if weights and blen.tlen > 0:
-                step.bwd_plan, step.part_adapter = ctx.backward_tables(self.device)
-                step.part_segments = ctx.part_segments(self.device, plan)
-                tabs = self._train_tables(ctx.train_order())
+                order, step.bwd_plan, step.part_adapter, step.part_segments = ctx.train_bundle(self.device, plan)
+                tabs = self._train_tables(order)
                 step.a_tab, step.b_tab = tabs["a_tab"], tabs["b_tab"]
                 step.grad_layout = tabs
             result = fused_add_lora.apply(result, x, step, *weights)
