@@ -66,17 +66,19 @@ BWD = [
 ]
 
 
-def _run_rm(K, d, dt, x, g, A, B, tp, part_ad, r, v=None, scale=None):
+def _run_rm(K, d, dt, x, g, A, B, tp, part_ad, r, v=None, scale=None, tail=0):
     n_rows = tp[-1]
     Ad, Bd = [dev_t(a, dt, d) for a in A], [dev_t(b, dt, d) for b in B]
     dA, dB = [torch.full_like(a, 5.0) for a in Ad], [torch.full_like(b, 5.0) for b in Bd]
-    dx = torch.full((n_rows, x.shape[1]), 5.0, dtype=TDT[dt], device=d)
+    dx = torch.full((n_rows + tail, x.shape[1]), 5.0, dtype=TDT[dt], device=d)
     plan = K.SegmentPlan(torch.tensor(tp, dtype=torch.int32, device=d),
                          torch.tensor(part_ad, dtype=torch.int32, device=d), n_rows, defer=True)
     K.smlm_lora_backward(dx, ptrs(dA, d), ptrs(dB, d), dev_t(g, dt, d), dev_t(x, dt, d),
                          None if v is None else dev_t(v, dt, d), ptrs(Ad, d), ptrs(Bd, d), plan, r, scale,
-                         is_row_major=True)
-    return to_np(dx), [to_np(t) for t in dA], [to_np(t) for t in dB]
+                         is_row_major=True, zero_dx_tail=tail > 0)
+    if tail:  # rows past the plan's: cleared by the call
+        assert torch.count_nonzero(dx[n_rows:]) == 0
+    return to_np(dx[:n_rows]), [to_np(t) for t in dA], [to_np(t) for t in dB]
 
 
 @pytest.mark.parametrize("dt", ["fp16", "bf16"])
@@ -90,7 +92,7 @@ def test_row_major_backward_dyadic_bit_exact(K, oracle, gpu_device, case, dt):
     A = [dyadic(rng, (h_in, r), 8, 64) for _ in range(NA)]
     B = [dyadic(rng, (r, h_out), 8, 8) for _ in range(NA)]
     part_ad = list(range(len(tp) - 1))
-    dx, dA, dB = _run_rm(K, gpu_device, dt, x, g, A, B, tp, part_ad, r)
+    dx, dA, dB = _run_rm(K, gpu_device, dt, x, g, A, B, tp, part_ad, r, tail=11)
     gx, ga, gb = oracle.add_lora_backward_rowmajor(g, x, [A[a] for a in part_ad], [B[a] for a in part_ad], tp, dt)
     assert np.array_equal(dx, gx)
     for p, a in enumerate(part_ad):
